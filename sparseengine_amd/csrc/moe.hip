@@ -1,0 +1,347 @@
+// Mixture-of-experts support kernels for gfx950: router top-k, grouping of (token, slot)
+// assignments by expert, a general tiled grouped GEMM (float and bfloat16, any sizes), the
+// sum over a token's slots, and the SwiGLU product of a dense feed-forward.
+//
+// Router: score = sigmoid(logit) (or softmax over the experts); experts are chosen by
+// score + bias, NaN counting as +inf, lowest index first among equal values; the output
+// holds the chosen experts with a value strictly above the k-th one in index order, then the
+// ties at the k-th value in index order.  Weights are the unbiased scores of the chosen
+// experts, optionally divided by their sum, times a scaling factor.  All float.
+#include "common.h"
+
+#define ROUTER_MAX_PER_LANE 16  // experts <= 64 * 16
+
+__global__ void router_topk_kernel(const float* __restrict__ logits, int64_t stride,
+                                   const float* __restrict__ bias, int32_t* __restrict__ ids,
+                                   float* __restrict__ weights, int tokens, int experts, int top_k,
+                                   int softmax_scoring, int normalize, float scaling) {
+  const int lane = threadIdx.x & (SE_WAVE - 1);
+  const int token = blockIdx.x * (blockDim.x / SE_WAVE) + threadIdx.x / SE_WAVE;
+  if (token >= tokens) return;  // whole waves leave together; no block barrier below
+  const float* row = logits + static_cast<int64_t>(token) * stride;
+
+  float score[ROUTER_MAX_PER_LANE], sel[ROUTER_MAX_PER_LANE];
+  float row_max = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+    const int e = i * SE_WAVE + lane;
+    score[i] = e < experts ? row[e] : -INFINITY;
+    row_max = fmaxf(row_max, score[i]);
+  }
+  if (softmax_scoring) {
+    row_max = wave_max(row_max);
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+      const int e = i * SE_WAVE + lane;
+      score[i] = e < experts ? expf(score[i] - row_max) : 0.f;
+      part += score[i];
+    }
+    const float denom = wave_sum(part);
+#pragma unroll
+    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) score[i] /= denom;
+  } else {
+#pragma unroll
+    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) score[i] = 1.f / (1.f + expf(-score[i]));
+  }
+  uint32_t taken = 0;     // bit i: element i of this lane is chosen
+  uint32_t excluded = 0;  // bit i: element i does not exist
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+    const int e = i * SE_WAVE + lane;
+    if (e < experts) {
+      float s = score[i] + (bias ? bias[e] : 0.f);
+      sel[i] = (s == s) ? s : INFINITY;
+    } else {
+      sel[i] = -INFINITY;
+      excluded |= 1u << i;
+    }
+  }
+  // k rounds of arg-max (largest value, lowest index among equals); the last value is the threshold
+  float threshold = 0.f;
+  for (int round = 0; round < top_k; ++round) {
+    float best = -INFINITY;
+    int best_idx = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+      if ((taken | excluded) & (1u << i)) continue;
+      const int e = i * SE_WAVE + lane;
+      if (best_idx == 0x7fffffff || sel[i] > best) {
+        best = sel[i];
+        best_idx = e;
+      }
+    }
+#pragma unroll
+    for (int off = SE_WAVE / 2; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, SE_WAVE);
+      const int other_idx = __shfl_xor(best_idx, off, SE_WAVE);
+      const bool take_other =
+          other_idx != 0x7fffffff &&
+          (best_idx == 0x7fffffff || other > best || (other == best && other_idx < best_idx));
+      if (take_other) {
+        best = other;
+        best_idx = other_idx;
+      }
+    }
+    if ((best_idx & (SE_WAVE - 1)) == lane) taken |= 1u << (best_idx / SE_WAVE);
+    threshold = best;
+  }
+  // output order: strictly greater than the threshold by index, then the chosen ties by index
+  int greater_before = 0, ties_before = 0;
+  int my_slot[ROUTER_MAX_PER_LANE];
+  const uint64_t lower_lanes = (lane == 0) ? 0ull : (~0ull >> (SE_WAVE - lane));
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+    const bool chosen = taken & (1u << i);
+    const bool greater = chosen && sel[i] > threshold;
+    const bool tie = chosen && !greater;
+    const uint64_t gmask = __ballot(greater);
+    const uint64_t tmask = __ballot(tie);
+    my_slot[i] = greater ? greater_before + __popcll(gmask & lower_lanes)
+                         : -(1 + ties_before + __popcll(tmask & lower_lanes));
+    greater_before += __popcll(gmask);
+    ties_before += __popcll(tmask);
+  }
+  float part = 0.f;
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i)
+    if (taken & (1u << i)) part += score[i];
+  const float total = wave_sum(part);
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+    if (!(taken & (1u << i))) continue;
+    const int slot = my_slot[i] >= 0 ? my_slot[i] : greater_before + (-my_slot[i] - 1);
+    ids[static_cast<int64_t>(token) * top_k + slot] = i * SE_WAVE + lane;
+    weights[static_cast<int64_t>(token) * top_k + slot] =
+        (normalize ? score[i] / total : score[i]) * scaling;
+  }
+}
+
+// ---------------------------------------------------------------------------------------- //
+// Group the A = tokens * top_k assignments by expert.  Every expert's run is padded to a
+// multiple of `tile_rows`; padding entries hold A.  One block does the whole job.
+//   sorted[capacity]      assignment ids in expert order (capacity >= A + experts*(tile_rows-1))
+//   tile_expert[max_tiles] expert of each tile of `tile_rows` sorted entries
+//   counters[0] = number of tiles, counters[1] = number of sorted entries
+// The order of assignments inside one expert's run is not fixed; every row of a tile is
+// computed independently of its neighbours, so results do not depend on it.
+// ---------------------------------------------------------------------------------------- //
+__global__ void moe_align_kernel(const int32_t* __restrict__ ids, int assignments, int experts,
+                                 int tile_rows, int32_t* __restrict__ sorted,
+                                 int32_t* __restrict__ tile_expert, int32_t* __restrict__ counters) {
+  extern __shared__ int32_t sh[];
+  int32_t* counts = sh;                 // [experts]
+  int32_t* offsets = sh + experts;      // [experts + 1] start of each run in `sorted`
+  int32_t* cursor = offsets + experts + 1;  // [experts]
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int a = threadIdx.x; a < assignments; a += blockDim.x) atomicAdd(&counts[ids[a]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t run = 0;
+    for (int e = 0; e < experts; ++e) {
+      offsets[e] = run;
+      run += (counts[e] + tile_rows - 1) / tile_rows * tile_rows;
+    }
+    offsets[experts] = run;
+    counters[0] = run / tile_rows;
+    counters[1] = run;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+    cursor[e] = offsets[e];
+    for (int p = offsets[e] + counts[e]; p < offsets[e + 1]; ++p) sorted[p] = assignments;
+    for (int t = offsets[e] / tile_rows; t < offsets[e + 1] / tile_rows; ++t) tile_expert[t] = e;
+  }
+  __syncthreads();
+  for (int a = threadIdx.x; a < assignments; a += blockDim.x) {
+    const int pos = atomicAdd(&cursor[ids[a]], 1);
+    sorted[pos] = a;
+  }
+}
+
+// ---------------------------------------------------------------------------------------- //
+// General grouped GEMM over the sorted assignments, float accumulation, any sizes.
+// A tile is GM = 16 sorted rows; a block computes GN = 64 output columns of it.
+//   MODE 0 (gate-up + SwiGLU): in row = x[a / top_k, :K]; w = w13[e] of shape [2N, K];
+//       out[a, n] = silu(g) * u with g = in . w[n], u = in . w[N + n]; g and u are rounded to
+//       the storage type, silu is taken in float and rounded, the product is rounded.
+//   MODE 1 (down): in row = act[a, :K]; w = w2[e] of shape [N, K];
+//       out[a, n] = (in . w[n]) * route_weight[a]   (weight applied to the float accumulator)
+// ---------------------------------------------------------------------------------------- //
+#define GG_M 16
+#define GG_N 64
+#define GG_K 32
+
+template <typename T, int MODE>
+__global__ void grouped_gemm_generic_kernel(const T* __restrict__ in, const T* __restrict__ w,
+                                            T* __restrict__ out,
+                                            const int32_t* __restrict__ sorted,
+                                            const int32_t* __restrict__ tile_expert,
+                                            const int32_t* __restrict__ counters,
+                                            const float* __restrict__ route_weight, int assignments,
+                                            int top_k, int N, int K) {
+  const int tile = blockIdx.y;
+  if (tile >= counters[0]) return;  // uniform over the block
+  __shared__ float xs[GG_M][GG_K + 1];
+  __shared__ float wg[GG_N][GG_K + 1];
+  __shared__ float wu[MODE == 0 ? GG_N : 1][GG_K + 1];
+  __shared__ int32_t rows[GG_M];
+  const int expert = tile_expert[tile];
+  const int n0 = blockIdx.x * GG_N;
+  if (threadIdx.x < GG_M) rows[threadIdx.x] = sorted[tile * GG_M + threadIdx.x];
+  __syncthreads();
+  const int64_t w_rows = MODE == 0 ? 2 * static_cast<int64_t>(N) : N;
+  const T* we = w + static_cast<int64_t>(expert) * w_rows * K;
+  const int r = threadIdx.x / 16;          // row of the tile
+  const int cg = threadIdx.x % 16;         // column group: columns cg, cg+16, cg+32, cg+48
+  float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += GG_K) {
+    for (int idx = threadIdx.x; idx < GG_M * GG_K; idx += blockDim.x) {
+      const int rr = idx / GG_K, kk = idx % GG_K;
+      const int a = rows[rr];
+      float v = 0.f;
+      if (a < assignments && k0 + kk < K) {
+        const int64_t src = MODE == 0 ? a / top_k : a;
+        v = to_float(in[src * K + k0 + kk]);
+      }
+      xs[rr][kk] = v;
+    }
+    for (int idx = threadIdx.x; idx < GG_N * GG_K; idx += blockDim.x) {
+      const int nn = idx / GG_K, kk = idx % GG_K;
+      const bool ok = n0 + nn < N && k0 + kk < K;
+      wg[nn][kk] = ok ? to_float(we[static_cast<int64_t>(n0 + nn) * K + k0 + kk]) : 0.f;
+      if (MODE == 0)
+        wu[nn][kk] = ok ? to_float(we[static_cast<int64_t>(N + n0 + nn) * K + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < GG_K; ++kk) {
+      const float xv = xs[r][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        g[j] += xv * wg[cg + 16 * j][kk];
+        if (MODE == 0) u[j] += xv * wu[cg + 16 * j][kk];
+      }
+    }
+    __syncthreads();
+  }
+  const int a = rows[r];
+  if (a >= assignments) return;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + cg + 16 * j;
+    if (n >= N) continue;
+    float y;
+    if (MODE == 0) {
+      const float gate = round_to<T>(g[j]);
+      const float up = round_to<T>(u[j]);
+      const float act = round_to<T>(gate / (1.f + expf(-gate)));
+      y = act * up;
+    } else {
+      y = g[j] * route_weight[a];
+    }
+    out[static_cast<int64_t>(a) * N + n] = from_float<T>(y);
+  }
+}
+
+// out[t, c] = sum over the token's top_k slots of y[t * top_k + k, c], float accumulation in slot order
+template <typename T>
+__global__ void moe_sum_kernel(const T* __restrict__ y, T* __restrict__ out, int top_k,
+                               int hidden) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top_k; ++k) acc += to_float(y[(t * top_k + k) * hidden + c]);
+    out[t * hidden + c] = from_float<T>(acc);
+  }
+}
+
+// out[t, c] = silu(x[t, c]) * x[t, width + c] with the roundings of the fused expert path
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ out, int width) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float gate = to_float(x[t * 2 * width + c]);
+    const float up = to_float(x[t * 2 * width + width + c]);
+    const float act = round_to<T>(gate / (1.f + expf(-gate)));
+    out[t * width + c] = from_float<T>(act * up);
+  }
+}
+
+extern "C" {
+
+int se_router_topk(const float* logits, int64_t stride, const float* bias, int32_t* ids,
+                   float* weights, int tokens, int experts, int top_k, int softmax_scoring,
+                   int normalize, float scaling, hipStream_t stream) {
+  if (tokens <= 0) return SE_OK;
+  if (experts <= 0 || experts > SE_WAVE * ROUTER_MAX_PER_LANE) return SE_ERR_SHAPE;
+  if (top_k <= 0 || top_k > experts) return SE_ERR_SHAPE;
+  const int waves = 4;
+  router_topk_kernel<<<(tokens + waves - 1) / waves, waves * SE_WAVE, 0, stream>>>(
+      logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize,
+      scaling);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+int se_moe_align(const int32_t* ids, int assignments, int experts, int tile_rows, int32_t* sorted,
+                 int32_t* tile_expert, int32_t* counters, hipStream_t stream) {
+  if (assignments <= 0) return SE_OK;
+  if (experts <= 0 || experts > 4096 || tile_rows <= 0) return SE_ERR_SHAPE;
+  const size_t shmem = (3 * static_cast<size_t>(experts) + 1) * sizeof(int32_t);
+  moe_align_kernel<<<1, 1024, shmem, stream>>>(ids, assignments, experts, tile_rows, sorted,
+                                               tile_expert, counters);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+// mode 0: gate-up + SwiGLU (w = [experts, 2N, K]); mode 1: down (w = [experts, N, K]).
+// max_tiles bounds the grid; tiles beyond counters[0] leave at once.
+int se_grouped_gemm_generic(const void* in, const void* w, void* out, const int32_t* sorted,
+                            const int32_t* tile_expert, const int32_t* counters,
+                            const float* route_weight, int assignments, int top_k, int N, int K,
+                            int max_tiles, int mode, int dtype, hipStream_t stream) {
+  if (assignments <= 0) return SE_OK;
+  if (N <= 0 || K <= 0 || max_tiles <= 0 || max_tiles > 65535) return SE_ERR_SHAPE;
+  dim3 grid((N + GG_N - 1) / GG_N, max_tiles);
+#define SE_GG(T, MODE)                                                                          \
+  grouped_gemm_generic_kernel<T, MODE><<<grid, 256, 0, stream>>>(                               \
+      static_cast<const T*>(in), static_cast<const T*>(w), static_cast<T*>(out), sorted,        \
+      tile_expert, counters, route_weight, assignments, top_k, N, K)
+  if (dtype == SE_F32) {
+    if (mode == 0) SE_GG(float, 0); else SE_GG(float, 1);
+  } else {
+    if (mode == 0) SE_GG(bf16_t, 0); else SE_GG(bf16_t, 1);
+  }
+#undef SE_GG
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+int se_moe_sum(const void* y, void* out, int tokens, int top_k, int hidden, int dtype,
+               hipStream_t stream) {
+  if (tokens <= 0) return SE_OK;
+  if (dtype == SE_F32)
+    moe_sum_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(y),
+                                                      static_cast<float*>(out), top_k, hidden);
+  else
+    moe_sum_kernel<bf16_t><<<tokens, 256, 0, stream>>>(static_cast<const bf16_t*>(y),
+                                                       static_cast<bf16_t*>(out), top_k, hidden);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+int se_silu_mul(const void* x, void* out, int tokens, int width, int dtype, hipStream_t stream) {
+  if (tokens <= 0) return SE_OK;
+  if (dtype == SE_F32)
+    silu_mul_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(x),
+                                                       static_cast<float*>(out), width);
+  else
+    silu_mul_kernel<bf16_t><<<tokens, 256, 0, stream>>>(static_cast<const bf16_t*>(x),
+                                                        static_cast<bf16_t*>(out), width);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,323 @@
+"""Python face of the HIP kernels: shape checks on the host, then one ctypes call per kernel.
+
+All tensors live on the GPU; every call goes to the current stream and allocates nothing
+unless it says so.  A wrong shape or dtype raises ``ValueError`` before anything is launched;
+a size a kernel does not take raises ``KernelShapeError`` naming the limit.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+
+import torch
+
+from . import library
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelShapeError(ValueError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError(f"kernels take float32 or bfloat16 storage, got {dtype}") from None
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(status: int, what: str):
+    if status == 0:
+        return
+    if status == -1:
+        raise KernelShapeError(f"{what}: the kernel refuses these sizes")
+    raise RuntimeError(f"{what}: kernel launch failed (status {status})")
+
+
+def _require(cond: bool, message: str):
+    if not cond:
+        raise ValueError(message)
+
+
+def _i32(t: torch.Tensor, name: str):
+    _require(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
+
+
+_SIGNATURES = {
+    "norm": {
+        "se_embedding": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "se_rms_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
+                        c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p],
+    },
+    "rope_kv": {
+        "se_qk_norm_rope_store": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                  c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int,
+                                  c_int, c_int, c_int, c_void_p],
+    },
+    "attention_generic": {
+        "se_paged_attention_generic": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p,
+                                       c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
+                                       c_int, c_float, c_int, c_int, c_void_p],
+    },
+    "moe": {
+        "se_router_topk": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                           c_int, c_int, c_float, c_void_p],
+        "se_moe_align": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+        "se_grouped_gemm_generic": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_void_p],
+        "se_moe_sum": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "se_silu_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    },
+    "sampling": {
+        "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                      c_void_p, c_void_p],
+    },
+}
+
+
+class _Functions:
+    """Lazy table of bound entry points; a library is loaded (and built) at its first use."""
+
+    def __init__(self):
+        self._cache = {}
+
+    def get(self, lib_name: str, fn_name: str):
+        key = (lib_name, fn_name)
+        fn = self._cache.get(key)
+        if fn is None:
+            lib = library.load(lib_name)
+            fn = getattr(lib, fn_name)
+            fn.argtypes = _SIGNATURES[lib_name][fn_name]
+            fn.restype = c_int
+            self._cache[key] = fn
+        return fn
+
+
+_fn = _Functions()
+
+
+def moe_tile_bounds(assignments: int, experts: int, tile_rows: int) -> tuple[int, int]:
+    """(capacity of the sorted list, largest possible number of tiles) for an alignment."""
+    touched = min(experts, assignments)
+    return assignments + touched * (tile_rows - 1), assignments // tile_rows + touched
+
+
+class MoeWorkspace:
+    """Scratch tensors of the expert pipeline, sized for a largest number of tokens."""
+
+    def __init__(self, max_tokens: int, top_k: int, experts: int, hidden: int, intermediate: int,
+                 dtype: torch.dtype, device, tile_rows: int = 16):
+        assignments = max_tokens * top_k
+        capacity, max_tiles = moe_tile_bounds(assignments, experts, tile_rows)
+        self.max_tokens, self.top_k, self.experts = max_tokens, top_k, experts
+        self.hidden, self.intermediate, self.dtype, self.tile_rows = hidden, intermediate, dtype, tile_rows
+        self.sorted = torch.empty(capacity, dtype=torch.int32, device=device)
+        self.tile_expert = torch.empty(max_tiles, dtype=torch.int32, device=device)
+        self.counters = torch.zeros(2, dtype=torch.int32, device=device)
+        self.act = torch.empty(assignments, intermediate, dtype=dtype, device=device)
+        self.slot_out = torch.empty(assignments, hidden, dtype=dtype, device=device)
+
+    def fits(self, tokens, top_k, experts, hidden, intermediate, dtype) -> bool:
+        return (tokens <= self.max_tokens and top_k == self.top_k and experts == self.experts
+                and hidden == self.hidden and intermediate == self.intermediate and dtype == self.dtype)
+
+
+class HipKernels:
+    """The kernel interface of the engine, served by the gfx950 libraries."""
+
+    libraries = ("norm", "rope_kv", "attention_generic", "moe", "sampling")
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise library.KernelLibraryError(
+                "the HIP kernels need a GPU: torch.cuda.is_available() is False")
+
+    # ------------------------------------------------------------------ embedding / norms
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor):
+        _i32(ids, "ids")
+        tokens, hidden = out.shape
+        _require(ids.numel() == tokens and table.shape[1] == hidden and table.dtype == out.dtype
+                 and table.is_contiguous() and out.is_contiguous(), "embedding: shape/dtype mismatch")
+        _check(_fn.get("norm", "se_embedding")(_ptr(ids), _ptr(table), _ptr(out), tokens, hidden,
+                                               _code(out.dtype), _stream()), "embedding")
+
+    def rms_norm(self, x, weight, eps: float, out, residual=None, rows=None, write_residual=True):
+        """``out = norm(x (+ residual)) * weight``; with ``residual`` the rounded sum replaces it
+        (unless ``write_residual`` is False).  ``rows`` (int32) selects input rows: ``out[j]`` is
+        the norm of row ``rows[j]``.  ``out`` may be ``x``."""
+        hidden = x.shape[-1]
+        n_out = out.shape[0]
+        _require(x.dim() == 2 and out.dim() == 2 and out.shape[1] == hidden, "rms_norm: x/out shapes")
+        _require(x.stride(1) == 1 and out.stride(1) == 1, "rms_norm: rows must be dense")
+        _require(weight.shape == (hidden,) and weight.is_contiguous(), "rms_norm: weight shape")
+        _require(out.dtype == x.dtype, "rms_norm: out dtype")
+        if residual is not None:
+            _require(residual.shape == x.shape and residual.dtype == x.dtype and residual.stride(1) == 1,
+                     "rms_norm: residual shape/dtype")
+        if rows is not None:
+            _i32(rows, "rows")
+            _require(rows.numel() == n_out, "rms_norm: rows/out mismatch")
+            write_residual = False
+        else:
+            _require(n_out == x.shape[0], "rms_norm: out rows")
+        if hidden > 15360:
+            raise KernelShapeError(f"rms_norm: hidden size {hidden} is above the kernel's limit 15360")
+        _check(_fn.get("norm", "se_rms_norm")(
+            _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), n_out, hidden, float(eps),
+            x.stride(0), residual.stride(0) if residual is not None else 0, out.stride(0),
+            int(bool(write_residual)), _code(x.dtype), _code(weight.dtype), _stream()), "rms_norm")
+
+    # ------------------------------------------------------------------ attention inputs
+    def qk_norm_rope_store(self, qkv, positions, cos_sin, q_weight, k_weight, eps, heads, kv_heads,
+                           head_dim, rotary_dim, cache=None, slots=None, page_size=0):
+        """In place on ``qkv [T, (heads + 2 kv_heads) * head_dim]``: flat QK norm (if weights are
+        given), partial rotation by ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half), and
+        the write of k and v to ``cache [pages, 2, kv_heads, page_size, head_dim]`` at ``slots``."""
+        tokens = qkv.shape[0]
+        width = (heads + 2 * kv_heads) * head_dim
+        _require(qkv.dim() == 2 and qkv.shape[1] == width and qkv.stride(1) == 1, "qkv shape")
+        _i32(positions, "positions")
+        _require(positions.numel() == tokens, "positions length")
+        _require(rotary_dim % 2 == 0 and 0 <= rotary_dim <= head_dim, "rotary_dim must be even and <= head_dim")
+        if rotary_dim:
+            _require(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
+                     and cos_sin.shape[1] == rotary_dim, "cos_sin table shape/dtype")
+        if q_weight is not None:
+            _require(q_weight.shape == (heads * head_dim,) and k_weight.shape == (kv_heads * head_dim,)
+                     and q_weight.dtype == k_weight.dtype, "qk norm weight shapes")
+        write_kv = cache is not None
+        if write_kv:
+            _i32(slots, "slots")
+            _require(slots.numel() == tokens, "slots length")
+            _require(cache.dtype == qkv.dtype and cache.is_contiguous() and cache.dim() == 5
+                     and tuple(cache.shape[1:]) == (2, kv_heads, page_size, head_dim), "cache layout")
+        wd = _code(q_weight.dtype) if q_weight is not None else _code(qkv.dtype)
+        _check(_fn.get("rope_kv", "se_qk_norm_rope_store")(
+            _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(cos_sin) if rotary_dim else None,
+            _ptr(q_weight), _ptr(k_weight), float(eps), tokens, heads, kv_heads, head_dim, rotary_dim,
+            _ptr(cache), _ptr(slots), page_size, int(write_kv), _code(qkv.dtype), wd, _stream()),
+            "qk_norm_rope_store")
+
+    def paged_attention(self, q, cache, meta, out, scale: float, window: int = 0):
+        """Causal attention of every token of the step against its request's pages.
+
+        ``q``: ``[T, heads, head_dim]`` view (token stride free, heads dense); ``cache``:
+        ``[pages, 2, kv_heads, page_size, head_dim]``; ``meta``: an object with ``block_table``
+        (int32 ``[rows, max_pages]``), ``token_row`` and ``positions`` (int32 ``[T]``);
+        ``out``: ``[T, heads * head_dim]``."""
+        tokens, heads, head_dim = q.shape
+        kv_heads, page_size = cache.shape[2], cache.shape[3]
+        _require(q.stride(2) == 1 and q.stride(1) == head_dim, "q heads must be dense")
+        _require(cache.dim() == 5 and cache.shape[1] == 2 and cache.shape[4] == head_dim
+                 and cache.is_contiguous() and cache.dtype == q.dtype, "cache layout")
+        _require(out.shape == (tokens, heads * head_dim) and out.stride(1) == 1 and out.dtype == q.dtype,
+                 "attention out shape")
+        _i32(meta.token_row, "token_row"); _i32(meta.positions, "positions")
+        _require(meta.block_table.dtype == torch.int32 and meta.block_table.dim() == 2
+                 and meta.block_table.stride(1) == 1, "block_table layout")
+        _require(meta.token_row.numel() == tokens and meta.positions.numel() == tokens, "meta length")
+        if head_dim % 8 or head_dim > 512:
+            raise KernelShapeError(f"attention: head_dim {head_dim} must be a multiple of 8, at most 512")
+        if heads % kv_heads:
+            raise KernelShapeError(f"attention: {heads} heads do not divide into {kv_heads} kv heads")
+        _check(_fn.get("attention_generic", "se_paged_attention_generic")(
+            _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
+            _ptr(meta.token_row), _ptr(meta.positions), _ptr(out), out.stride(0), tokens, heads,
+            kv_heads, head_dim, page_size, float(scale), int(window or 0), _code(q.dtype), _stream()),
+            "paged_attention")
+
+    # ------------------------------------------------------------------ mixture of experts
+    def router_topk(self, logits, bias, top_k: int, ids, weights, scoring="sigmoid", normalize=True,
+                    scaling: float = 1.0):
+        tokens, experts = logits.shape
+        _require(logits.dtype == torch.float32 and logits.stride(1) == 1, "router logits must be float32")
+        if bias is not None:
+            _require(bias.dtype == torch.float32 and bias.shape == (experts,) and bias.is_contiguous(),
+                     "router bias must be float32 [experts]")
+        _i32(ids, "ids")
+        _require(ids.shape == (tokens, top_k) and weights.shape == (tokens, top_k)
+                 and weights.dtype == torch.float32 and weights.is_contiguous(), "router outputs")
+        if scoring not in ("sigmoid", "softmax"):
+            raise ValueError(f"router scoring '{scoring}' is unknown (sigmoid, softmax)")
+        if experts > 1024:
+            raise KernelShapeError(f"router: {experts} experts are above the kernel's limit 1024")
+        _require(1 <= top_k <= experts, "1 <= top_k <= experts")
+        _check(_fn.get("moe", "se_router_topk")(
+            _ptr(logits), logits.stride(0), _ptr(bias), _ptr(ids), _ptr(weights), tokens, experts,
+            top_k, int(scoring == "softmax"), int(bool(normalize)), float(scaling), _stream()),
+            "router_topk")
+
+    def moe_align(self, ids, experts: int, ws: MoeWorkspace):
+        _i32(ids, "ids")
+        assignments = ids.numel()
+        capacity, max_tiles = moe_tile_bounds(assignments, experts, ws.tile_rows)
+        _require(ws.sorted.numel() >= capacity and ws.tile_expert.numel() >= max_tiles, "workspace too small")
+        if experts > 4096:
+            raise KernelShapeError(f"moe_align: {experts} experts are above the kernel's limit 4096")
+        _check(_fn.get("moe", "se_moe_align")(
+            _ptr(ids), assignments, experts, ws.tile_rows, _ptr(ws.sorted), _ptr(ws.tile_expert),
+            _ptr(ws.counters), _stream()), "moe_align")
+        return max_tiles
+
+    def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace):
+        """``out[t] = sum_k weights[t,k] * W2_e(silu(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``;
+        ``w13 [E, 2I, h]`` holds gate rows then up rows, ``w2 [E, h, I]``."""
+        tokens, hidden = x.shape
+        experts, two_i, _ = w13.shape
+        inter = two_i // 2
+        top_k = ids.shape[1]
+        _require(x.is_contiguous() and out.is_contiguous() and out.shape == x.shape, "moe x/out")
+        _require(w13.shape == (experts, 2 * inter, hidden) and w2.shape == (experts, hidden, inter)
+                 and w13.is_contiguous() and w2.is_contiguous(), "expert weight shapes")
+        _require(w13.dtype == x.dtype and w2.dtype == x.dtype and out.dtype == x.dtype, "moe dtypes")
+        _require(ids.shape == (tokens, top_k) and weights.shape == (tokens, top_k)
+                 and weights.dtype == torch.float32 and weights.is_contiguous(), "routing shapes")
+        _require(ws.fits(tokens, top_k, experts, hidden, inter, x.dtype), "moe workspace does not fit")
+        assignments = tokens * top_k
+        max_tiles = self.moe_align(ids, experts, ws)
+        if max_tiles > 65535:
+            raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
+        gg = _fn.get("moe", "se_grouped_gemm_generic")
+        code = _code(x.dtype)
+        _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                  _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, code,
+                  _stream()), "moe gate-up")
+        _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                  _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
+                  code, _stream()), "moe down")
+        _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
+                                            _stream()), "moe_sum")
+
+    def silu_mul(self, x, out):
+        tokens, two_w = x.shape
+        _require(x.is_contiguous() and out.is_contiguous() and out.shape == (tokens, two_w // 2)
+                 and out.dtype == x.dtype, "silu_mul shapes")
+        _check(_fn.get("moe", "se_silu_mul")(_ptr(x), _ptr(out), tokens, two_w // 2, _code(x.dtype),
+                                             _stream()), "silu_mul")
+
+    # ------------------------------------------------------------------ sampling
+    def sample(self, logits, temperature, top_k, top_p, seeds, out):
+        """One token per row of float ``logits``; ``temperature`` (float32), ``top_k`` (int32),
+        ``top_p`` (float32) and ``seeds`` (int64, used as 64 raw bits) have one entry per row
+        and may each be None (greedy / off / off / 0)."""
+        rows, vocab = logits.shape
+        _require(logits.dtype == torch.float32 and logits.stride(1) == 1, "logits must be float32")
+        _i32(out, "out")
+        _require(out.numel() == rows, "sample out length")
+        for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                            ("top_p", top_p, torch.float32), ("seeds", seeds, torch.int64)):
+            if t is not None:
+                _require(t.dtype == dt and t.numel() == rows and t.is_contiguous(), f"sample {name}")
+        _check(_fn.get("sampling", "se_sample")(
+            _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+            _ptr(seeds), _ptr(out), _stream()), "sample")

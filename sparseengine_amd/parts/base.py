@@ -1,0 +1,118 @@
+"""What every part of a layer has in common, and the registries that find a part by the
+``kind`` of its spec.
+
+A part is built from its spec alone (no allocation), declares its parameters by local name, is
+handed the allocated tensors once (``bind``) and then runs on a ``ForwardBatch``.  It never
+learns which model it is in: names of checkpoint tensors, layer counts and the like stay with
+the architecture module.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamDecl:
+    """Shape and storage policy of one parameter.
+
+    policy "engine":  the engine's dtype, except that a tensor the checkpoint stores in 32-bit
+                      float stays float32;
+    policy "float32": always float32 (router tables);
+    policy "int32":   integer tables.
+    """
+    shape: tuple[int, ...]
+    policy: str = "engine"
+
+
+@dataclass(frozen=True)
+class PagedKVRequest:
+    """A mixer that keeps keys and values of ``window`` (None: all) past tokens in pages."""
+    kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateRequest:
+    """A mixer that keeps tensors of fixed size per request: name -> (shape, dtype or None for
+    the engine's dtype).  They are zeroed when a request is admitted."""
+    tensors: tuple[tuple[str, tuple[int, ...], torch.dtype | None], ...]
+
+
+class Part:
+    """Base of mixers, feed-forwards, norms, position encodings and blocks."""
+    kernel_libraries: tuple[str, ...] = ()
+
+    def param_decls(self) -> dict[str, ParamDecl]:
+        return {}
+
+    def bind(self, params: dict[str, torch.Tensor]) -> None:
+        self.params = params
+
+    def children(self) -> dict[str, "Part"]:
+        return {}
+
+    # flattened views over the tree of parts ---------------------------------------------
+    def all_param_decls(self, prefix: str = "") -> dict[str, ParamDecl]:
+        out = {prefix + name: decl for name, decl in self.param_decls().items()}
+        for child_name, child in self.children().items():
+            out.update(child.all_param_decls(f"{prefix}{child_name}."))
+        return out
+
+    def bind_all(self, tensors: dict[str, torch.Tensor], prefix: str = "") -> None:
+        self.bind({name: tensors[prefix + name] for name in self.param_decls()})
+        for child_name, child in self.children().items():
+            child.bind_all(tensors, f"{prefix}{child_name}.")
+
+    def all_kernel_libraries(self) -> set[str]:
+        libs = set(self.kernel_libraries)
+        for child in self.children().values():
+            libs |= child.all_kernel_libraries()
+        return libs
+
+
+class PartRegistry:
+    """kind -> factory(spec, **context).  One instance per family of parts."""
+
+    def __init__(self, family: str):
+        self.family = family
+        self._factories: dict[str, Callable] = {}
+
+    def register(self, kind: str, factory: Callable | None = None):
+        def add(f):
+            self._factories[kind] = f
+            return f
+        return add(factory) if factory is not None else add
+
+    def build(self, spec, **context):
+        kind = getattr(spec, "kind", None)
+        if kind not in self._factories:
+            raise KeyError(f"no {self.family} registered for kind {kind!r}; known: "
+                           f"{sorted(self._factories)}")
+        return self._factories[kind](spec, **context)
+
+    def kinds(self) -> list[str]:
+        return sorted(self._factories)
+
+
+MIXERS = PartRegistry("mixer")
+FEED_FORWARDS = PartRegistry("feed-forward")
+NORMS = PartRegistry("norm")
+POSITIONS = PartRegistry("position encoding")
+BLOCKS = PartRegistry("block")
+
+
+@dataclass
+class StepScratch:
+    """Buffers a part asks for once and reuses every step, sized for the largest step."""
+    tensors: dict[str, torch.Tensor] = field(default_factory=dict)
+
+    def get(self, key: str, shape: tuple[int, ...], dtype: torch.dtype, device) -> torch.Tensor:
+        t = self.tensors.get(key)
+        if t is None or t.dtype != dtype or any(a < b for a, b in zip(t.shape, shape)) or t.dim() != len(shape):
+            t = torch.empty(shape, dtype=dtype, device=device)
+            self.tensors[key] = t
+        return t

@@ -1,0 +1,368 @@
+"""Each HIP kernel alone against its plain twin, at sizes other than the engine's."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from tests.twin_kernels import TwinKernels
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from sparseengine_amd.kernels.hip_ops import HipKernels
+    return HipKernels()
+
+
+@pytest.fixture(scope="module")
+def twin():
+    return TwinKernels()
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1.6e-2)
+
+
+def randn(*shape, dtype, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,hidden,vocab", [(1, 64, 50), (37, 3072, 1000), (5, 200, 77)])
+def test_embedding(hip, dtype, tokens, hidden, vocab):
+    table = randn(vocab, hidden, dtype=dtype)
+    ids = torch.randint(0, vocab, (tokens,), dtype=torch.int32).cuda()
+    out = torch.empty(tokens, hidden, dtype=dtype, device="cuda")
+    hip.embedding(ids, table, out)
+    assert torch.equal(out, table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", [None, torch.float32])
+@pytest.mark.parametrize("tokens,hidden", [(1, 64), (7, 3072), (33, 200), (3, 6144), (2, 15360)])
+def test_rms_norm_plain_and_fused(hip, twin, dtype, wdtype, tokens, hidden):
+    wdtype = wdtype or dtype
+    x = randn(tokens, hidden, dtype=dtype, seed=1)
+    res = randn(tokens, hidden, dtype=dtype, seed=2)
+    w = (1 + 0.2 * torch.randn(hidden)).to(wdtype).cuda()
+    # plain
+    out_h, out_t = torch.empty_like(x), torch.empty_like(x)
+    hip.rms_norm(x, w, 1e-5, out_h)
+    twin.rms_norm(x, w, 1e-5, out_t)
+    torch.testing.assert_close(out_h, out_t, **tol(dtype))
+    torch.testing.assert_close(out_h.float(), torch.nn.functional.rms_norm(x.float(), (hidden,), w.float(), 1e-5), **tol(dtype))
+    # fused add, in place: the residual is the rounded sum, bit for bit
+    xh, rh, xt, rt = x.clone(), res.clone(), x.clone(), res.clone()
+    hip.rms_norm(xh, w, 1e-5, xh, residual=rh)
+    twin.rms_norm(xt, w, 1e-5, xt, residual=rt)
+    assert torch.equal(rh, (x.float() + res.float()).to(dtype))
+    torch.testing.assert_close(xh, xt, **tol(dtype))
+    # row selection leaves the residual alone
+    rows = torch.tensor([tokens - 1, 0], dtype=torch.int32).cuda()
+    oh = torch.empty(2, hidden, dtype=dtype, device="cuda")
+    ot = torch.empty_like(oh)
+    r_before = res.clone()
+    hip.rms_norm(x, w, 1e-5, oh, residual=res, rows=rows)
+    twin.rms_norm(x, w, 1e-5, ot, residual=res, rows=rows)
+    torch.testing.assert_close(oh, ot, **tol(dtype))
+    assert torch.equal(res, r_before)
+
+
+def test_rms_norm_refuses_wide_rows(hip):
+    from sparseengine_amd.kernels.hip_ops import KernelShapeError
+    x = torch.zeros(1, 16384, device="cuda")
+    with pytest.raises(KernelShapeError):
+        hip.rms_norm(x, torch.ones(16384, device="cuda"), 1e-6, torch.empty_like(x))
+
+
+def rope_table(max_pos, rotary_dim, theta):
+    inv = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    f = torch.arange(max_pos, dtype=torch.float32)[:, None] * inv[None]
+    return torch.cat((f.cos(), f.sin()), -1).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rotary,norm,page", [
+    (4, 2, 16, 8, True, 16), (6, 3, 32, 32, False, 16), (48, 8, 128, 64, True, 64),
+    (5, 5, 48, 16, True, 32), (6, 1, 128, 64, True, 16), (3, 1, 80, 0, False, 16)])
+def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary, norm, page):
+    tokens, pages = 9, 7
+    width = (heads + 2 * kv_heads) * head_dim
+    qkv = randn(tokens, width, dtype=dtype, seed=3)
+    positions = torch.tensor([0, 1, 17, 127, 1023, 5, 6, 7, 300], dtype=torch.int32).cuda()
+    table = rope_table(2048, rotary, 5e6) if rotary else torch.zeros(1, 1, device="cuda")
+    qw = (1 + 0.1 * torch.randn(heads * head_dim)).to(dtype).cuda() if norm else None
+    kw = (1 + 0.1 * torch.randn(kv_heads * head_dim)).to(dtype).cuda() if norm else None
+    slots = torch.tensor([3 * page + 1, 0, page - 1, 5 * page, -1, 2 * page + 3, 2 * page + 4, 6 * page + page - 1, page],
+                         dtype=torch.int32).cuda()
+    cache_h = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device="cuda")
+    cache_t = cache_h.clone()
+    a, b = qkv.clone(), qkv.clone()
+    hip.qk_norm_rope_store(a, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_h, slots, page)
+    twin.qk_norm_rope_store(b, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_t, slots, page)
+    torch.testing.assert_close(a, b, **tol(dtype))
+    torch.testing.assert_close(cache_h, cache_t, **tol(dtype))
+    # v is never touched; without a norm the dims beyond the rotary part are bit-equal to the input
+    assert torch.equal(a[:, (heads + kv_heads) * head_dim:], qkv[:, (heads + kv_heads) * head_dim:])
+    if not norm:
+        q_in = qkv[:, :heads * head_dim].view(tokens, heads, head_dim)
+        assert torch.equal(a[:, :heads * head_dim].view(tokens, heads, head_dim)[..., rotary:], q_in[..., rotary:])
+    # the cache holds exactly what the step's k and v rows hold
+    kq = a[:, heads * head_dim:(heads + kv_heads) * head_dim].view(tokens, kv_heads, head_dim)
+    for t in range(tokens):
+        s = int(slots[t])
+        if s >= 0:
+            assert torch.equal(cache_h[s // page, 0, :, s % page], kq[t])
+
+
+def make_paged(dtype, kv_heads, head_dim, page, lens, seed=0, extra_pages=3):
+    """Random k/v for requests of the given lengths scattered over shuffled pages."""
+    g = torch.Generator().manual_seed(seed)
+    need = [(n + page - 1) // page for n in lens]
+    total = sum(need) + extra_pages
+    perm = torch.randperm(total, generator=g).tolist()
+    cache = (torch.randn(total, 2, kv_heads, page, head_dim, generator=g)).to(dtype).cuda()
+    table = torch.full((len(lens), max(need) + 1), -1, dtype=torch.int32)
+    for r, n in enumerate(need):
+        for j in range(n):
+            table[r, j] = perm.pop()
+    return cache, table.cuda()
+
+
+def dense_attention(q, cache, table, row, pos, scale, window, page):
+    """Reference through the library routine: gather the request's keys, call SDPA for one query."""
+    first = max(0, pos - window + 1) if window else 0
+    n = torch.arange(first, pos + 1, device="cuda")
+    pages = table[row, n // page].long()
+    k = cache[pages, 0, :, n % page, :].float().transpose(0, 1)   # [Hkv, n, D]
+    v = cache[pages, 1, :, n % page, :].float().transpose(0, 1)
+    H, D = q.shape
+    group = H // k.shape[0]
+    k = k.repeat_interleave(group, 0)
+    v = v.repeat_interleave(group, 0)
+    o = torch.nn.functional.scaled_dot_product_attention(q.float()[:, None, :], k, v, scale=scale)
+    return o[:, 0, :].reshape(-1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page,window", [
+    (4, 2, 16, 16, 0), (6, 3, 32, 16, 0), (48, 8, 128, 64, 0), (12, 2, 64, 32, 0),
+    (5, 1, 48, 16, 0), (8, 8, 80, 16, 0), (4, 2, 16, 16, 20), (6, 1, 128, 64, 100)])
+def test_paged_attention_mixed_batch(hip, twin, dtype, heads, kv_heads, head_dim, page, window):
+    # three requests: a whole prompt, a portion on top of a cached prefix, a single decoded token
+    lens = [37, 150, 301]
+    q_lens = [37, 23, 1]
+    cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=heads)
+    token_row, positions = [], []
+    for r, (n, ql) in enumerate(zip(lens, q_lens)):
+        token_row += [r] * ql
+        positions += list(range(n - ql, n))
+    T = len(token_row)
+    meta = SimpleNamespace(block_table=table, token_row=torch.tensor(token_row, dtype=torch.int32).cuda(),
+                           positions=torch.tensor(positions, dtype=torch.int32).cuda())
+    qkv = randn(T, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=9)
+    q = qkv[:, :heads * head_dim].view(T, heads, head_dim)
+    scale = head_dim ** -0.5
+    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device="cuda")
+    out_t = torch.empty_like(out_h)
+    hip.paged_attention(q, cache, meta, out_h, scale, window)
+    twin.paged_attention(q, cache, meta, out_t, scale, window)
+    torch.testing.assert_close(out_h, out_t, **tol(dtype))
+    for t in (0, 36, 37, 59, 60):
+        ref = dense_attention(q[t], cache, table, token_row[t], positions[t], scale, window, page)
+        torch.testing.assert_close(out_h[t].float(), ref, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_one_far_key(hip, dtype):
+    """One key far back in a long context is made to dominate: the output must be its value."""
+    heads, kv_heads, head_dim, page = 8, 2, 64, 16
+    n = 1000
+    cache, table = make_paged(dtype, kv_heads, head_dim, page, [n], seed=5)
+    q = randn(1, heads, head_dim, dtype=dtype, seed=6)
+    for target in (0, 15, 16, 513, 998, 999):
+        c = cache.clone()
+        pg, off = int(table[0, target // page]), target % page
+        for h in range(heads):
+            kvh = h // (heads // kv_heads)
+        # key of the target = 40 * direction of the first query head of each group
+        for kvh in range(kv_heads):
+            qh = q[0, kvh * (heads // kv_heads)].float()
+            c[pg, 0, kvh, off] = (qh / qh.norm() * 60).to(dtype)
+        meta = SimpleNamespace(block_table=table, token_row=torch.zeros(1, dtype=torch.int32).cuda(),
+                               positions=torch.tensor([n - 1], dtype=torch.int32).cuda())
+        out = torch.empty(1, heads * head_dim, dtype=dtype, device="cuda")
+        hip.paged_attention(q, c, meta, out, 1.0, 0)
+        for kvh in range(kv_heads):
+            head = kvh * (heads // kv_heads)
+            got = out[0, head * head_dim:(head + 1) * head_dim].float()
+            torch.testing.assert_close(got, c[pg, 1, kvh, off].float(), rtol=2e-2, atol=2e-2)
+
+
+def test_router_matches_library_topk(hip, twin):
+    torch.manual_seed(27)
+    for tokens, experts, k in [(4096, 256, 8), (33, 8, 2), (17, 16, 4), (5, 100, 7), (3, 1, 1), (9, 1000, 16)]:
+        logits = (torch.randn(tokens, experts) * 3).cuda()
+        bias = (torch.randn(experts) * 0.1).cuda()
+        ids = torch.empty(tokens, k, dtype=torch.int32, device="cuda")
+        w = torch.empty(tokens, k, device="cuda")
+        hip.router_topk(logits, bias, k, ids, w)
+        s = torch.sigmoid(logits)
+        ref_ids = torch.topk(s + bias, k, dim=-1).indices
+        assert torch.equal(ids.long().sort(-1).values, ref_ids.sort(-1).values)
+        ref_w = s.gather(1, ids.long())
+        ref_w = ref_w / ref_w.sum(-1, keepdim=True)
+        torch.testing.assert_close(w, ref_w, rtol=1e-5, atol=1e-6)
+        ids_t = torch.empty_like(ids); w_t = torch.empty_like(w)
+        twin.router_topk(logits, bias, k, ids_t, w_t)
+        assert torch.equal(ids, ids_t)
+
+
+def test_router_ties_nonfinite_and_bias(hip, twin):
+    # tie order and non-finite rows as in the reference's tests/test_minimax_m2_router.py:68-122
+    logits = torch.zeros(4, 256).cuda()
+    logits[1, :9] = 1
+    logits[2, 120:129] = 1
+    logits[3] = (torch.arange(256).cuda() // 8).float()
+    bias = torch.zeros(256).cuda()
+    ids = torch.empty(4, 8, dtype=torch.int32, device="cuda"); w = torch.empty(4, 8, device="cuda")
+    hip.router_topk(logits, bias, 8, ids, w)
+    assert ids[0].tolist() == list(range(8))
+    assert ids[1].tolist() == list(range(8))
+    assert ids[2].tolist() == list(range(120, 128))
+    s3 = torch.sigmoid(logits[3])   # saturates to 1.0 from index 136 on: the ties go to the lowest indices
+    assert ids[3].tolist() == torch.nonzero(s3 == s3.max()).flatten()[:8].tolist()
+    torch.testing.assert_close(w, torch.full_like(w, 0.125))
+    logits = torch.zeros(6, 256).cuda()
+    logits[0, 3] = float("nan"); logits[1, 7] = float("inf"); logits[2, 9] = -float("inf")
+    logits[3] = 100; logits[4] = -100
+    bias2 = bias.clone(); bias2[5] = float("nan")
+    hip.router_topk(logits[:5], bias, 8, ids := torch.empty(5, 8, dtype=torch.int32, device="cuda"),
+                    w := torch.empty(5, 8, device="cuda"))
+    assert 3 in ids[0].tolist() and torch.isnan(w[0]).all()
+    assert 7 in ids[1].tolist() and 9 not in ids[2].tolist()
+    assert ids[3].tolist() == list(range(8)) and ids[4].tolist() == list(range(8))
+    hip.router_topk(logits[5:], bias2, 8, ids6 := torch.empty(1, 8, dtype=torch.int32, device="cuda"),
+                    w6 := torch.empty(1, 8, device="cuda"))
+    assert ids6[0].tolist() == [5, 0, 1, 2, 3, 4, 6, 7]
+    # a bias of +2 on experts 0..7 selects exactly them and leaves the weights unbiased
+    logits = torch.linspace(-4, 4, 256)[None].cuda()
+    bias3 = torch.zeros(256).cuda(); bias3[:8] = 2
+    hip.router_topk(logits, bias3, 8, ids6, w6)
+    assert sorted(ids6[0].tolist()) == list(range(8))
+    s = torch.sigmoid(logits[0, :8])
+    torch.testing.assert_close(w6[0].sort().values, (s / s.sum()).sort().values)
+    # softmax scoring, no renormalisation, scaling
+    logits = torch.randn(7, 40).cuda()
+    ids7 = torch.empty(7, 3, dtype=torch.int32, device="cuda"); w7 = torch.empty(7, 3, device="cuda")
+    hip.router_topk(logits, None, 3, ids7, w7, scoring="softmax", normalize=False, scaling=2.5)
+    ref = torch.topk(torch.softmax(logits, -1), 3)
+    assert torch.equal(ids7.long().sort(-1).values, ref.indices.sort(-1).values)
+    torch.testing.assert_close(w7.sort(-1).values, (ref.values * 2.5).sort(-1).values)
+
+
+def test_moe_align_groups_every_assignment_once(hip):
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    for tokens, k, experts in [(1, 8, 256), (2048, 8, 256), (33, 2, 8), (100, 4, 16), (7, 1, 1)]:
+        ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
+        ws = MoeWorkspace(tokens, k, experts, 16, 16, torch.float32, "cuda")
+        ws.sorted.fill_(-7); ws.tile_expert.fill_(-7)
+        hip.moe_align(ids, experts, ws)
+        n_tiles, n_sorted = ws.counters.tolist()
+        assert n_sorted == n_tiles * 16
+        sorted_ids = ws.sorted[:n_sorted].cpu()
+        real = sorted_ids[sorted_ids < tokens * k]
+        assert sorted(real.tolist()) == list(range(tokens * k))
+        flat = ids.flatten().cpu()
+        te = ws.tile_expert[:n_tiles].cpu()
+        assert (te[1:] >= te[:-1]).all()
+        for t in range(n_tiles):
+            chunk = sorted_ids[t * 16:(t + 1) * 16]
+            chunk = chunk[chunk < tokens * k]
+            assert chunk.numel() > 0 and (flat[chunk.long()] == te[t]).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,hidden,inter,experts,k", [
+    (1, 64, 32, 8, 2), (45, 96, 48, 16, 4), (130, 200, 72, 5, 5), (9, 256, 128, 1, 1), (64, 384, 160, 32, 8)])
+def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    x = randn(tokens, hidden, dtype=dtype, seed=11)
+    w13 = randn(experts, 2 * inter, hidden, dtype=dtype, scale=hidden ** -0.5, seed=12)
+    w2 = randn(experts, hidden, inter, dtype=dtype, scale=inter ** -0.5, seed=13)
+    ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
+    weights = torch.rand(tokens, k).cuda()
+    weights = weights / weights.sum(-1, keepdim=True)
+    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+    out_h = torch.empty_like(x); out_t = torch.empty_like(x)
+    hip.moe_experts(x, w13, w2, ids, weights, out_h, ws)
+    twin.moe_experts(x, w13, w2, ids, weights, out_t)
+    torch.testing.assert_close(out_h, out_t, **tol(dtype))
+    if experts == 1:   # one expert, k = 1: a plain SwiGLU feed-forward
+        xf = x.float()
+        ref = (torch.nn.functional.silu(xf @ w13[0, :inter].float().T) * (xf @ w13[0, inter:].float().T)) @ w2[0].float().T
+        torch.testing.assert_close(out_h.float(), ref, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(hip, twin, dtype):
+    x = randn(13, 2 * 72, dtype=dtype, seed=4)
+    a = torch.empty(13, 72, dtype=dtype, device="cuda"); b = torch.empty_like(a)
+    hip.silu_mul(x, a); twin.silu_mul(x, b)
+    torch.testing.assert_close(a, b, **tol(dtype))
+    torch.testing.assert_close(a.float(), torch.nn.functional.silu(x[:, :72].float()) * x[:, 72:].float(), **tol(dtype))
+
+
+def test_sampling(hip, twin):
+    torch.manual_seed(3)
+    rows, vocab = 6, 1000
+    logits = (torch.randn(rows, vocab) * 2).cuda()
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    # greedy, top_k = 1 and a tiny top_p all give the arg-max (reference tests/test_sampler.py:39-58)
+    hip.sample(logits, None, None, None, None, out)
+    assert torch.equal(out.long(), logits.argmax(-1))
+    temp = torch.full((rows,), 0.7).cuda()
+    seeds = torch.arange(rows, dtype=torch.int64).cuda() * 7919 + 1
+    hip.sample(logits, temp, torch.ones(rows, dtype=torch.int32).cuda(), None, seeds, out)
+    assert torch.equal(out.long(), logits.argmax(-1))
+    hip.sample(logits, temp, None, torch.full((rows,), 0.01).cuda(), seeds, out)
+    assert torch.equal(out.long(), logits.argmax(-1))
+    # mixed rows against the twin: same noise, same choice
+    temp = torch.tensor([0.0, 0.8, 1.0, 0.7, 1.3, 0.5]).cuda()
+    top_k = torch.tensor([0, 0, 5, 0, 50, 3], dtype=torch.int32).cuda()
+    top_p = torch.tensor([1.0, 1.0, 1.0, 0.6, 0.9, 0.5]).cuda()
+    ref = torch.empty_like(out)
+    hip.sample(logits, temp, top_k, top_p, seeds, out)
+    twin.sample(logits, temp, top_k, top_p, seeds, ref)
+    assert torch.equal(out, ref)
+    # a row's draw does not depend on the rest of the batch
+    one = torch.empty(1, dtype=torch.int32, device="cuda")
+    for r in range(rows):
+        hip.sample(logits[r:r + 1], temp[r:r + 1], top_k[r:r + 1], top_p[r:r + 1], seeds[r:r + 1], one)
+        assert int(one) == int(out[r])
+
+
+def test_sampling_distribution(hip):
+    # 32768 draws at temperature 0.7 stay within 0.015 of softmax(l / 0.7) (reference tests/test_sampler.py:351-367)
+    torch.manual_seed(5)
+    vocab, draws = 12, 32768
+    row = torch.randn(vocab) * 1.5
+    logits = row[None].repeat(draws, 1).cuda()
+    temp = torch.full((draws,), 0.7).cuda()
+    seeds = (torch.arange(draws, dtype=torch.int64) * 0x9E3779B1 + 12345).cuda()
+    out = torch.empty(draws, dtype=torch.int32, device="cuda")
+    hip.sample(logits, temp, None, None, seeds, out)
+    freq = torch.bincount(out.long().cpu(), minlength=vocab).float() / draws
+    assert (freq - torch.softmax(row / 0.7, -1)).abs().max() < 0.015
+    # top-k then top-p: the nucleus is taken over the survivors of top-k (tests/test_sampler.py:332-349)
+    logits = torch.tensor([[3.0, 2.0, 1.0, 0.0, -1.0]]).repeat(draws, 1).cuda()
+    hip.sample(logits, torch.ones(draws).cuda(), torch.full((draws,), 3, dtype=torch.int32).cuda(),
+               torch.full((draws,), 0.7).cuda(), seeds, out)
+    freq = torch.bincount(out.long().cpu(), minlength=5).float() / draws
+    p3 = torch.softmax(torch.tensor([3.0, 2.0, 1.0]), -1)   # 0.665, 0.245, 0.090: nucleus 0.7 keeps two
+    expect = torch.tensor([p3[0], p3[1], 0, 0, 0]) / (p3[0] + p3[1])
+    assert (freq - expect).abs().max() < 0.015

@@ -1,0 +1,188 @@
+"""Plain tensor-library twins of the HIP kernels, with the kernels' interface and data layout.
+
+Two uses, both in tests only: each kernel is checked against its twin on the GPU, and the
+engine's host logic (cache, batches, scheduler, replay) is exercised on the CPU by handing it
+this object instead of the HIP kernels.  Arithmetic is float32 with the kernels' rounding points
+(``_r`` rounds through the storage dtype).
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+
+def _r(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    return x.to(dtype).float()
+
+
+class TwinWorkspace:
+    def __init__(self, *args, **kwargs):
+        pass
+
+
+class TwinKernels:
+    libraries = ()
+
+    # ------------------------------------------------------------------ embedding / norms
+    def embedding(self, ids, table, out):
+        out.copy_(table[ids.long()])
+
+    def rms_norm(self, x, weight, eps, out, residual=None, rows=None, write_residual=True):
+        z = x.float()
+        if residual is not None:
+            z = z + residual.float()
+        if rows is not None:
+            z = z[rows.long()]
+        elif residual is not None and write_residual:
+            residual.copy_(z.to(residual.dtype))
+        y = z * torch.rsqrt(z.square().mean(-1, keepdim=True) + eps) * weight.float()
+        out.copy_(y.to(out.dtype))
+
+    # ------------------------------------------------------------------ attention inputs
+    def qk_norm_rope_store(self, qkv, positions, cos_sin, q_weight, k_weight, eps, heads, kv_heads,
+                           head_dim, rotary_dim, cache=None, slots=None, page_size=0):
+        T = qkv.shape[0]
+        dt = qkv.dtype
+        qw, kw = heads * head_dim, kv_heads * head_dim
+        q = qkv[:, :qw].float()
+        k = qkv[:, qw:qw + kw].float()
+        v = qkv[:, qw + kw:]
+        if q_weight is not None:
+            def flat(x, w):
+                inv = torch.rsqrt(x.square().sum(-1, keepdim=True) / x.shape[-1] + eps)
+                return _r(_r(x * inv, dt) * _r(w.float(), dt), dt)
+            q, k = flat(q, q_weight), flat(k, k_weight)
+        if rotary_dim:
+            half = rotary_dim // 2
+            cs = cos_sin[positions.long()]
+            cos, sin = cs[:, None, :half], cs[:, None, half:]
+
+            def rot(x, n):
+                x = x.view(T, n, head_dim)
+                x1, x2 = x[..., :half], x[..., half:rotary_dim]
+                return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., rotary_dim:]), -1).reshape(T, -1)
+            q, k = rot(q, heads), rot(k, kv_heads)
+        qkv[:, :qw] = q.to(dt)
+        qkv[:, qw:qw + kw] = k.to(dt)
+        if cache is not None:
+            keep = slots >= 0
+            s = slots[keep].long()
+            page, off = s // page_size, s % page_size
+            cache[page, 0, :, off, :] = qkv[keep, qw:qw + kw].view(-1, kv_heads, head_dim)
+            cache[page, 1, :, off, :] = v[keep].reshape(-1, kv_heads, head_dim)
+
+    def paged_attention(self, q, cache, meta, out, scale, window=0):
+        T, H, D = q.shape
+        Hkv, ps = cache.shape[2], cache.shape[3]
+        group = H // Hkv
+        dt = q.dtype
+        for t in range(T):
+            pos = int(meta.positions[t])
+            row = int(meta.token_row[t])
+            first = max(0, pos - window + 1) if window else 0
+            n = torch.arange(first, pos + 1, device=q.device)
+            pages = meta.block_table[row, (n // ps)].long()
+            keys = cache[pages, 0, :, n % ps, :].float()      # [n, Hkv, D]
+            vals = cache[pages, 1, :, n % ps, :].float()
+            qt = q[t].float().view(Hkv, group, D)
+            scores = torch.einsum("hgd,nhd->hgn", qt, keys) * scale
+            m = scores.max(-1, keepdim=True).values
+            p = torch.exp(scores - m)
+            o = torch.einsum("hgn,nhd->hgd", _r(p, dt), vals) / p.sum(-1, keepdim=True)
+            out[t] = o.reshape(-1).to(dt)
+
+    # ------------------------------------------------------------------ mixture of experts
+    def router_topk(self, logits, bias, top_k, ids, weights, scoring="sigmoid", normalize=True, scaling=1.0):
+        s = torch.sigmoid(logits) if scoring == "sigmoid" else torch.softmax(logits, -1)
+        sel = s + bias if bias is not None else s.clone()
+        sel = torch.where(torch.isnan(sel), torch.full_like(sel, float("inf")), sel)
+        T, E = sel.shape
+        # the k largest, lowest index first among equals; then the reference's output order
+        order = torch.argsort(sel, dim=-1, descending=True, stable=True)[:, :top_k]
+        thr = sel.gather(1, order[:, -1:])
+        chosen = torch.zeros_like(sel, dtype=torch.bool).scatter_(1, order, True)
+        greater = chosen & (sel > thr)
+        ties = chosen & ~greater
+        idx = torch.arange(E, device=sel.device).expand(T, E)
+        key = torch.where(greater, idx, torch.where(ties, idx + E, idx + 2 * E))
+        out_ids = torch.argsort(key, dim=-1, stable=True)[:, :top_k]
+        w = s.gather(1, out_ids)
+        if normalize:
+            w = w / w.sum(-1, keepdim=True)
+        ids.copy_(out_ids.to(torch.int32))
+        weights.copy_(w * scaling)
+
+    def moe_experts(self, x, w13, w2, ids, weights, out, ws=None):
+        dt = x.dtype
+        T, h = x.shape
+        E, two_i, _ = w13.shape
+        I = two_i // 2
+        K = ids.shape[1]
+        slot_out = torch.zeros(T, K, h, dtype=torch.float32, device=x.device)
+        xf = x.float()
+        for e in range(E):
+            tok, slot = torch.where(ids == e)
+            if tok.numel() == 0:
+                continue
+            gu = xf[tok] @ w13[e].float().T
+            gate, up = _r(gu[:, :I], dt), _r(gu[:, I:], dt)
+            act = _r(_r(gate * torch.sigmoid(gate), dt) * up, dt)
+            y = (act @ w2[e].float().T) * weights[tok, slot, None]
+            slot_out[tok, slot] = _r(y, dt)
+        out.copy_(slot_out.sum(1).to(dt))
+
+    def silu_mul(self, x, out):
+        dt = x.dtype
+        w = x.shape[1] // 2
+        gate, up = x[:, :w].float(), x[:, w:].float()
+        out.copy_((_r(gate * torch.sigmoid(gate), dt) * up).to(dt))
+
+    # ------------------------------------------------------------------ sampling
+    @staticmethod
+    def uniform(seed: int, vocab: int) -> np.ndarray:
+        with np.errstate(over="ignore"):
+            i = np.arange(1, vocab + 1, dtype=np.uint64)
+            x = np.uint64(seed & (2**64 - 1)) + np.uint64(0x9E3779B97F4A7C15) * i
+            x ^= x >> np.uint64(30)
+            x *= np.uint64(0xBF58476D1CE4E5B9)
+            x ^= x >> np.uint64(27)
+            x *= np.uint64(0x94D049BB133111EB)
+            x ^= x >> np.uint64(31)
+        return ((x >> np.uint64(41)).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 8388608.0)
+
+    def sample(self, logits, temperature, top_k, top_p, seeds, out):
+        rows, vocab = logits.shape
+        for r in range(rows):
+            row = logits[r].float().cpu()
+            temp = float(temperature[r]) if temperature is not None else 0.0
+            if not temp > 1e-10:
+                out[r] = int(torch.argmax(row))
+                continue
+            l = row * np.float32(1.0 / np.float32(temp))
+            keep = torch.ones(vocab, dtype=torch.bool)
+            k = int(top_k[r]) if top_k is not None else 0
+            if 0 < k < vocab:
+                kth = torch.topk(l, k).values[-1]
+                keep &= l >= kth
+            p = float(top_p[r]) if top_p is not None else 1.0
+            if p < 1.0:
+                e = torch.where(keep, torch.exp(l - l.max()), torch.zeros_like(l))
+                order = torch.argsort(l, descending=True, stable=True)
+                sorted_e = e[order]
+                # mass of strictly more probable tokens
+                cum = torch.cumsum(sorted_e, 0) - sorted_e
+                sl = l[order]
+                first_of_value = torch.ones_like(sl, dtype=torch.bool)
+                first_of_value[1:] = sl[1:] != sl[:-1]
+                start = torch.cummax(torch.where(first_of_value, torch.arange(vocab), torch.zeros(vocab, dtype=torch.long)), 0).values
+                strictly_more = cum[start]
+                ok = strictly_more <= np.float32(p) * e.sum()
+                keep_sorted = ok
+                keep2 = torch.zeros(vocab, dtype=torch.bool)
+                keep2[order] = keep_sorted
+                keep &= keep2
+            seed = int(seeds[r]) if seeds is not None else 0
+            u = torch.from_numpy(self.uniform(seed, vocab))
+            noisy = l - torch.log(-torch.log(u))
+            noisy[~keep] = float("-inf")
+            out[r] = int(torch.argmax(noisy))
