@@ -1,0 +1,168 @@
+"""The batch of one step as the parts see it.
+
+A step is a list of items ``(row, tokens, want)``: a request's next tokens (a portion of its
+prompt, or one decoded token) and the places among them whose logits are asked for.  The builder
+reserves cache room for all items at once, packs every integer the kernels need into one host
+buffer and sends it with a single copy.  Nothing here is global: the ``ForwardBatch`` object is
+passed down to the parts (the reference passes a module-level context, utils/context.py:26-41,
+and builds prefill and decode batches apart, engine/cache_manager/standard.py:2065-2206).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..parts.base import StepScratch
+
+
+@dataclass
+class StepItem:
+    row: int
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)     # indices into ``tokens``
+
+
+@dataclass
+class GroupMeta:
+    """Per cache group: where every token of the step lives and how to find its request's pages."""
+    block_table: torch.Tensor      # int32 [items, pages]: compact table of the step's requests
+    token_row: torch.Tensor        # int32 [T] index of the token's item = row of block_table
+    positions: torch.Tensor        # int32 [T]
+    slots: torch.Tensor            # int32 [T] page * page_size + offset of the token's own key
+    page_size: int
+    # host copies for kernels that build a work list
+    item_q_start: np.ndarray = None
+    item_q_len: np.ndarray = None
+    item_ctx_len: np.ndarray = None
+    item_meta: torch.Tensor = None     # int32 [3, items] on the device: q_start, q_len, ctx_len
+    max_ctx_len: int = 0
+    max_q_len: int = 0
+
+
+class ForwardBatch:
+    def __init__(self, kernels, cache: CacheManager, dtype: torch.dtype, device, scratch: StepScratch):
+        self.kernels = kernels
+        self.cache = cache
+        self.dtype = dtype
+        self.device = device
+        self.scratch = scratch
+        self.num_tokens = 0
+        self.num_items = 0
+        self.token_ids = None          # int32 [T]
+        self.positions = None          # int32 [T]
+        self.token_item = None         # int32 [T]
+        self.item_rows = None          # int32 [items]: the cache row (state slot) of every item
+        self.item_rows_host = None
+        self.want_index = None         # int32 [wanted] token indices whose logits are returned
+        self.groups: dict[int, GroupMeta] = {}
+        self.taps: dict | None = None
+
+    # views the mixers use ---------------------------------------------------------------
+    def kv_view(self, position: int):
+        """(layer tensor, GroupMeta) of the schedule position that owns the cache."""
+        return self.cache.kv_layer(position), self.groups[self.cache.group_of_position[position]]
+
+    def state_view(self, position: int) -> dict[str, torch.Tensor]:
+        """name -> [rows, ...] state tensors of the position; index them with ``item_rows``."""
+        return self.cache.state[position]
+
+    def buffer(self, key: str, shape, dtype=None) -> torch.Tensor:
+        """A reusable scratch tensor whose leading dims are cut to ``shape``."""
+        shape = tuple(int(s) for s in shape)
+        dtype = dtype or self.dtype
+        # one buffer per (purpose, row shape): only the leading dim is ever cut, so views stay dense
+        full = self.scratch.get(f"{key}{shape[1:]}", shape, dtype, self.device)
+        return full if full.shape[0] == shape[0] else full.narrow(0, 0, shape[0])
+
+
+class BatchBuilder:
+    """Turns step items into a ``ForwardBatch``: cache reservation + one packed host-to-device copy."""
+
+    def __init__(self, kernels, cache: CacheManager, dtype, device, vocab_size: int):
+        self.kernels, self.cache, self.dtype, self.device = kernels, cache, dtype, torch.device(device)
+        self.vocab_size = vocab_size
+        self.scratch = StepScratch()
+        self._host = None
+        self._dev = None
+        self._copied = None            # event after the last host-to-device copy
+
+    def _buffers(self, n: int):
+        if self._host is None or self._host.numel() < n:
+            size = max(n, 4096) * 2
+            pin = self.device.type == "cuda"
+            self._host = torch.empty(size, dtype=torch.int32, pin_memory=pin)
+            self._dev = torch.empty(size, dtype=torch.int32, device=self.device)
+        return self._host, self._dev
+
+    def build(self, items: list[StepItem]) -> ForwardBatch:
+        if not items:
+            raise ValueError("a step needs at least one item")
+        cache = self.cache
+        lengths = [len(it.tokens) for it in items]
+        for it in items:
+            if not it.tokens:
+                raise ValueError("an item without tokens")
+            bad = [t for t in it.tokens if not 0 <= t < self.vocab_size]
+            if bad:
+                raise ValueError(f"token id {bad[0]} is outside the vocabulary [0, {self.vocab_size})")
+            if any(not 0 <= w < len(it.tokens) for w in it.want):
+                raise ValueError("a wanted place lies outside the item's tokens")
+        starts = [int(cache.row_len[it.row]) for it in items]
+        allocation = cache.append([(it.row, n) for it, n in zip(items, lengths)])   # all or nothing
+
+        T, B = sum(lengths), len(items)
+        q_start = np.zeros(B, dtype=np.int32)
+        q_start[1:] = np.cumsum(lengths[:-1])
+        q_len = np.asarray(lengths, dtype=np.int32)
+        ctx_len = np.asarray([s + n for s, n in zip(starts, lengths)], dtype=np.int32)
+        token_ids = np.concatenate([np.asarray(it.tokens, dtype=np.int32) for it in items])
+        positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, lengths)])
+        token_item = np.repeat(np.arange(B, dtype=np.int32), lengths)
+        want = np.asarray([q_start[i] + w for i, it in enumerate(items) for w in it.want], dtype=np.int32)
+        rows = np.asarray([it.row for it in items], dtype=np.int32)
+
+        tables = {}
+        for group in cache.groups:
+            width = max(1, -(-int(ctx_len.max()) // cache.page_size))
+            tables[group.index] = np.ascontiguousarray(group.table[rows, :width])
+
+        parts = [token_ids, positions, token_item, rows, q_start, q_len, ctx_len, want]
+        for group in cache.groups:
+            parts += [allocation.slots[group.index], tables[group.index].reshape(-1)]
+        total = sum(p.size for p in parts)
+        if self._copied is not None:
+            self._copied.synchronize()  # the last step's copy has left the pinned buffer
+        host, dev = self._buffers(total)
+        host_np = host.numpy()
+        offsets, cursor = [], 0
+        for p in parts:
+            host_np[cursor:cursor + p.size] = p.reshape(-1)
+            offsets.append(cursor)
+            cursor += p.size
+        dev[:total].copy_(host[:total], non_blocking=True)
+        if self.device.type == "cuda":
+            self._copied = torch.cuda.Event()
+            self._copied.record()
+
+        def view(i, shape=None):
+            v = dev[offsets[i]:offsets[i] + parts[i].size]
+            return v if shape is None else v.view(shape)
+
+        fb = ForwardBatch(self.kernels, cache, self.dtype, self.device, self.scratch)
+        fb.num_tokens, fb.num_items = T, B
+        fb.token_ids, fb.positions, fb.token_item = view(0), view(1), view(2)
+        fb.item_rows, fb.item_rows_host = view(3), rows
+        fb.want_index = view(7)
+        # q_start, q_len, ctx_len lie next to each other: one [3, items] device view
+        item_meta = dev[offsets[4]:offsets[4] + 3 * B].view(3, B)
+        for gi, group in enumerate(cache.groups):
+            fb.groups[group.index] = GroupMeta(
+                block_table=view(8 + 2 * gi + 1, tables[group.index].shape),
+                token_row=fb.token_item, positions=fb.positions, slots=view(8 + 2 * gi),
+                page_size=cache.page_size, item_q_start=q_start, item_q_len=q_len,
+                item_ctx_len=ctx_len, item_meta=item_meta, max_ctx_len=int(ctx_len.max()),
+                max_q_len=int(q_len.max()))
+        return fb

@@ -1,0 +1,146 @@
+"""The model runner: model + cache manager + the one step function.
+
+``step(entries)`` takes a batch of (request, its next tokens, wanted places): portions of prompts
+beside single decoded tokens, cut anywhere.  It runs exactly those tokens, as one batch, against
+the cache earlier steps left, and returns float32 logits at the wanted places.  Sampling is not
+done here.  (The reference's step is ``ModelRunner.run(seqs, is_prefill)``,
+engine/model_runner.py:2572-2660: prefill chunks *or* decode tokens, sampled inside.)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..config.registry import Architecture, read_config_json, resolve_architecture
+from ..parts import build_model
+from ..weights import loader as weight_loader
+from ..weights import random_weights
+from .batch import BatchBuilder, StepItem
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}") from None
+
+
+def require_true_float32() -> None:
+    """No reduced-precision matrix mode for float32 products of the BLAS library."""
+    torch.backends.cuda.matmul.allow_tf32 = False
+    torch.backends.cudnn.allow_tf32 = False
+    torch.set_float32_matmul_precision("highest")
+
+
+@dataclass
+class StepEntry:
+    request_id: object
+    tokens: list[int]
+    want: list[int] = field(default_factory=list)
+
+
+class ModelRunner:
+    def __init__(self, arch: Architecture, cfg, params_factory, *, dtype, device="cuda", kv_page_size=64,
+                 num_kvcache_tokens: int, max_num_seqs: int = 8, max_model_len: int | None = None,
+                 mlp_chunk_size: int = 16384, kernels=None):
+        self.arch, self.model_config = arch, cfg
+        self.dtype = resolve_dtype(dtype)
+        self.device = torch.device(device)
+        require_true_float32()
+        if kernels is None:
+            from ..kernels.hip_ops import HipKernels      # raises if there is no GPU or no library
+            kernels = HipKernels()
+        self.kernels = kernels
+        self.spec = arch.build_spec(cfg)
+        self.model = build_model(self.spec, chunk_tokens=mlp_chunk_size)
+        if getattr(kernels, "libraries", None):
+            from ..kernels import library
+            library.ensure_built(sorted(self.model.all_kernel_libraries()))
+        decls = self.model.all_param_decls()
+        self.params = params_factory(decls, self.dtype, self.device)
+        self.model.bind_all(self.params)
+
+        self.max_model_len = int(max_model_len or self.spec.max_position)
+        if self.max_model_len > self.spec.max_position:
+            raise ValueError(f"max_model_len {self.max_model_len} exceeds the model's "
+                             f"max_position_embeddings {self.spec.max_position}")
+        self.kv_page_size = int(kv_page_size)
+        num_pages = max(1, int(num_kvcache_tokens) // self.kv_page_size)
+        self.cache = CacheManager(self.model.cache_requests(), max_rows=max_num_seqs,
+                                  max_model_len=self.max_model_len, page_size=self.kv_page_size,
+                                  num_pages=num_pages, dtype=self.dtype, device=self.device)
+        self.builder = BatchBuilder(kernels, self.cache, self.dtype, self.device, self.spec.vocab_size)
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_folder(cls, folder: str, **kwargs) -> "ModelRunner":
+        raw = read_config_json(folder)
+        arch = resolve_architecture(raw)
+        cfg = arch.parse_config(raw)
+
+        def factory(decls, dtype, device):
+            return weight_loader.load_parameters(folder, arch, cfg, decls, dtype, device)
+        return cls(arch, cfg, factory, **kwargs)
+
+    @classmethod
+    def from_random(cls, raw_config: dict, seed: int = 0, options: dict | None = None,
+                    on_device: bool = False, **kwargs) -> "ModelRunner":
+        arch = resolve_architecture(raw_config)
+        cfg = arch.parse_config(raw_config)
+
+        def factory(decls, dtype, device):
+            dtypes = random_weights.random_parameter_dtypes(arch, cfg, decls, dtype)
+            params = weight_loader.allocate_parameters(decls, dtypes, device)
+            random_weights.fill_random(params, arch, cfg, decls, seed, options, on_device=on_device)
+            return params
+        return cls(arch, cfg, factory, **kwargs)
+
+    # ------------------------------------------------------------------ requests
+    def admit(self, request_id) -> int:
+        return self.cache.admit(request_id)
+
+    def release(self, request_id) -> None:
+        self.cache.free(request_id)
+
+    def can_step(self, entries) -> bool:
+        """Whether the cache has room for these (request_id, new token count) pairs; requests
+        not yet admitted are counted with an empty row."""
+        need = {g.index: 0 for g in self.cache.groups}
+        new_rows = 0
+        for request_id, n in entries:
+            if self.cache.has_row(request_id):
+                for gi, pages in self.cache.pages_needed(self.cache.row_of(request_id), n).items():
+                    need[gi] += pages
+            else:
+                new_rows += 1
+                for gi in need:
+                    need[gi] += self.cache.pages_for_tokens(n)
+        free = self.cache.free_pages()
+        return new_rows <= self.cache.num_free_rows and all(need[g] <= free[g] for g in need)
+
+    # ------------------------------------------------------------------ the step
+    @torch.no_grad()
+    def step(self, entries: list[StepEntry], taps: dict | None = None) -> torch.Tensor:
+        """Run the entries' tokens as one batch; float32 logits ``[wanted, vocab]`` in the order
+        of the entries and of their ``want`` lists.  A request that holds no row yet is admitted.
+        If the cache cannot take the step, ``OutOfPages`` is raised and nothing has changed."""
+        admitted = []
+        try:
+            items = []
+            for e in entries:
+                if not self.cache.has_row(e.request_id):
+                    self.cache.admit(e.request_id)
+                    admitted.append(e.request_id)
+                items.append(StepItem(self.cache.row_of(e.request_id), list(e.tokens), list(e.want)))
+            fb = self.builder.build(items)
+        except Exception:
+            for request_id in admitted:
+                self.cache.free(request_id)
+            raise
+        fb.taps = taps
+        return self.model.forward(fb)

@@ -1,0 +1,63 @@
+"""Causal grouped-query attention over the paged cache.
+
+Order inside the mixer, as in the reference (models/minimax_m2.py:334-359): merged q/k/v
+projection -> flat QK RMSNorm over the whole q row and the whole k row (optional) -> rotation of
+the leading rotary dims of every head -> k (normed, rotated) and v written to this step's slots
+-> attention of the step's queries over everything the request has cached, its own tokens
+included -> output projection.  Norm, rotation and the cache write are one kernel.
+"""
+from __future__ import annotations
+
+from ..config.specs import AttentionSpec
+from .base import MIXERS, POSITIONS, PagedKVRequest, ParamDecl, Part
+from .linear import linear
+
+
+class GQAAttention(Part):
+    kernel_libraries = ("rope_kv", "attention_generic")
+
+    def __init__(self, spec: AttentionSpec, hidden_size: int):
+        if spec.num_kv_heads <= 0 or spec.num_heads % spec.num_kv_heads:
+            raise ValueError(f"{spec.num_heads} query heads do not divide into {spec.num_kv_heads} kv heads")
+        if spec.head_dim % 16:
+            raise ValueError(f"head_dim must be a multiple of 16, got {spec.head_dim}")
+        if spec.qk_norm not in ("none", "flat"):
+            raise ValueError(f"qk_norm {spec.qk_norm!r} is unknown (none, flat)")
+        self.spec = spec
+        self.hidden_size = int(hidden_size)
+        self.q_width = spec.num_heads * spec.head_dim
+        self.kv_width = spec.num_kv_heads * spec.head_dim
+        self.position = POSITIONS.build(spec.position, head_dim=spec.head_dim)
+
+    def param_decls(self):
+        decls = {"qkv": ParamDecl((self.q_width + 2 * self.kv_width, self.hidden_size)),
+                 "o": ParamDecl((self.hidden_size, self.q_width))}
+        if self.spec.qk_norm == "flat":
+            decls["q_norm"] = ParamDecl((self.q_width,))
+            decls["k_norm"] = ParamDecl((self.kv_width,))
+        return decls
+
+    def bind(self, params):
+        super().bind(params)
+        self.position.prepare(params["qkv"].device)
+
+    def cache_request(self):
+        return PagedKVRequest(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
+
+    def forward(self, fb, x, cache_position: int, write_cache: bool = True):
+        s, p, T = self.spec, self.params, x.shape[0]
+        cache, meta = fb.kv_view(cache_position)
+        qkv = linear(x, p["qkv"], out=fb.buffer("attn.qkv", (T, self.q_width + 2 * self.kv_width)))
+        fb.kernels.qk_norm_rope_store(
+            qkv, meta.positions, self.position.table, p.get("q_norm"), p.get("k_norm"), s.qk_norm_eps,
+            s.num_heads, s.num_kv_heads, s.head_dim, self.position.rotary_dim,
+            cache if write_cache else None, meta.slots if write_cache else None, meta.page_size)
+        attended = fb.buffer("attn.out", (T, self.q_width))
+        q = qkv[:, :self.q_width].view(T, s.num_heads, s.head_dim)
+        fb.kernels.paged_attention(q, cache, meta, attended, s.scale, s.window or 0)
+        if fb.taps is not None:
+            fb.taps.setdefault("attention_inputs", []).append(qkv.clone())
+        return linear(attended, p["o"], out=fb.buffer("attn.proj", (T, self.hidden_size)))
+
+
+MIXERS.register("gqa_attention", lambda spec, hidden_size: GQAAttention(spec, hidden_size))

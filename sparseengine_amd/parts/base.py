@@ -77,8 +77,9 @@ class Part:
 class PartRegistry:
     """kind -> factory(spec, **context).  One instance per family of parts."""
 
-    def __init__(self, family: str):
+    def __init__(self, family: str, attribute: str = "kind"):
         self.family = family
+        self.attribute = attribute      # the field of a spec that names its kind
         self._factories: dict[str, Callable] = {}
 
     def register(self, kind: str, factory: Callable | None = None):
@@ -88,7 +89,7 @@ class PartRegistry:
         return add(factory) if factory is not None else add
 
     def build(self, spec, **context):
-        kind = getattr(spec, "kind", None)
+        kind = getattr(spec, self.attribute, None)
         if kind not in self._factories:
             raise KeyError(f"no {self.family} registered for kind {kind!r}; known: "
                            f"{sorted(self._factories)}")
@@ -102,7 +103,7 @@ MIXERS = PartRegistry("mixer")
 FEED_FORWARDS = PartRegistry("feed-forward")
 NORMS = PartRegistry("norm")
 POSITIONS = PartRegistry("position encoding")
-BLOCKS = PartRegistry("block")
+BLOCKS = PartRegistry("block", attribute="block")
 
 
 @dataclass
@@ -112,7 +113,7 @@ class StepScratch:
 
     def get(self, key: str, shape: tuple[int, ...], dtype: torch.dtype, device) -> torch.Tensor:
         t = self.tensors.get(key)
-        if t is None or t.dtype != dtype or any(a < b for a, b in zip(t.shape, shape)) or t.dim() != len(shape):
+        if t is None or t.dtype != dtype or t.shape[1:] != tuple(shape[1:]) or t.shape[0] < shape[0]:
             t = torch.empty(shape, dtype=dtype, device=device)
             self.tensors[key] = t
         return t

@@ -1,0 +1,103 @@
+"""Feed-forward parts: routed SwiGLU experts and a dense gated MLP.
+
+Routed experts, as the reference computes them (models/minimax_m2.py:140-172,212-269;
+kernels/triton/moe_biased_sigmoid.py:202-238; kernels/triton/moe.py:1311-1440): router logits
+in float32 from float32 weights; score = sigmoid (or softmax); experts picked by score + bias,
+weights are the unbiased scores of the picked experts, renormalised; each (token, slot) runs
+``W2_e(silu(W1_e x) * W3_e x)`` times its weight; the slots of a token are summed in float.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import DenseMLPSpec, MoESpec
+from .base import FEED_FORWARDS, ParamDecl, Part
+from .linear import linear
+
+
+class RoutedExperts(Part):
+    kernel_libraries = ("moe",)
+
+    def __init__(self, spec: MoESpec, hidden_size: int, chunk_tokens: int = 16384):
+        if not 1 <= spec.top_k <= spec.num_experts:
+            raise ValueError(f"top_k must be in [1, num_experts={spec.num_experts}], got {spec.top_k}")
+        if spec.activation != "silu":
+            raise NotImplementedError(f"expert activation {spec.activation!r} is not supported (silu)")
+        if spec.scoring not in ("sigmoid", "softmax"):
+            raise NotImplementedError(f"router scoring {spec.scoring!r} is not supported (sigmoid, softmax)")
+        self.spec = spec
+        self.hidden_size = int(hidden_size)
+        self.chunk_tokens = int(chunk_tokens)
+        self._workspace = None
+
+    def param_decls(self):
+        s = self.spec
+        decls = {"router": ParamDecl((s.num_experts, self.hidden_size), "float32"),
+                 "w13": ParamDecl((s.num_experts, 2 * s.intermediate_size, self.hidden_size)),
+                 "w2": ParamDecl((s.num_experts, self.hidden_size, s.intermediate_size))}
+        if s.selection_bias:
+            decls["router_bias"] = ParamDecl((s.num_experts,), "float32")
+        return decls
+
+    def _workspace_for(self, fb, tokens: int, dtype):
+        s = self.spec
+        ws = fb.scratch.tensors.get("moe.workspace")
+        if ws is None or not ws.fits(tokens, s.top_k, s.num_experts, self.hidden_size, s.intermediate_size, dtype):
+            from ..kernels.hip_ops import MoeWorkspace
+            factory = getattr(fb.kernels, "make_moe_workspace", None) or MoeWorkspace
+            ws = factory(max(tokens, 1), s.top_k, s.num_experts, self.hidden_size, s.intermediate_size,
+                         dtype, fb.device)
+            fb.scratch.tensors["moe.workspace"] = ws
+        return ws
+
+    def forward(self, fb, x):
+        s, p, T = self.spec, self.params, x.shape[0]
+        out = fb.buffer("ffn.out", (T, self.hidden_size))
+        for start in range(0, T, self.chunk_tokens):
+            stop = min(T, start + self.chunk_tokens)
+            self._forward_chunk(fb, x[start:stop], out[start:stop])
+        return out
+
+    def _forward_chunk(self, fb, x, out):
+        s, p, T = self.spec, self.params, x.shape[0]
+        logits = torch.mm(x.float(), p["router"].t(), out=fb.buffer("moe.logits", (T, s.num_experts), torch.float32))
+        ids = fb.buffer("moe.ids", (T, s.top_k), torch.int32)
+        weights = fb.buffer("moe.weights", (T, s.top_k), torch.float32)
+        fb.kernels.router_topk(logits, p.get("router_bias"), s.top_k, ids, weights, scoring=s.scoring,
+                               normalize=s.norm_topk_prob, scaling=s.routed_scaling_factor)
+        if fb.taps is not None:
+            fb.taps.setdefault("router", []).append((ids.clone(), weights.clone()))
+        w13, w2 = p["w13"], p["w2"]
+        if w13.dtype == x.dtype:
+            fb.kernels.moe_experts(x, w13, w2, ids, weights, out, self._workspace_for(fb, T, x.dtype))
+        else:   # expert weights kept in float32 under a bfloat16 engine
+            x32 = x.float()
+            out32 = torch.empty_like(x32)
+            fb.kernels.moe_experts(x32, w13, w2, ids, weights, out32, self._workspace_for(fb, T, x32.dtype))
+            out.copy_(out32)
+
+
+class DenseMLP(Part):
+    """``down(silu(gate x) * up x)``; ``gate_up`` holds the gate rows, then the up rows."""
+    kernel_libraries = ("moe",)
+
+    def __init__(self, spec: DenseMLPSpec, hidden_size: int, chunk_tokens: int = 16384):
+        if spec.activation != "silu":
+            raise NotImplementedError(f"activation {spec.activation!r} is not supported (silu)")
+        self.spec = spec
+        self.hidden_size = int(hidden_size)
+
+    def param_decls(self):
+        i = self.spec.intermediate_size
+        return {"gate_up": ParamDecl((2 * i, self.hidden_size)), "down": ParamDecl((self.hidden_size, i))}
+
+    def forward(self, fb, x):
+        T, i = x.shape[0], self.spec.intermediate_size
+        gate_up = linear(x, self.params["gate_up"], out=fb.buffer("mlp.gate_up", (T, 2 * i)))
+        act = fb.buffer("mlp.act", (T, i))
+        fb.kernels.silu_mul(gate_up, act)
+        return linear(act, self.params["down"], out=fb.buffer("ffn.out", (T, self.hidden_size)))
+
+
+FEED_FORWARDS.register("moe", lambda spec, hidden_size, chunk_tokens=16384: RoutedExperts(spec, hidden_size, chunk_tokens))
+FEED_FORWARDS.register("dense_mlp", lambda spec, hidden_size, chunk_tokens=16384: DenseMLP(spec, hidden_size, chunk_tokens))

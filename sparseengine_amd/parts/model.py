@@ -1,0 +1,83 @@
+"""A decoder put together from a ``ModelSpec``: embedding, the layers in schedule order, final
+norm and output head.  It knows parts and specs only, no architecture.
+
+The step returns logits only for the wanted token places: the final norm and the head run on
+those rows alone (the reference keeps the last row of every request, layers/embed_head.py:75-84).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import ModelSpec
+from .base import BLOCKS, NORMS, ParamDecl, Part
+from .linear import linear
+
+
+class Embedding(Part):
+    kernel_libraries = ("norm",)
+
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+
+    def param_decls(self):
+        return {"weight": ParamDecl((self.vocab_size, self.hidden_size))}
+
+
+class OutputHead(Part):
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+
+    def param_decls(self):
+        return {"weight": ParamDecl((self.vocab_size, self.hidden_size))}
+
+
+class DecoderModel(Part):
+    def __init__(self, spec: ModelSpec, chunk_tokens: int = 16384):
+        self.spec = spec
+        self.embed = Embedding(spec.vocab_size, spec.hidden_size)
+        self.layers = [BLOCKS.build(layer, hidden_size=spec.hidden_size, chunk_tokens=chunk_tokens)
+                       for layer in spec.layers]
+        self.final_norm = NORMS.build(spec.final_norm, hidden_size=spec.hidden_size)
+        self.head = None if spec.tie_word_embeddings else OutputHead(spec.vocab_size, spec.hidden_size)
+
+    def children(self):
+        parts = {"embed": self.embed, "final_norm": self.final_norm}
+        parts.update({f"layers.{i}": layer for i, layer in enumerate(self.layers)})
+        if self.head is not None:
+            parts["head"] = self.head
+        return parts
+
+    def cache_requests(self) -> dict[int, object]:
+        """schedule position -> what its mixer keeps (positions reading another cache: nothing)."""
+        out = {}
+        for position, entry in enumerate(self.spec.schedule):
+            if entry.cache_from is None:
+                request = self.layers[entry.layer].cache_request()
+                if request is not None:
+                    out[position] = request
+        return out
+
+    def forward(self, fb) -> torch.Tensor:
+        """float32 logits ``[wanted, vocab]`` of the step."""
+        spec = self.spec
+        x = fb.buffer("model.hidden", (fb.num_tokens, spec.hidden_size))
+        fb.kernels.embedding(fb.token_ids, self.embed.params["weight"], x)
+        residual = None
+        for position, entry in enumerate(spec.schedule):
+            own = entry.cache_from is None
+            x, residual = self.layers[entry.layer].forward(
+                fb, x, residual, position if own else entry.cache_from, own)
+            if fb.taps is not None:
+                fb.taps.setdefault("layer_out", []).append((x.float() + residual.float()))
+        wanted = fb.want_index.numel()
+        if wanted == 0:
+            return torch.empty(0, spec.vocab_size, dtype=torch.float32, device=fb.device)
+        last = fb.buffer("model.wanted", (wanted, spec.hidden_size))
+        self.final_norm.forward_rows(fb, x, residual, fb.want_index, last)
+        weight = (self.head or self.embed).params["weight"]
+        logits = linear(last, weight, out=fb.buffer("model.logits", (wanted, spec.vocab_size)))
+        return logits.to(torch.float32, copy=True)      # the caller's own tensor, not the scratch buffer
+
+
+def build_model(spec: ModelSpec, chunk_tokens: int = 16384) -> DecoderModel:
+    return DecoderModel(spec, chunk_tokens)

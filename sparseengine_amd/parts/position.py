@@ -1,0 +1,101 @@
+"""Position encodings.  A position part owns its table and says how a head is rotated; the
+attention mixer hands table and sizes to the fused kernel.
+
+Rotary: ``theta_d = base^(-2d/R)`` for ``d in [0, R/2)``, table ``[max_position, R]`` = cos half then
+sin half in float32, built on the host exactly as the reference does
+(layers/rotary_embedding.py:15-24,217-222); scaled variants follow :26-101.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..config.specs import NoPositionSpec, RotarySpec
+from .base import POSITIONS, Part
+
+
+def rotary_inverse_frequencies(rotary_dim: int, theta: float, scaling: dict | None):
+    """(inv_freq float32 [R/2], factor that multiplies cos and sin)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    if not scaling:
+        return inv_freq, 1.0
+    kind = str(scaling.get("rope_type", scaling.get("type", "default"))).lower()
+    if kind == "default":
+        return inv_freq, 1.0
+    factor = float(scaling["factor"])
+    if kind == "linear":
+        return inv_freq / factor, 1.0
+    if kind == "llama3":
+        # long wavelengths are slowed by `factor`, short ones kept, the band between blended
+        original = float(scaling["original_max_position_embeddings"])
+        low, high = float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
+        wavelength = 2 * math.pi / inv_freq
+        slowed = torch.where(wavelength > original / low, inv_freq / factor, inv_freq)
+        blend = (original / wavelength - low) / (high - low)
+        blended = (1 - blend) * slowed / factor + blend * slowed
+        in_band = (wavelength >= original / high) & (wavelength <= original / low)
+        return torch.where(in_band, blended, slowed), 1.0
+    if kind == "yarn":
+        original = float(scaling["original_max_position_embeddings"])
+        beta_fast, beta_slow = float(scaling.get("beta_fast", 32.0)), float(scaling.get("beta_slow", 1.0))
+
+        def dim_of_rotations(rotations: float) -> float:
+            return rotary_dim * math.log(original / (rotations * 2 * math.pi)) / (2 * math.log(theta))
+
+        low, high = dim_of_rotations(beta_fast), dim_of_rotations(beta_slow)
+        if bool(scaling.get("truncate", True)):
+            low, high = math.floor(low), math.ceil(high)
+        low, high = max(low, 0), min(high, rotary_dim - 1)
+        if low == high:
+            high += 0.001
+        ramp = torch.clamp((torch.arange(rotary_dim // 2, dtype=torch.float32) - low) / (high - low), 0, 1)
+        inv = inv_freq / factor * ramp + inv_freq * (1 - ramp)
+
+        def mscale(f: float, multiplier: float = 1.0) -> float:
+            return 1.0 if f <= 1.0 else 0.1 * multiplier * math.log(f) + 1.0
+
+        attention = scaling.get("attention_factor")
+        if attention is None:
+            m, m_all = scaling.get("mscale"), scaling.get("mscale_all_dim")
+            attention = mscale(factor, float(m)) / mscale(factor, float(m_all)) if m and m_all else mscale(factor)
+        return inv, float(attention)
+    raise NotImplementedError(f"rope scaling type {kind!r} is not supported "
+                              "(default, linear, llama3, yarn)")
+
+
+class RotaryPosition(Part):
+    """Rotation of the leading ``rotary_dim`` dims of each head, NeoX pairing ``(d, d + R/2)``."""
+
+    def __init__(self, spec: RotarySpec, head_dim: int):
+        if spec.rotary_dim % 2 or not 0 < spec.rotary_dim <= head_dim:
+            raise ValueError(f"rotary_dim must be even and in (0, head_dim={head_dim}], got {spec.rotary_dim}")
+        if spec.pairing != "neox":
+            raise NotImplementedError(f"rotary pairing {spec.pairing!r} is not supported (neox)")
+        if spec.max_position <= 0:
+            raise ValueError("a rotary encoding needs max_position > 0")
+        self.spec = spec
+        self.rotary_dim = spec.rotary_dim
+        self.table = None
+
+    def prepare(self, device) -> None:
+        spec = self.spec
+        inv_freq, factor = rotary_inverse_frequencies(spec.rotary_dim, spec.theta,
+                                                      dict(spec.scaling) if spec.scaling else None)
+        angles = torch.arange(spec.max_position, dtype=torch.float32)[:, None] * inv_freq[None, :]
+        self.table = torch.cat((angles.cos() * factor, angles.sin() * factor), dim=-1).contiguous().to(device)
+
+
+class NoPosition(Part):
+    rotary_dim = 0
+    table = None
+
+    def __init__(self, spec=None, head_dim: int = 0):
+        pass
+
+    def prepare(self, device) -> None:
+        pass
+
+
+POSITIONS.register("rotary", lambda spec, head_dim: RotaryPosition(spec, head_dim))
+POSITIONS.register("none", lambda spec, head_dim: NoPosition(spec, head_dim))

@@ -204,18 +204,29 @@ class PlainMiniMaxM2:
         o = causal_gqa_attention(q, k, v, c.head_dim ** -0.5)
         return o.reshape(u.shape[0], -1) @ self.w[f"model.layers.{layer}.self_attn.o_proj.weight"].T
 
-    def router(self, layer: int, m: torch.Tensor):
+    def router(self, layer: int, m: torch.Tensor, forced_ids=None, log=None):
+        """``forced_ids`` ([T, K], from another run) replaces the selection but not the weights:
+        used to compare a reduced-precision run whose near-ties fall the other way.  ``log[layer]``
+        receives the selection scores ``sigmoid(g) + bias`` so that such a choice can be checked."""
         c, p = self.cfg, f"model.layers.{layer}.block_sparse_moe."
         logits = m @ self.w[p + "gate.weight"].T
-        return biased_sigmoid_router(logits, self.w[p + "e_score_correction_bias"], c.num_experts_per_tok)
+        bias = self.w[p + "e_score_correction_bias"]
+        if log is not None:
+            log[layer] = torch.sigmoid(logits) + bias
+        if forced_ids is None:
+            return biased_sigmoid_router(logits, bias, c.num_experts_per_tok)
+        ids = torch.as_tensor(forced_ids, dtype=torch.long)
+        weights = torch.sigmoid(logits).gather(1, ids)
+        return weights / weights.sum(dim=-1, keepdim=True), ids
 
-    def moe(self, layer: int, m: torch.Tensor):
+    def moe(self, layer: int, m: torch.Tensor, forced_ids=None, log=None):
         c, p = self.cfg, f"model.layers.{layer}.block_sparse_moe.experts."
-        weights, ids = self.router(layer, m)
+        weights, ids = self.router(layer, m, forced_ids, log)
         stack = lambda proj: torch.stack([self.w[f"{p}{e}.{proj}.weight"] for e in range(c.num_local_experts)])
         return swiglu_experts(m, stack("w1"), stack("w3"), stack("w2"), ids, weights)
 
-    def hidden_states(self, token_ids, start_position: int = 0, taps: dict | None = None):
+    def hidden_states(self, token_ids, start_position: int = 0, taps: dict | None = None,
+                      forced_routing=None, routing_log=None):
         """Final-normed hidden state of every token.  Residual wiring:
         models/minimax_m2.py:381-397, models/qwen3.py:291-325."""
         c = self.cfg
@@ -231,16 +242,18 @@ class PlainMiniMaxM2:
                 u, residual = add_rms_norm(x, residual, self.w[p + "input_layernorm.weight"], c.rms_norm_eps)
             a = self.attention(layer, u, positions)
             m, residual = add_rms_norm(a, residual, self.w[p + "post_attention_layernorm.weight"], c.rms_norm_eps)
-            x = self.moe(layer, m)
+            x = self.moe(layer, m, None if forced_routing is None else forced_routing[layer], routing_log)
             if taps is not None:
                 taps[layer] = x + residual
         y, _ = add_rms_norm(x, residual, self.w["model.norm.weight"], c.rms_norm_eps)
         return y
 
-    def logits(self, token_ids, start_position: int = 0) -> torch.Tensor:
+    def logits(self, token_ids, start_position: int = 0, forced_routing=None, routing_log=None) -> torch.Tensor:
         """``[len, vocab]`` logits of a whole sequence (layers/embed_head.py:75-84: plain
         linear, no scale, no soft-cap)."""
-        return self.hidden_states(token_ids, start_position) @ self.w["lm_head.weight"].T
+        hidden = self.hidden_states(token_ids, start_position, forced_routing=forced_routing,
+                                    routing_log=routing_log)
+        return hidden @ self.w["lm_head.weight"].T
 
     def greedy(self, prompt, max_tokens: int) -> list[int]:
         tokens = list(prompt)

@@ -1,0 +1,153 @@
+"""The engine on the GPU against the plain implementation: every way of cutting and batching the
+same requests gives the same logits, in float32 and in bfloat16."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import traces
+from tests.helpers import CONFIGS, make_folder, random_tokens
+from tests.plain.minimax_m2 import PlainMiniMaxM2
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+LENGTHS = {"A": [5, 17, 31, 100, 64, 129, 250, 1, 48], "B": [1, 9, 40, 100, 200, 333, 65, 16, 500]}
+
+
+def bound(dtype, ref):
+    """Largest allowed |engine - plain|.  float32: a few units of float rounding of the largest
+    logit.  bfloat16: activations are rounded to 8 bits of mantissa about thirty times on the way
+    to a logit; 4 % of the largest logit covers that and no more."""
+    scale = float(np.abs(ref).max())
+    return 2e-5 * max(scale, 1.0) if dtype == "float32" else 0.04 * scale
+
+
+@pytest.fixture(scope="module", params=["A_loud", "B_loud", "A", "B"])
+def model(request, tmp_path_factory):
+    key = request.param
+    folder = make_folder(tmp_path_factory.mktemp("models"), key)
+    vocab = CONFIGS[key][0]["vocab_size"]
+    requests = {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate(LENGTHS[key[0]])}
+    plain = PlainMiniMaxM2(folder)
+    expected = {rid: plain.logits(toks).numpy() for rid, toks in requests.items()}
+    return folder, requests, expected, plain
+
+
+def run_records(folder, dtype, records, max_tokens, page_size):
+    """Replay in-process.  Returns (logits per step, router choices per request and layer)."""
+    from sparseengine_amd.engine.replay import replay_step
+    from sparseengine_amd.engine.runner import ModelRunner
+    runner = ModelRunner.from_folder(folder, dtype=dtype, kv_page_size=page_size,
+                                     num_kvcache_tokens=-(-max_tokens // 64) * 64, max_num_seqs=4)
+    out, routing = {}, {}
+    for rec in records:
+        taps = {}
+        logits = replay_step(runner, rec, None, taps=taps)
+        if logits is not None:
+            out[rec["step"]] = logits
+        cursor = 0
+        for e in rec["entries"]:
+            n = len(e["tokens"])
+            per_layer = routing.setdefault(e["id"], [[] for _ in taps["router"]])
+            for layer, (ids, _) in enumerate(taps["router"]):
+                per_layer[layer].append(ids[cursor:cursor + n].cpu())
+            cursor += n
+        runner.cache.check_invariants()
+    assert runner.cache.num_free_rows == 4 and all(
+        g.pool.free_count == g.pool.num_pages for g in runner.cache.groups), "pages or rows leaked"
+    return out, {rid: [torch.cat(chunks) for chunks in layers] for rid, layers in routing.items()}
+
+
+ROUTING_SLACK = 0.02    # in units of the selection score sigmoid(g) + bias, which lies in about [-1, 2]
+
+
+def compare(dtype, got, model, routing):
+    """float32: against the plain logits as they are.  bfloat16: rounding may tip a near-tie of the
+    router the other way, which changes a logit by far more than rounding does; so the plain
+    implementation is run with the engine's choice of experts, after checking that every such
+    choice is a top-k of the plain scores up to ``ROUTING_SLACK``."""
+    folder, requests, expected, plain = model
+    for rid, toks in requests.items():
+        ref = expected[rid]
+        if dtype == "bfloat16":
+            log = {}
+            ref = plain.logits(toks, forced_routing=[r.long() for r in routing[rid]], routing_log=log).numpy()
+            for layer, chosen in enumerate(routing[rid]):
+                scores = log[layer]
+                k = chosen.shape[1]
+                kth = torch.topk(scores, k, dim=-1).values[:, -1:]
+                picked = scores.gather(1, chosen.long())
+                assert (picked >= kth - ROUTING_SLACK).all(), f"{rid} layer {layer}: an expert far below the top-{k} was chosen"
+                assert sorted(set(map(int, chosen[0]))) == sorted(map(int, chosen[0])) and chosen.shape[0] == len(toks)
+        assert got[rid].shape == ref.shape, rid
+        err = np.abs(got[rid] - ref).max(axis=-1)
+        worst = int(err.argmax())
+        assert err[worst] <= bound(dtype, ref), (
+            f"request {rid} (length {len(ref)}): first position over the bound "
+            f"{int(np.argmax(err > bound(dtype, ref)))}, worst position {worst}, error {err[worst]:.3g}, "
+            f"bound {bound(dtype, ref):.3g}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_whole_requests(model, dtype, page_size):
+    folder, requests = model[:2]
+    records = traces.whole(requests)
+    logits, routing = run_records(folder, dtype, records, 512, page_size)
+    compare(dtype, traces.gather(records, logits), model, routing)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefill_then_last_32_one_by_one(model, dtype):
+    folder, requests = model[:2]
+    records = traces.prefill_then_decode(requests, tail=32)
+    logits, routing = run_records(folder, dtype, records, 512, 16)
+    compare(dtype, traces.gather(records, logits), model, routing)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [16, 32])
+def test_portions_of_changing_size(model, dtype, page_size):
+    folder, requests = model[:2]
+    records = traces.changing_portions(requests, seed=page_size)
+    logits, routing = run_records(folder, dtype, records, 512, page_size)
+    compare(dtype, traces.gather(records, logits), model, routing)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [0, 1])
+def test_mixed_requests_reuse_pages(model, dtype, seed):
+    folder, requests = model[:2]
+    records, peak = traces.mixed(requests, seed=seed)
+    # the pool is exactly the peak need: pages of finished requests must be used again
+    total = sum(-(-len(t) // 64) * 64 for t in requests.values())
+    assert peak < total
+    logits, routing = run_records(folder, dtype, records, peak, 16)
+    compare(dtype, traces.gather(records, logits), model, routing)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model, dtype, tmp_path):
+    """The program itself, as a user calls it: stdin in, files and 'done' lines out.  It has no
+    taps, so its bfloat16 logits are compared with an in-process replay of the same trace (which
+    must agree to the bit, being the same engine) and that replay with the plain implementation."""
+    folder, requests, expected, plain = model
+    records, peak = traces.mixed(requests, seed=3)
+    out_dir = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out_dir), "--max-tokens", str(peak), "--page-size", "16"],
+        input="".join(json.dumps(r) + "\n" for r in records), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {r['step']}" for r in records]
+    vocab = next(iter(expected.values())).shape[1]
+    logits = {r["step"]: np.fromfile(out_dir / f"{r['step']}.f32", dtype="<f4").reshape(-1, vocab) for r in records}
+    inproc, routing = run_records(folder, dtype, records, peak, 16)
+    for step, arr in inproc.items():
+        assert np.array_equal(arr, logits[step]), f"step {step}: the program and the in-process replay differ"
+    compare(dtype, traces.gather(records, logits), model, routing)
