@@ -1,0 +1,206 @@
+"""The Python entry point: ``LLM(model, **config).generate(prompts, sampling_params)``.
+
+Surface and meanings follow the reference (engine/llm_engine.py:232-348,1119-1133,1754-1762,
+1976-2055): keyword arguments are exactly the fields of ``Config`` (an unknown one raises),
+prompts are strings or lists of token ids, ``generate`` returns ``[{"text", "token_ids"}]`` in
+the order of submission, ``step`` returns the finished requests and the signed token count of
+the step (positive: prompt tokens, negative: decoded tokens).
+"""
+from __future__ import annotations
+
+import os
+import sys
+import time
+
+import torch
+
+from ..config.method_registry import resolve_method
+from ..config.runtime import Config
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .runner import ModelRunner, StepEntry
+from .scheduler import MemoryOracle, Scheduler
+from .sequence import Sequence
+
+
+class CacheOracle(MemoryOracle):
+    """The scheduler's view of the cache manager, in pages of the tightest group."""
+
+    def __init__(self, cache):
+        self.cache = cache
+
+    def free_pages(self):
+        return min(g.pool.free_count for g in self.cache.groups) if self.cache.groups else 1 << 30
+
+    def total_pages(self):
+        return min(g.pool.num_pages for g in self.cache.groups) if self.cache.groups else 1 << 30
+
+    def free_rows(self):
+        return self.cache.num_free_rows
+
+    def pages_for_tokens(self, tokens):
+        return self.cache.pages_for_tokens(tokens)
+
+    def pages_to_append(self, seq_id, new_tokens):
+        if new_tokens <= 0:
+            return 0
+        if not self.cache.has_row(seq_id):
+            return self.cache.pages_for_tokens(new_tokens)
+        needed = self.cache.pages_needed(self.cache.row_of(seq_id), new_tokens)
+        return max(needed.values()) if needed else 0
+
+    def tokens_that_fit(self, seq_id, pages):
+        ps = self.cache.page_size
+        length = int(self.cache.row_len[self.cache.row_of(seq_id)]) if self.cache.has_row(seq_id) else 0
+        return (-length) % ps + max(0, pages) * ps
+
+    def admit(self, seq_id):
+        self.cache.admit(seq_id)
+
+    def holds(self, seq_id):
+        return self.cache.has_row(seq_id)
+
+    def release(self, seq_id):
+        self.cache.free(seq_id)
+
+
+class LLM:
+    def __init__(self, model: str, **kwargs):
+        kernels = kwargs.pop("_kernels", None)           # test seam: the kernel twins on the CPU
+        device = kwargs.pop("_device", "cuda")
+        self.config = config = Config.from_kwargs(model, **kwargs)
+        self.method = resolve_method(config.sparse_method).runtime_factory()
+        cache_tokens = config.num_kvcache_slots
+        common = dict(dtype=config.dtype, device=device, kv_page_size=config.kv_page_size,
+                      max_num_seqs=config.max_num_seqs_in_gpu, max_model_len=config.max_model_len,
+                      mlp_chunk_size=config.mlp_chunk_size, kernels=kernels)
+        if config.tiny_random:
+            self.runner = ModelRunner.from_random(config.raw_model_config, seed=config.tiny_random_seed,
+                                                  num_kvcache_tokens=cache_tokens,
+                                                  gpu_memory_utilization=config.gpu_memory_utilization, **common)
+        else:
+            self.runner = ModelRunner.from_folder(model, num_kvcache_tokens=cache_tokens,
+                                                  gpu_memory_utilization=config.gpu_memory_utilization, **common)
+        self.oracle = CacheOracle(self.runner.cache)
+        self.scheduler = Scheduler(
+            self.oracle, max_num_batched_tokens=config.max_num_batched_tokens,
+            max_num_seqs_in_batch=config.max_num_seqs_in_batch, max_decoding_seqs=config.max_decoding_seqs,
+            engine_prefill_chunk_size=config.engine_prefill_chunk_size,
+            decode_reservation_tokens=config.decode_reservation_tokens, eos=config.eos,
+            eos_token_ids=config.eos_token_ids)
+        self.sampler = Sampler(self.runner.kernels, self.runner.device, config.sampler_seed)
+        self.tokenizer = self._load_tokenizer(model)
+        self.vocab_size = self.runner.spec.vocab_size
+        self.last_step_seconds = 0.0
+
+    @staticmethod
+    def _load_tokenizer(folder: str):
+        path = os.path.join(folder, "tokenizer.json")
+        if not os.path.isfile(path):
+            return None
+        from tokenizers import Tokenizer
+        return Tokenizer.from_file(path)
+
+    # ------------------------------------------------------------------ requests
+    def _tokenize(self, prompt) -> list[int]:
+        if isinstance(prompt, str):
+            if self.tokenizer is None:
+                raise ValueError("the model folder has no tokenizer.json; pass prompts as lists of token ids")
+            ids = self.tokenizer.encode(prompt).ids
+        else:
+            ids = [int(t) for t in prompt]
+        if not ids:
+            raise ValueError("an empty prompt cannot be generated from")
+        return ids
+
+    def add_request(self, prompt, sampling_params: SamplingParams) -> int:
+        ids = self._tokenize(prompt)
+        bad = [t for t in ids if not 0 <= t < self.vocab_size]
+        if bad:
+            raise ValueError(f"prompt token {bad[0]} is outside the vocabulary [0, {self.vocab_size})")
+        if len(ids) + sampling_params.max_tokens > self.config.max_model_len:
+            raise ValueError(
+                f"Prompt length + max_tokens exceeds max_model_len: {len(ids)} + {sampling_params.max_tokens} "
+                f"> {self.config.max_model_len}. Reduce prompt/decoding length or increase max_model_len "
+                "if the model supports it.")
+        sampling_params.validate_for_vocab(self.vocab_size)
+        seq = Sequence(ids, sampling_params)
+        self.scheduler.add(seq)
+        return seq.seq_id
+
+    def abort_request(self, seq_id: int) -> bool:
+        return bool(self.scheduler.abort([seq_id]))
+
+    def is_finished(self) -> bool:
+        return self.scheduler.is_finished()
+
+    # ------------------------------------------------------------------ one engine step
+    def step(self):
+        """Schedule, run, sample, account.  Returns (finished, signed token count) where finished is
+        a list of (seq_id, completion token ids, token logprobs, top logprobs)."""
+        started = time.perf_counter()
+        schedule = self.scheduler.schedule()
+        if not schedule.items:
+            return [], 0
+        entries = [StepEntry(i.seq.seq_id, i.seq.next_tokens(i.num_tokens), [i.num_tokens - 1] if i.wants_logits else [])
+                   for i in schedule.items]
+        try:
+            logits = self.runner.step(entries)
+            wanting = [i.seq for i in schedule.items if i.wants_logits]
+            sampled, logprobs = {}, {}
+            if wanting:
+                rows = [(s.sampling_params, s.prompt_token_ids, s.completion_token_ids) for s in wanting]
+                logits = self.sampler.apply_penalties(logits, rows)
+                tokens = self.sampler.sample(logits, rows, [(s.seed, s.num_completion_tokens) for s in wanting])
+                chosen, tops = self.sampler.logprobs(logits, tokens, [s.sampling_params.logprobs for s in wanting])
+                for s, t, c, top in zip(wanting, tokens, chosen, tops):
+                    sampled[s.seq_id] = t
+                    logprobs[s.seq_id] = (c, top)
+            self.method.after_step(None)
+        except Exception:
+            self.scheduler.fail_step(schedule)
+            raise
+        prefill, decode = schedule.num_prefill_tokens, schedule.num_decode_tokens
+        finished = self.scheduler.postprocess(schedule, sampled, logprobs)
+        if self.config.validate_runtime_invariants:
+            self.runner.cache.check_invariants()
+        self.last_step_seconds = time.perf_counter() - started
+        outputs = [(s.seq_id, s.completion_token_ids, s.token_logprobs, s.top_logprobs) for s in finished]
+        return outputs, (prefill if prefill else -decode)
+
+    # ------------------------------------------------------------------ the blocking call
+    def generate(self, prompts, sampling_params, use_tqdm: bool = True) -> list[dict]:
+        if isinstance(sampling_params, list) and len(sampling_params) != len(prompts):
+            raise ValueError("prompts and sampling_params must have the same length when sampling_params "
+                             f"is a list: prompts={len(prompts)} sampling_params={len(sampling_params)}.")
+        if not isinstance(sampling_params, list):
+            sampling_params = [sampling_params] * len(prompts)
+        order = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+        outputs = {}
+        prefill_rate = decode_rate = 0.0
+        while not self.is_finished():
+            t0 = time.perf_counter()
+            finished, count = self.step()
+            dt = max(time.perf_counter() - t0, 1e-9)
+            if count > 0:
+                prefill_rate = count / dt
+            elif count < 0:
+                decode_rate = -count / dt
+            for seq_id, token_ids, _, _ in finished:
+                outputs[seq_id] = token_ids
+            if use_tqdm and finished:
+                print(f"\rGenerating {len(outputs)}/{len(prompts)}  prefill {int(prefill_rate)} tok/s  "
+                      f"decode {int(decode_rate)} tok/s", end="", file=sys.stderr, flush=True)
+        if use_tqdm:
+            print(file=sys.stderr)
+        results = []
+        for seq_id in order:
+            ids = outputs[seq_id]
+            text = self.tokenizer.decode(ids, skip_special_tokens=True) if self.tokenizer is not None else ""
+            results.append({"text": text, "token_ids": ids})
+        return results
+
+    def exit(self) -> None:
+        self.runner = None
+        if torch.cuda.is_available():
+            torch.cuda.empty_cache()

@@ -46,8 +46,8 @@ class StepEntry:
 
 class ModelRunner:
     def __init__(self, arch: Architecture, cfg, params_factory, *, dtype, device="cuda", kv_page_size=64,
-                 num_kvcache_tokens: int, max_num_seqs: int = 8, max_model_len: int | None = None,
-                 mlp_chunk_size: int = 16384, kernels=None):
+                 num_kvcache_tokens: int | None = None, max_num_seqs: int = 8, max_model_len: int | None = None,
+                 mlp_chunk_size: int = 16384, kernels=None, gpu_memory_utilization: float = 0.9):
         self.arch, self.model_config = arch, cfg
         self.dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
@@ -70,11 +70,30 @@ class ModelRunner:
             raise ValueError(f"max_model_len {self.max_model_len} exceeds the model's "
                              f"max_position_embeddings {self.spec.max_position}")
         self.kv_page_size = int(kv_page_size)
+        requests = self.model.cache_requests()
+        if num_kvcache_tokens is None or int(num_kvcache_tokens) <= 0:
+            num_kvcache_tokens = self.derive_cache_tokens(requests, max_num_seqs, gpu_memory_utilization)
         num_pages = max(1, int(num_kvcache_tokens) // self.kv_page_size)
-        self.cache = CacheManager(self.model.cache_requests(), max_rows=max_num_seqs,
+        self.cache = CacheManager(requests, max_rows=max_num_seqs,
                                   max_model_len=self.max_model_len, page_size=self.kv_page_size,
                                   num_pages=num_pages, dtype=self.dtype, device=self.device)
         self.builder = BatchBuilder(kernels, self.cache, self.dtype, self.device, self.spec.vocab_size)
+
+    def derive_cache_tokens(self, requests, max_num_seqs: int, utilization: float) -> int:
+        """Tokens of cache that fit the memory left after the weights: ``utilization`` of the card
+        minus what is in use, capped by what ``max_num_seqs`` requests of full length could hold."""
+        from ..parts.base import PagedKVRequest
+        itemsize = torch.empty((), dtype=self.dtype).element_size()
+        per_token = sum(2 * r.kv_heads * r.head_dim * itemsize for r in requests.values()
+                        if isinstance(r, PagedKVRequest))
+        cap = max_num_seqs * self.max_model_len
+        if per_token == 0 or self.device.type != "cuda":
+            return cap
+        free, total = torch.cuda.mem_get_info(self.device)
+        usable = free - int((1.0 - utilization) * total) - (2 << 30)      # 2 GiB kept for step buffers
+        if usable <= per_token * self.kv_page_size:
+            raise RuntimeError("no GPU memory is left for the cache after the weights")
+        return min(cap, usable // per_token)
 
     # ------------------------------------------------------------------ construction
     @classmethod

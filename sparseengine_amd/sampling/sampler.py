@@ -1,0 +1,84 @@
+"""Sampling of one token per logits row.
+
+Greedy rows take the arg-max; other rows are scaled by 1/temperature, cut to the top-k, then to
+the nucleus of mass top_p among the survivors, and drawn from what is left (the reference's
+order, layers/sampler.py:66-122).  The draw is the arg-max of logit + Gumbel noise, the same
+distribution as the reference's ``probs / Exp(1)`` arg-max; the noise is a counter-based function
+of (sampler seed, request seed, position), so a request's tokens do not depend on which other
+requests share its batch.  Penalties (layers/sampler.py:11-64) are applied to the float logits
+before the kernel; log-probabilities are ``log_softmax`` of the penalised float logits.
+"""
+from __future__ import annotations
+
+import torch
+
+_MASK = (1 << 64) - 1
+
+
+def mix64(x: int) -> int:
+    """splitmix64 finaliser."""
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & _MASK
+    return x ^ (x >> 31)
+
+
+def row_seed(sampler_seed: int, request_seed: int, position: int) -> int:
+    """64 bits that identify one draw; returned as a signed value that fits an int64 tensor."""
+    value = mix64(mix64(mix64(sampler_seed & _MASK) ^ (request_seed & _MASK)) ^ (position & _MASK))
+    return value - (1 << 64) if value >= (1 << 63) else value
+
+
+class Sampler:
+    def __init__(self, kernels, device, sampler_seed: int = 0):
+        self.kernels = kernels
+        self.device = torch.device(device)
+        self.sampler_seed = int(sampler_seed)
+
+    def apply_penalties(self, logits: torch.Tensor, rows) -> torch.Tensor:
+        """``rows``: per logits row (params, prompt ids, completion ids)."""
+        if not any(p.presence_penalty != 0.0 or p.repetition_penalty != 1.0 for p, _, _ in rows):
+            return logits
+        logits = logits.clone()
+        for r, (p, prompt, completion) in enumerate(rows):
+            if p.repetition_penalty != 1.0 and (prompt or completion):
+                seen = torch.tensor(sorted(set(prompt) | set(completion)), dtype=torch.long, device=logits.device)
+                values = logits[r, seen]
+                logits[r, seen] = torch.where(values > 0, values / p.repetition_penalty, values * p.repetition_penalty)
+            if p.presence_penalty != 0.0 and completion:
+                seen = torch.tensor(sorted(set(completion)), dtype=torch.long, device=logits.device)
+                logits[r, seen] -= p.presence_penalty
+        return logits
+
+    def sample(self, logits: torch.Tensor, rows, seeds_and_positions) -> list[int]:
+        """``logits`` float32 ``[n, vocab]``; ``rows`` as in ``apply_penalties``;
+        ``seeds_and_positions``: per row (request seed, index of the token being drawn)."""
+        n = logits.shape[0]
+        params = [p for p, _, _ in rows]
+        out = torch.empty(n, dtype=torch.int32, device=logits.device)
+        if all(p.greedy for p in params):
+            self.kernels.sample(logits, None, None, None, None, out)
+            return out.tolist()
+        temperature = torch.tensor([0.0 if p.greedy else p.temperature for p in params], dtype=torch.float32)
+        top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32) if any(p.top_k for p in params) else None
+        top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32) if any(p.top_p < 1.0 for p in params) else None
+        seeds = torch.tensor([row_seed(self.sampler_seed, s, pos) for s, pos in seeds_and_positions], dtype=torch.int64)
+        to = lambda t: None if t is None else t.to(logits.device)
+        self.kernels.sample(logits, to(temperature), to(top_k), to(top_p), to(seeds), out)
+        return out.tolist()
+
+    @staticmethod
+    def logprobs(logits: torch.Tensor, tokens: list[int], top: list[int | None]):
+        """(log-probability of each chosen token, per row {token: logprob} of its top entries)."""
+        if all(t is None for t in top):
+            return [None] * len(tokens), [None] * len(tokens)
+        logp = torch.log_softmax(logits, dim=-1)
+        chosen = logp.gather(1, torch.tensor(tokens, device=logits.device)[:, None])[:, 0].tolist()
+        tops = []
+        for r, k in enumerate(top):
+            if not k:
+                tops.append(None if k is None else {})
+                continue
+            values, ids = torch.topk(logp[r], k)
+            tops.append(dict(zip(ids.tolist(), values.tolist())))
+        return [c if k is not None else None for c, k in zip(chosen, top)], tops
