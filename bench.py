@@ -1,0 +1,168 @@
+"""Decode and prefill throughput at MiniMax-M2 layer sizes on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Model: the sizes of MiniMax M2 (hidden 3072, 48 query / 8 kv heads of 128, rotary 64, 256 experts
+top-8 of width 1536, vocabulary 200064) cut to 16 of its 62 layers, random weights, bfloat16.
+A "step" is one decode step of a batch of 8 requests whose prompts were 2048 random token ids
+(sampling greedily, token ids read back each step).  One JSON line is printed: ``value`` is decoded
+tokens per second at batch 8; ``prefill`` is a 2048-token prompt in one step; ``points`` holds
+decode at batch 1 and 64; ``roofline`` prices the batch-8 decode step against 8 TB/s.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK = 8.0e12            # bytes / s
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+MODEL = dict(
+    architectures=["MiniMaxM2ForCausalLM"], model_type="minimax_m2", hidden_size=3072,
+    num_attention_heads=48, num_key_value_heads=8, head_dim=128, rotary_dim=64, rope_theta=5000000.0,
+    num_local_experts=256, num_experts_per_tok=8, intermediate_size=1536, vocab_size=200064,
+    rms_norm_eps=1e-6, use_qk_norm=True, max_position_embeddings=8192, tie_word_embeddings=False)
+FULL_MODEL_LAYERS = 62
+PROMPT_LEN = 2048
+CONTEXT_LEN = 8192
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=16)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated")
+    parser.add_argument("--kv-requests", type=int, default=64, help="requests of full context the cache is sized for")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+        return 2
+
+    import torch
+
+    import sparseengine_amd  # noqa: F401
+    from sparseengine_amd.engine.runner import ModelRunner, StepEntry
+    from sparseengine_amd.sampling.params import SamplingParams
+    from sparseengine_amd.sampling.sampler import Sampler
+
+    cfg = dict(MODEL, num_hidden_layers=args.layers)
+    t0 = time.time()
+    runner = ModelRunner.from_random(
+        cfg, seed=0, options=dict(std=0.02, norm_std=0.1, bias_std=0.01), on_device=True, dtype=args.dtype,
+        kv_page_size=64, num_kvcache_tokens=args.kv_requests * CONTEXT_LEN, max_num_seqs=max(64, args.batch),
+        max_model_len=CONTEXT_LEN)
+    torch.cuda.synchronize()
+    print(f"[bench] model built in {time.time() - t0:.1f} s, "
+          f"{torch.cuda.memory_allocated() / 2**30:.1f} GiB allocated", file=sys.stderr, flush=True)
+    sampler = Sampler(runner.kernels, runner.device, 0)
+    greedy = SamplingParams(temperature=0.0, max_tokens=1 << 20, ignore_eos=True)
+    gen = torch.Generator().manual_seed(0)
+
+    def prompt():
+        return torch.randint(0, cfg["vocab_size"], (PROMPT_LEN,), generator=gen).tolist()
+
+    def sync():
+        torch.cuda.synchronize()
+
+    def prefill(ids, n_at_once=4):
+        """Prompts of the requests ``ids``, a few whole prompts per step; returns their first tokens."""
+        first = {}
+        for i in range(0, len(ids), n_at_once):
+            chunk = ids[i:i + n_at_once]
+            logits = runner.step([StepEntry(r, prompt(), [PROMPT_LEN - 1]) for r in chunk])
+            tokens = sampler.sample(logits, [(greedy, [], [])] * len(chunk), [(0, 0)] * len(chunk))
+            first.update(dict(zip(chunk, tokens)))
+        return first
+
+    def decode(batch, steps, warmup, tag):
+        ids = [f"{tag}{i}" for i in range(batch)]
+        last = prefill(ids)
+        rows = [(greedy, [], [])] * batch
+        seeds = [(0, 0)] * batch
+
+        def one():
+            logits = runner.step([StepEntry(r, [last[r]], [0]) for r in ids])
+            for r, t in zip(ids, sampler.sample(logits, rows, seeds)):
+                last[r] = t
+        for _ in range(warmup):
+            one()
+        sync()
+        start = time.perf_counter()
+        for _ in range(steps):
+            one()
+        sync()
+        seconds = time.perf_counter() - start
+        taps = {}
+        runner.step([StepEntry(r, [last[r]], []) for r in ids], taps=taps)       # untimed: which experts a step touches
+        distinct = [int(torch.unique(i).numel()) for i, _ in taps["router"]]
+        context = PROMPT_LEN + warmup + steps / 2
+        for r in ids:
+            runner.release(r)
+        return seconds / steps, distinct, context
+
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    h, H, Hkv, D, E, K, I, V, L = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
+                                   cfg["head_dim"], cfg["num_local_experts"], cfg["num_experts_per_tok"],
+                                   cfg["intermediate_size"], cfg["vocab_size"], args.layers)
+    dense_layer = ((H + 2 * Hkv) * D * h + h * H * D) * itemsize + E * h * 4
+    expert_bytes = 3 * I * h * itemsize
+    kv_token_layer = 2 * Hkv * D * itemsize
+
+    def decode_bytes(batch, distinct, context):
+        return (L * dense_layer + sum(distinct) * expert_bytes + V * h * itemsize
+                + batch * context * kv_token_layer * L)
+
+    # ---- prefill of one 2048-token prompt
+    times = []
+    for i in range(4):
+        sync()
+        t = time.perf_counter()
+        runner.step([StepEntry(f"p{i}", prompt(), [PROMPT_LEN - 1])])
+        sync()
+        times.append(time.perf_counter() - t)
+        runner.release(f"p{i}")
+    prefill_s = min(times[1:])
+    T = PROMPT_LEN
+    prefill_flops = L * (2 * T * h * (H + 2 * Hkv) * D + 2 * T * H * D * h + 2 * T * h * E + 2 * T * K * 3 * I * h
+                         + 4 * H * D * T * (T + 1) / 2) + 2 * V * h
+    peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
+    print(f"[bench] prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+
+    # ---- decode
+    step_s, distinct, context = decode(args.batch, args.steps, args.warmup, "d")
+    print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+    points = {}
+    for b in [int(x) for x in args.points.split(",") if x]:
+        s, _, _ = decode(b, max(8, args.steps // 2), max(2, args.warmup // 2), f"b{b}_")
+        points[f"decode_b{b}"] = round(b / s, 1)
+        print(f"[bench] decode batch {b}: {s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+
+    achieved = decode_bytes(args.batch, distinct, context) / step_s
+    line = {
+        "metric": "decode tok/s @ batch 8 (MiniMax-M2 sizes, 16 layers, 1 GPU)", "value": round(args.batch / step_s, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random token ids, random weights",
+        "config": {"model": "MiniMax-M2 layer sizes", "num_layers": L, "model_layers": FULL_MODEL_LAYERS,
+                   "global_batch": args.batch, "seq_len": CONTEXT_LEN, "prompt_len": PROMPT_LEN, "hidden_size": h,
+                   "num_attention_heads": H, "num_key_value_heads": Hkv, "head_dim": D, "rotary_dim": cfg["rotary_dim"],
+                   "num_local_experts": E, "num_experts_per_tok": K, "intermediate_size": I, "vocab_size": V,
+                   "kv_page_size": 64, "kv_cache_tokens": args.kv_requests * CONTEXT_LEN, "parallelism": "single GPU"},
+        "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(prefill_flops / prefill_s / peak, 5)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

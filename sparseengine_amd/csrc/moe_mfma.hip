@@ -1,0 +1,187 @@
+// Grouped expert GEMMs on the matrix cores (bfloat16 in, float accumulate) for gfx950.
+//
+// Work is a list of tiles of BM = 16 * MB sorted assignments that share one expert (see
+// moe_align in moe.hip).  A workgroup of four wavefronts computes BN = 16 * NB output columns of
+// one tile; the four wavefronts split the reduction dimension K into quarters, each streaming
+// its quarter of the expert's weight rows straight from memory into MFMA operands
+// (v_mfma_f32_16x16x32_bf16: weights are the A operand, the tile's activation rows the B
+// operand), and the four partial tiles are summed through LDS before the epilogue.
+//
+//   MODE 0 (gate-up + SwiGLU): in row = x[a / top_k]; w = w13[e] = [gate rows; up rows], [2N, K];
+//       out[a, n] = silu(g) * u; g and u are rounded to bfloat16, silu is taken in float and
+//       rounded, the product is rounded.
+//   MODE 1 (down): in row = act[a]; w = w2[e], [N, K]; out[a, n] = (in . w[n]) * route_weight[a].
+//
+// Every output element is one dot product in a fixed order of K, so a row's result does not
+// depend on its place in the tile or on what else is in the batch.
+// Requires K % 128 == 0 and N % BN == 0; other sizes take the general kernel in moe.hip.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+template <int MODE, int MB, int NB>
+__global__ void __launch_bounds__(256)
+grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                         bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                         const int32_t* __restrict__ tile_expert,
+                         const int32_t* __restrict__ counters,
+                         const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                         int K) {
+  constexpr int BM = 16 * MB;
+  constexpr int BN = 16 * NB;
+  constexpr int NBT = MODE == 0 ? 2 * NB : NB;  // weight blocks per wave: gate blocks, then up blocks
+  const int tile = blockIdx.y;
+  if (tile >= counters[0]) return;  // uniform over the block
+
+  constexpr int P = NB * MB;                   // output blocks of 16 x 16 (gate/up pairs in MODE 0)
+  constexpr int PARTS = MODE == 0 ? 2 : 1;
+  // block p is finished by wave p % 4; the other three waves leave their partial sums here
+  __shared__ floatx4 partial[P][3][PARTS][SE_WAVE];
+  __shared__ int32_t rows[BM];
+
+  const int lane = threadIdx.x & (SE_WAVE - 1);
+  const int wave = threadIdx.x / SE_WAVE;
+  const int expert = tile_expert[tile];
+  const int n0 = blockIdx.x * BN;
+  if (threadIdx.x < BM) rows[threadIdx.x] = sorted[tile * BM + threadIdx.x];
+  __syncthreads();
+
+  const int col = lane & 15;   // row of the weight block (A) / row of the activation block (B)
+  const int kgroup = lane >> 4;  // which 8 of the 32 k of a step this lane holds
+  const int64_t w_rows = MODE == 0 ? 2 * static_cast<int64_t>(N) : N;
+  const bf16_t* we = w + static_cast<int64_t>(expert) * w_rows * K;
+
+  const bf16_t* a_ptr[NBT];
+#pragma unroll
+  for (int nb = 0; nb < NBT; ++nb) {
+    const int block_row = (MODE == 0 && nb >= NB) ? N + n0 + (nb - NB) * 16 : n0 + nb * 16;
+    a_ptr[nb] = we + static_cast<int64_t>(block_row + col) * K + kgroup * 8;
+  }
+  const bf16_t* b_ptr[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int a = rows[mb * 16 + col];
+    const int64_t src = a < assignments ? (MODE == 0 ? a / top_k : a) : 0;  // padding reads row 0
+    b_ptr[mb] = in + src * K + kgroup * 8;
+  }
+
+  floatx4 acc[NBT][MB];
+#pragma unroll
+  for (int nb = 0; nb < NBT; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int k_begin = wave * (K / 4);
+  const int k_end = k_begin + K / 4;
+#pragma unroll 2
+  for (int k = k_begin; k < k_end; k += 32) {
+    uint4 af[NBT], bf[MB];
+#pragma unroll
+    for (int nb = 0; nb < NBT; ++nb) af[nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + k);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) bf[mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k);
+#pragma unroll
+    for (int nb = 0; nb < NBT; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            __builtin_bit_cast(bf16x8, af[nb]), __builtin_bit_cast(bf16x8, bf[mb]), acc[nb][mb], 0, 0, 0);
+  }
+
+  // lane (kgroup, col) holds, for i < 4, the sum for weight row 4 * kgroup + i and activation row col
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int p = nb * MB + mb;
+      const int owner = p & 3;
+      if (wave != owner) {
+        const int slot = ((wave - owner + 4) & 3) - 1;
+#pragma unroll
+        for (int part = 0; part < PARTS; ++part) partial[p][slot][part][lane] = acc[part * NB + nb][mb];
+      }
+    }
+  __syncthreads();
+
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int p = nb * MB + mb;
+      if ((p & 3) != wave) continue;
+      floatx4 total[PARTS];
+#pragma unroll
+      for (int part = 0; part < PARTS; ++part) {
+        total[part] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {  // the quarters of K are always added in the same order
+          if (s == wave)
+            total[part] += acc[part * NB + nb][mb];
+          else
+            total[part] += partial[p][((s - wave + 4) & 3) - 1][part][lane];
+        }
+      }
+      const int a = rows[mb * 16 + col];
+      if (a >= assignments) continue;
+      uint16_t y[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v;
+        if (MODE == 0) {
+          const float gate = round_to<bf16_t>(total[0][i]);
+          const float up = round_to<bf16_t>(total[PARTS - 1][i]);
+          const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
+          v = act * up;
+        } else {
+          v = total[0][i] * route_weight[a];
+        }
+        y[i] = float_to_bf16_bits(v);
+      }
+      uint2 packed;
+      packed.x = static_cast<uint32_t>(y[0]) | (static_cast<uint32_t>(y[1]) << 16);
+      packed.y = static_cast<uint32_t>(y[2]) | (static_cast<uint32_t>(y[3]) << 16);
+      *reinterpret_cast<uint2*>(out + static_cast<int64_t>(a) * N + n0 + nb * 16 + 4 * kgroup) = packed;
+    }
+}
+
+template <int MODE, int MB, int NB>
+static void launch(const void* in, const void* w, void* out, const int32_t* sorted,
+                   const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
+                   int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
+  dim3 grid(N / (16 * NB), max_tiles);
+  grouped_gemm_mfma_kernel<MODE, MB, NB><<<grid, 256, 0, stream>>>(
+      static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
+      tile_expert, counters, route_weight, assignments, top_k, N, K);
+}
+
+// tile_rows: 16, 32 or 64 (the alignment the sorted list was built with); col_blocks: 1 or 2.
+extern "C" int se_grouped_gemm_mfma(const void* in, const void* w, void* out, const int32_t* sorted,
+                                    const int32_t* tile_expert, const int32_t* counters,
+                                    const float* route_weight, int assignments, int top_k, int N,
+                                    int K, int max_tiles, int mode, int tile_rows, int col_blocks,
+                                    hipStream_t stream) {
+  if (assignments <= 0) return SE_OK;
+  if (K <= 0 || K % 128 || N <= 0 || N % (16 * col_blocks)) return SE_ERR_SHAPE;
+  if (max_tiles <= 0 || max_tiles > 65535) return SE_ERR_SHAPE;
+  if (mode != 0 && mode != 1) return SE_ERR_SHAPE;
+#define SE_CASE(MB, NB)                                                                             \
+  if (tile_rows == 16 * MB && col_blocks == NB) {                                                   \
+    if (mode == 0)                                                                                  \
+      launch<0, MB, NB>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,      \
+                        top_k, N, K, max_tiles, stream);                                            \
+    else                                                                                            \
+      launch<1, MB, NB>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,      \
+                        top_k, N, K, max_tiles, stream);                                            \
+    SE_CHECK_LAUNCH();                                                                              \
+    return SE_OK;                                                                                   \
+  }
+  SE_CASE(1, 1)
+  SE_CASE(1, 2)
+  SE_CASE(2, 1)
+  SE_CASE(2, 2)
+  SE_CASE(4, 1)
+  SE_CASE(4, 2)
+#undef SE_CASE
+  return SE_ERR_SHAPE;
+}

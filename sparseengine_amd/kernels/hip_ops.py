@@ -78,6 +78,10 @@ _SIGNATURES = {
         "se_moe_sum": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "se_silu_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     },
+    "moe_mfma": {
+        "se_grouped_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    },
     "sampling": {
         "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p],
@@ -115,12 +119,15 @@ def moe_tile_bounds(assignments: int, experts: int, tile_rows: int) -> tuple[int
 class MoeWorkspace:
     """Scratch tensors of the expert pipeline, sized for a largest number of tokens."""
 
+    TILE_ROWS = (16, 32, 64)      # alignments the expert kernels may ask for
+
     def __init__(self, max_tokens: int, top_k: int, experts: int, hidden: int, intermediate: int,
-                 dtype: torch.dtype, device, tile_rows: int = 16):
+                 dtype: torch.dtype, device):
         assignments = max_tokens * top_k
-        capacity, max_tiles = moe_tile_bounds(assignments, experts, tile_rows)
+        bounds = [moe_tile_bounds(assignments, experts, rows) for rows in self.TILE_ROWS]
+        capacity, max_tiles = max(b[0] for b in bounds), max(b[1] for b in bounds)
         self.max_tokens, self.top_k, self.experts = max_tokens, top_k, experts
-        self.hidden, self.intermediate, self.dtype, self.tile_rows = hidden, intermediate, dtype, tile_rows
+        self.hidden, self.intermediate, self.dtype = hidden, intermediate, dtype
         self.sorted = torch.empty(capacity, dtype=torch.int32, device=device)
         self.tile_expert = torch.empty(max_tiles, dtype=torch.int32, device=device)
         self.counters = torch.zeros(2, dtype=torch.int32, device=device)
@@ -135,7 +142,7 @@ class MoeWorkspace:
 class HipKernels:
     """The kernel interface of the engine, served by the gfx950 libraries."""
 
-    libraries = ("norm", "rope_kv", "attention_generic", "moe", "sampling")
+    libraries = ("norm", "rope_kv", "attention_generic", "moe", "moe_mfma", "sampling")
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -257,15 +264,15 @@ class HipKernels:
             top_k, int(scoring == "softmax"), int(bool(normalize)), float(scaling), _stream()),
             "router_topk")
 
-    def moe_align(self, ids, experts: int, ws: MoeWorkspace):
+    def moe_align(self, ids, experts: int, ws: MoeWorkspace, tile_rows: int = 16):
         _i32(ids, "ids")
         assignments = ids.numel()
-        capacity, max_tiles = moe_tile_bounds(assignments, experts, ws.tile_rows)
+        capacity, max_tiles = moe_tile_bounds(assignments, experts, tile_rows)
         _require(ws.sorted.numel() >= capacity and ws.tile_expert.numel() >= max_tiles, "workspace too small")
         if experts > 4096:
             raise KernelShapeError(f"moe_align: {experts} experts are above the kernel's limit 4096")
         _check(_fn.get("moe", "se_moe_align")(
-            _ptr(ids), assignments, experts, ws.tile_rows, _ptr(ws.sorted), _ptr(ws.tile_expert),
+            _ptr(ids), assignments, experts, tile_rows, _ptr(ws.sorted), _ptr(ws.tile_expert),
             _ptr(ws.counters), _stream()), "moe_align")
         return max_tiles
 
@@ -284,17 +291,34 @@ class HipKernels:
                  and weights.dtype == torch.float32 and weights.is_contiguous(), "routing shapes")
         _require(ws.fits(tokens, top_k, experts, hidden, inter, x.dtype), "moe workspace does not fit")
         assignments = tokens * top_k
-        max_tiles = self.moe_align(ids, experts, ws)
-        if max_tiles > 65535:
-            raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
-        gg = _fn.get("moe", "se_grouped_gemm_generic")
         code = _code(x.dtype)
-        _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
-                  _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, code,
-                  _stream()), "moe gate-up")
-        _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
-                  _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                  code, _stream()), "moe down")
+        if x.dtype == torch.bfloat16 and hidden % 128 == 0 and inter % 128 == 0:
+            # matrix-core path: tiles as tall as an expert's usual share of the step, blocks as wide
+            # as still leaves enough workgroups for the whole chip
+            share = assignments / min(experts, assignments)
+            tile_rows = 16 if share <= 16 else 32 if share <= 32 else 64
+            max_tiles = self.moe_align(ids, experts, ws, tile_rows)
+            if max_tiles > 65535:
+                raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
+            gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
+            wide = 2 if max_tiles * (inter // 32) >= 2048 else 1
+            _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                      _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
+                      wide, _stream()), "moe gate-up (mfma)")
+            _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                      _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
+                      tile_rows, wide, _stream()), "moe down (mfma)")
+        else:
+            max_tiles = self.moe_align(ids, experts, ws, 16)
+            if max_tiles > 65535:
+                raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
+            gg = _fn.get("moe", "se_grouped_gemm_generic")
+            _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                      _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, code,
+                      _stream()), "moe gate-up")
+            _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                      _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
+                      code, _stream()), "moe down")
         _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
                                             _stream()), "moe_sum")
 

@@ -16,7 +16,7 @@ from .linear import linear
 
 
 class RoutedExperts(Part):
-    kernel_libraries = ("moe",)
+    kernel_libraries = ("moe", "moe_mfma")
 
     def __init__(self, spec: MoESpec, hidden_size: int, chunk_tokens: int = 16384):
         if not 1 <= spec.top_k <= spec.num_experts:

@@ -270,25 +270,29 @@ def test_moe_align_groups_every_assignment_once(hip):
     for tokens, k, experts in [(1, 8, 256), (2048, 8, 256), (33, 2, 8), (100, 4, 16), (7, 1, 1)]:
         ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
         ws = MoeWorkspace(tokens, k, experts, 16, 16, torch.float32, "cuda")
-        ws.sorted.fill_(-7); ws.tile_expert.fill_(-7)
-        hip.moe_align(ids, experts, ws)
-        n_tiles, n_sorted = ws.counters.tolist()
-        assert n_sorted == n_tiles * 16
-        sorted_ids = ws.sorted[:n_sorted].cpu()
-        real = sorted_ids[sorted_ids < tokens * k]
-        assert sorted(real.tolist()) == list(range(tokens * k))
-        flat = ids.flatten().cpu()
-        te = ws.tile_expert[:n_tiles].cpu()
-        assert (te[1:] >= te[:-1]).all()
-        for t in range(n_tiles):
-            chunk = sorted_ids[t * 16:(t + 1) * 16]
-            chunk = chunk[chunk < tokens * k]
-            assert chunk.numel() > 0 and (flat[chunk.long()] == te[t]).all()
+        for rows in (16, 32, 64):
+            ws.sorted.fill_(-7); ws.tile_expert.fill_(-7)
+            hip.moe_align(ids, experts, ws, rows)
+            n_tiles, n_sorted = ws.counters.tolist()
+            assert n_sorted == n_tiles * rows
+            sorted_ids = ws.sorted[:n_sorted].cpu()
+            real = sorted_ids[sorted_ids < tokens * k]
+            assert sorted(real.tolist()) == list(range(tokens * k))
+            flat = ids.flatten().cpu()
+            te = ws.tile_expert[:n_tiles].cpu()
+            assert (te[1:] >= te[:-1]).all()
+            for t in range(n_tiles):
+                chunk = sorted_ids[t * rows:(t + 1) * rows]
+                chunk = chunk[chunk < tokens * k]
+                assert chunk.numel() > 0 and (flat[chunk.long()] == te[t]).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,hidden,inter,experts,k", [
-    (1, 64, 32, 8, 2), (45, 96, 48, 16, 4), (130, 200, 72, 5, 5), (9, 256, 128, 1, 1), (64, 384, 160, 32, 8)])
+    (1, 64, 32, 8, 2), (45, 96, 48, 16, 4), (130, 200, 72, 5, 5), (9, 256, 128, 1, 1), (64, 384, 160, 32, 8),
+    # sizes the matrix-core kernels take (hidden and width multiples of 128), tiles of 16, 32 and 64 rows
+    (1, 256, 128, 8, 2), (3, 384, 256, 16, 4), (70, 256, 128, 4, 2), (200, 512, 384, 6, 3), (33, 3072, 1536, 16, 8),
+    (2048, 256, 128, 64, 8)])
 def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     x = randn(tokens, hidden, dtype=dtype, seed=11)
