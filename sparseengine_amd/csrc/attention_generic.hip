@@ -4,6 +4,9 @@
 // any page size, float and bfloat16 storage, with an optional sliding window.  It is the
 // float path of the engine and the fallback for shapes the matrix-core kernels refuse.
 //
+// Cache layer layout: [pages, 2, kv_heads, page_size * head_dim]; keys [page_size][head_dim],
+// values transposed [head_dim][page_size].
+//
 // For the query at position p of a request the keys n in [max(0, p - window + 1), p] are read
 // from the request's pages through its block-table row: this step's own keys were written
 // before the call.  Scores, running maximum, running sum and the output accumulator are float;
@@ -97,11 +100,11 @@ __global__ void paged_attention_generic_kernel(
       const float pj = __shfl(p_store, j, SE_WAVE);
       const int sj = __shfl(slot, j, SE_WAVE);
       const T* vr = cache + (static_cast<int64_t>(sj / page_size) * 2 + 1) * plane + head_off +
-                    static_cast<int64_t>(sj % page_size) * head_dim;
+                    (sj % page_size);
 #pragma unroll
       for (int i = 0; i < ATT_MAX_D_PER_LANE; ++i) {
         const int d = lane + i * SE_WAVE;
-        if (d < head_dim) acc[i] += pj * to_float(vr[d]);
+        if (d < head_dim) acc[i] += pj * to_float(vr[static_cast<int64_t>(d) * page_size]);
       }
     }
   }

@@ -7,8 +7,10 @@
 // storage type and multiplies by the weight in the storage type before the rotation, as a
 // two-step tensor expression would; in float storage both roundings are the identity.
 //
-// Cache layer layout: [num_pages, 2 (k, v), kv_heads, page_size, head_dim]; a token's slot is
-// page * page_size + offset, negative slots are skipped.
+// Cache layer layout: [num_pages, 2 (k, v), kv_heads, page_size * head_dim]; inside a page a kv
+// head's keys lie [page_size][head_dim] and its values transposed, [head_dim][page_size] (the
+// matrix-core attention reads eight consecutive keys of one value dim as one operand).  A
+// token's slot is page * page_size + offset; negative slots are skipped.
 #include "common.h"
 
 template <typename T, typename W>
@@ -63,8 +65,8 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
     const int64_t page = slot / page_size;
     const int64_t off = slot % page_size;
     const int64_t plane = static_cast<int64_t>(kv_heads) * page_size * head_dim;
-    k_dst = (page * 2) * plane + off * head_dim;
-    v_dst = (page * 2 + 1) * plane + off * head_dim;
+    k_dst = (page * 2) * plane + off * head_dim;   // + head * page_size * head_dim + d
+    v_dst = (page * 2 + 1) * plane + off;          // + head * page_size * head_dim + d * page_size
   }
 
   // q: one thread per element; the thread of dim d < R/2 also produces its partner d + R/2.
@@ -101,7 +103,7 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
       k[c] = y;
       if (k_dst >= 0) cache[k_dst + head_off + d] = y;
     }
-    if (v_dst >= 0) cache[v_dst + head_off + d] = v[c];
+    if (v_dst >= 0) cache[v_dst + head_off + static_cast<int64_t>(d) * page_size] = v[c];
   }
 }
 

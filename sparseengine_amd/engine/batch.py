@@ -40,6 +40,9 @@ class GroupMeta:
     item_meta: torch.Tensor = None     # int32 [3, items] on the device: q_start, q_len, ctx_len
     max_ctx_len: int = 0
     max_q_len: int = 0
+    # (query heads per kv head, window) -> (units, num_units, tasks, num_tasks, partial slots) of
+    # the matrix-core attention kernel, prepared with the rest of the step's integers
+    work: dict = field(default_factory=dict)
 
 
 class ForwardBatch:
@@ -81,9 +84,13 @@ class ForwardBatch:
 class BatchBuilder:
     """Turns step items into a ``ForwardBatch``: cache reservation + one packed host-to-device copy."""
 
-    def __init__(self, kernels, cache: CacheManager, dtype, device, vocab_size: int):
+    def __init__(self, kernels, cache: CacheManager, dtype, device, vocab_size: int,
+                 attention_shapes: dict | None = None):
+        """``attention_shapes``: cache group index -> set of (query heads per kv head, window) whose
+        attention work lists are to be prepared with every batch."""
         self.kernels, self.cache, self.dtype, self.device = kernels, cache, dtype, torch.device(device)
         self.vocab_size = vocab_size
+        self.attention_shapes = attention_shapes or {}
         self.scratch = StepScratch()
         self._host = None
         self._dev = None
@@ -132,6 +139,14 @@ class BatchBuilder:
         parts = [token_ids, positions, token_item, rows, q_start, q_len, ctx_len, want]
         for group in cache.groups:
             parts += [allocation.slots[group.index], tables[group.index].reshape(-1)]
+        works = []
+        if self.attention_shapes:
+            from ..kernels.attention_work import build_attention_work
+            for group in cache.groups:
+                for ratio, window in sorted(self.attention_shapes.get(group.index, ())):
+                    work = build_attention_work(q_len, ctx_len, ratio, group.request.kv_heads, window)
+                    works.append((group.index, (ratio, window), work, len(parts)))
+                    parts += [work.units.reshape(-1), work.tasks.reshape(-1)]
         total = sum(p.size for p in parts)
         if self._copied is not None:
             self._copied.synchronize()  # the last step's copy has left the pinned buffer
@@ -165,4 +180,8 @@ class BatchBuilder:
                 page_size=cache.page_size, item_q_start=q_start, item_q_len=q_len,
                 item_ctx_len=ctx_len, item_meta=item_meta, max_ctx_len=int(ctx_len.max()),
                 max_q_len=int(q_len.max()))
+        for group_index, key, work, at in works:
+            fb.groups[group_index].work[key] = (view(at, work.units.shape), work.units.shape[0],
+                                                view(at + 1, work.tasks.shape), work.tasks.shape[0],
+                                                work.num_slots)
         return fb

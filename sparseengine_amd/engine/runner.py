@@ -77,7 +77,14 @@ class ModelRunner:
         self.cache = CacheManager(requests, max_rows=max_num_seqs,
                                   max_model_len=self.max_model_len, page_size=self.kv_page_size,
                                   num_pages=num_pages, dtype=self.dtype, device=self.device)
-        self.builder = BatchBuilder(kernels, self.cache, self.dtype, self.device, self.spec.vocab_size)
+        shapes = {}
+        if getattr(kernels, "libraries", None):
+            for position in requests:
+                key = getattr(self.model.layers[self.spec.schedule[position].layer].mixer, "work_key", None)
+                if key is not None:
+                    shapes.setdefault(self.cache.group_of_position[position], set()).add(key())
+        self.builder = BatchBuilder(kernels, self.cache, self.dtype, self.device, self.spec.vocab_size,
+                                    attention_shapes=shapes)
 
     def derive_cache_tokens(self, requests, max_num_seqs: int, utilization: float) -> int:
         """Tokens of cache that fit the memory left after the weights: ``utilization`` of the card

@@ -68,6 +68,11 @@ _SIGNATURES = {
                                        c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
                                        c_int, c_float, c_int, c_int, c_void_p],
     },
+    "attention_mfma": {
+        "se_paged_attention_mfma": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                    c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_void_p,
+                                    c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    },
     "moe": {
         "se_router_topk": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                            c_int, c_int, c_float, c_void_p],
@@ -142,12 +147,13 @@ class MoeWorkspace:
 class HipKernels:
     """The kernel interface of the engine, served by the gfx950 libraries."""
 
-    libraries = ("norm", "rope_kv", "attention_generic", "moe", "moe_mfma", "sampling")
+    libraries = ("norm", "rope_kv", "attention_generic", "attention_mfma", "moe", "moe_mfma", "sampling")
 
     def __init__(self):
         if not torch.cuda.is_available():
             raise library.KernelLibraryError(
                 "the HIP kernels need a GPU: torch.cuda.is_available() is False")
+        self._attention_partials = None      # (float32 O partials, float32 max/sum partials)
 
     # ------------------------------------------------------------------ embedding / norms
     def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor):
@@ -233,15 +239,51 @@ class HipKernels:
         _require(meta.block_table.dtype == torch.int32 and meta.block_table.dim() == 2
                  and meta.block_table.stride(1) == 1, "block_table layout")
         _require(meta.token_row.numel() == tokens and meta.positions.numel() == tokens, "meta length")
-        if head_dim % 8 or head_dim > 512:
-            raise KernelShapeError(f"attention: head_dim {head_dim} must be a multiple of 8, at most 512")
         if heads % kv_heads:
             raise KernelShapeError(f"attention: {heads} heads do not divide into {kv_heads} kv heads")
+        window = int(window or 0)
+        if (q.dtype == torch.bfloat16 and head_dim % 32 == 0 and head_dim <= 256 and page_size % 8 == 0
+                and getattr(meta, "item_meta", None) is not None):
+            return self._paged_attention_mfma(q, cache, meta, out, scale, window)
+        if head_dim % 8 or head_dim > 512:
+            raise KernelShapeError(f"attention: head_dim {head_dim} must be a multiple of 8, at most 512")
         _check(_fn.get("attention_generic", "se_paged_attention_generic")(
             _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
             _ptr(meta.token_row), _ptr(meta.positions), _ptr(out), out.stride(0), tokens, heads,
-            kv_heads, head_dim, page_size, float(scale), int(window or 0), _code(q.dtype), _stream()),
+            kv_heads, head_dim, page_size, float(scale), window, _code(q.dtype), _stream()),
             "paged_attention")
+
+    def _paged_attention_mfma(self, q, cache, meta, out, scale, window):
+        """Matrix-core path: work units (row tile x key range) from the step's item lengths."""
+        tokens, heads, head_dim = q.shape
+        kv_heads, page_size = cache.shape[2], cache.shape[3]
+        group = heads // kv_heads
+        work = None if getattr(meta, "work", None) is None else meta.work.get((group, window))
+        if work is None:                      # not prepared by the batch builder: build it here
+            from .attention_work import build_attention_work
+            host = build_attention_work(meta.item_q_len, meta.item_ctx_len, group, kv_heads, window)
+            work = (torch.from_numpy(host.units).to(q.device), host.units.shape[0],
+                    torch.from_numpy(host.tasks).to(q.device), host.tasks.shape[0], host.num_slots)
+            if getattr(meta, "work", None) is not None:
+                meta.work[(group, window)] = work
+        units, num_units, tasks, num_tasks, num_slots = work
+        part_o = part_ml = None
+        if num_slots:
+            need = num_slots * kv_heads * 16
+            if self._attention_partials is None or self._attention_partials[0].numel() < need * head_dim:
+                self._attention_partials = (torch.empty(need * head_dim, dtype=torch.float32, device=q.device),
+                                            torch.empty(need * 2, dtype=torch.float32, device=q.device))
+            part_o, part_ml = self._attention_partials
+            if part_ml.numel() < need * 2:
+                part_ml = torch.empty(need * 2, dtype=torch.float32, device=q.device)
+                self._attention_partials = (part_o, part_ml)
+        num_items = meta.item_meta.shape[1]
+        _require(meta.item_meta.dtype == torch.int32 and meta.item_meta.is_contiguous(), "item_meta layout")
+        _check(_fn.get("attention_mfma", "se_paged_attention_mfma")(
+            _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
+            _ptr(meta.item_meta), num_items, _ptr(units), num_units, _ptr(tasks) if num_tasks else None,
+            num_tasks, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim,
+            page_size, float(scale), window, _stream()), "paged_attention (mfma)")
 
     # ------------------------------------------------------------------ mixture of experts
     def router_topk(self, logits, bias, top_k: int, ids, weights, scoring="sigmoid", normalize=True,

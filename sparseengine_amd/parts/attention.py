@@ -14,7 +14,7 @@ from .linear import linear
 
 
 class GQAAttention(Part):
-    kernel_libraries = ("rope_kv", "attention_generic")
+    kernel_libraries = ("rope_kv", "attention_generic", "attention_mfma")
 
     def __init__(self, spec: AttentionSpec, hidden_size: int):
         if spec.num_kv_heads <= 0 or spec.num_heads % spec.num_kv_heads:
@@ -40,6 +40,10 @@ class GQAAttention(Part):
     def bind(self, params):
         super().bind(params)
         self.position.prepare(params["qkv"].device)
+
+    def work_key(self):
+        """(query heads per kv head, window): what the attention kernel's work list depends on."""
+        return self.spec.num_heads // self.spec.num_kv_heads, int(self.spec.window or 0)
 
     def cache_request(self):
         return PagedKVRequest(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)

@@ -133,13 +133,27 @@ def make_paged(dtype, kv_heads, head_dim, page, lens, seed=0, extra_pages=3):
     return cache, table.cuda()
 
 
+def make_meta(table, ctx_lens, q_lens):
+    """What the batch builder hands to the attention kernels for items of these lengths."""
+    import numpy as np
+    token_row, positions = [], []
+    for r, (n, ql) in enumerate(zip(ctx_lens, q_lens)):
+        token_row += [r] * ql
+        positions += list(range(n - ql, n))
+    q_start = np.concatenate(([0], np.cumsum(q_lens)[:-1])).astype(np.int32)
+    item_meta = torch.tensor(np.stack([q_start, np.asarray(q_lens), np.asarray(ctx_lens)]), dtype=torch.int32).cuda()
+    return SimpleNamespace(block_table=table, token_row=torch.tensor(token_row, dtype=torch.int32).cuda(),
+                           positions=torch.tensor(positions, dtype=torch.int32).cuda(), item_meta=item_meta,
+                           item_q_len=np.asarray(q_lens), item_ctx_len=np.asarray(ctx_lens), work={})
+
+
 def dense_attention(q, cache, table, row, pos, scale, window, page):
     """Reference through the library routine: gather the request's keys, call SDPA for one query."""
     first = max(0, pos - window + 1) if window else 0
     n = torch.arange(first, pos + 1, device="cuda")
     pages = table[row, n // page].long()
     k = cache[pages, 0, :, n % page, :].float().transpose(0, 1)   # [Hkv, n, D]
-    v = cache[pages, 1, :, n % page, :].float().transpose(0, 1)
+    v = cache[:, 1].view(cache.shape[0], cache.shape[2], cache.shape[4], page)[pages, :, :, n % page].float().transpose(0, 1)
     H, D = q.shape
     group = H // k.shape[0]
     k = k.repeat_interleave(group, 0)
@@ -151,7 +165,8 @@ def dense_attention(q, cache, table, row, pos, scale, window, page):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page,window", [
     (4, 2, 16, 16, 0), (6, 3, 32, 16, 0), (48, 8, 128, 64, 0), (12, 2, 64, 32, 0),
-    (5, 1, 48, 16, 0), (8, 8, 80, 16, 0), (4, 2, 16, 16, 20), (6, 1, 128, 64, 100)])
+    (5, 1, 48, 16, 0), (8, 8, 80, 16, 0), (4, 2, 16, 16, 20), (6, 1, 128, 64, 100), (6, 3, 32, 8, 0),
+    (12, 4, 96, 16, 0), (4, 1, 256, 32, 50), (14, 2, 160, 16, 0)])
 def test_paged_attention_mixed_batch(hip, twin, dtype, heads, kv_heads, head_dim, page, window):
     # three requests: a whole prompt, a portion on top of a cached prefix, a single decoded token
     lens = [37, 150, 301]
@@ -162,8 +177,7 @@ def test_paged_attention_mixed_batch(hip, twin, dtype, heads, kv_heads, head_dim
         token_row += [r] * ql
         positions += list(range(n - ql, n))
     T = len(token_row)
-    meta = SimpleNamespace(block_table=table, token_row=torch.tensor(token_row, dtype=torch.int32).cuda(),
-                           positions=torch.tensor(positions, dtype=torch.int32).cuda())
+    meta = make_meta(table, lens, q_lens)
     qkv = randn(T, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=9)
     q = qkv[:, :heads * head_dim].view(T, heads, head_dim)
     scale = head_dim ** -0.5
@@ -193,14 +207,14 @@ def test_paged_attention_finds_one_far_key(hip, dtype):
         for kvh in range(kv_heads):
             qh = q[0, kvh * (heads // kv_heads)].float()
             c[pg, 0, kvh, off] = (qh / qh.norm() * 60).to(dtype)
-        meta = SimpleNamespace(block_table=table, token_row=torch.zeros(1, dtype=torch.int32).cuda(),
-                               positions=torch.tensor([n - 1], dtype=torch.int32).cuda())
+        meta = make_meta(table, [n], [1])
         out = torch.empty(1, heads * head_dim, dtype=dtype, device="cuda")
         hip.paged_attention(q, c, meta, out, 1.0, 0)
         for kvh in range(kv_heads):
             head = kvh * (heads // kv_heads)
             got = out[0, head * head_dim:(head + 1) * head_dim].float()
-            torch.testing.assert_close(got, c[pg, 1, kvh, off].float(), rtol=2e-2, atol=2e-2)
+            value = c[pg, 1, kvh].view(head_dim, page)[:, off].float()     # values lie transposed in a page
+            torch.testing.assert_close(got, value, rtol=2e-2, atol=2e-2)
 
 
 def test_router_matches_library_topk(hip, twin):
@@ -370,3 +384,22 @@ def test_sampling_distribution(hip):
     p3 = torch.softmax(torch.tensor([3.0, 2.0, 1.0]), -1)   # 0.665, 0.245, 0.090: nucleus 0.7 keeps two
     expect = torch.tensor([p3[0], p3[1], 0, 0, 0]) / (p3[0] + p3[1])
     assert (freq - expect).abs().max() < 0.015
+
+
+@pytest.mark.parametrize("batch,ctx,q_len", [(1, 2049, 1), (3, 700, 1), (64, 300, 1), (2, 1500, 130), (1, 4100, 1)])
+def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
+    """Few rows and long contexts: the key ranges are split over many wavefronts and merged."""
+    heads, kv_heads, head_dim, page = 48, 8, 128, 64
+    dtype = torch.bfloat16
+    lens = [ctx - 3 * i for i in range(batch)]
+    cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=batch)
+    meta = make_meta(table, lens, [q_len] * batch)
+    T = batch * q_len
+    q = randn(T, heads, head_dim, dtype=dtype, seed=2)
+    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device="cuda")
+    hip.paged_attention(q, cache, meta, out_h, head_dim ** -0.5, 0)
+    assert meta.work[(heads // kv_heads, 0)][3] > 0 or batch * q_len > 100, "expected split units"
+    for t in sorted({0, T // 2, T - 1}):
+        row, pos = int(meta.token_row[t]), int(meta.positions[t])
+        ref = dense_attention(q[t], cache, table, row, pos, head_dim ** -0.5, 0, page)
+        torch.testing.assert_close(out_h[t].float(), ref, rtol=1.6e-2, atol=1.6e-2)
