@@ -39,6 +39,10 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated")
     parser.add_argument("--kv-requests", type=int, default=64, help="requests of full context the cache is sized for")
+    parser.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiling decode)")
+    parser.add_argument("--fake-context", action="store_true",
+                        help="profiling aid, never used for reported numbers: reserve the prompts' cache pages "
+                             "without computing them, so that a kernel trace holds decode steps only")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -82,7 +86,11 @@ def main() -> int:
 
     def decode(batch, steps, warmup, tag):
         ids = [f"{tag}{i}" for i in range(batch)]
-        last = prefill(ids)
+        if args.fake_context:
+            runner.cache.append([(runner.admit(r), PROMPT_LEN) for r in ids])
+            last = dict(zip(ids, torch.randint(0, cfg["vocab_size"], (batch,), generator=gen).tolist()))
+        else:
+            last = prefill(ids)
         rows = [(greedy, [], [])] * batch
         seeds = [(0, 0)] * batch
 
@@ -90,6 +98,8 @@ def main() -> int:
             logits = runner.step([StepEntry(r, [last[r]], [0]) for r in ids])
             for r, t in zip(ids, sampler.sample(logits, rows, seeds)):
                 last[r] = t
+            if args.fake_context:       # an empty cache gives every request the same token: draw them
+                last.update(zip(ids, torch.randint(0, cfg["vocab_size"], (batch,), generator=gen).tolist()))
         for _ in range(warmup):
             one()
         sync()
@@ -119,8 +129,8 @@ def main() -> int:
                 + batch * context * kv_token_layer * L)
 
     # ---- prefill of one 2048-token prompt
-    times = []
-    for i in range(4):
+    times = [0.0, 1.0] if args.no_prefill else []
+    for i in range(0 if args.no_prefill else 4):
         sync()
         t = time.perf_counter()
         runner.step([StepEntry(f"p{i}", prompt(), [PROMPT_LEN - 1])])

@@ -16,24 +16,6 @@
 #define ATT_MAX_D_PER_LANE 8  // head_dim <= 64 * 8
 
 template <typename T>
-struct Vec16;  // 16-byte vector of storage elements
-template <>
-struct Vec16<float> {
-  static constexpr int N = 4;
-  float4 v;
-  __device__ __forceinline__ float get(int i) const { return (&v.x)[i]; }
-};
-template <>
-struct Vec16<bf16_t> {
-  static constexpr int N = 8;
-  uint4 v;
-  __device__ __forceinline__ float get(int i) const {
-    const uint32_t word = (&v.x)[i >> 1];
-    return __uint_as_float((i & 1) ? (word & 0xffff0000u) : (word << 16));
-  }
-};
-
-template <typename T>
 __global__ void paged_attention_generic_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ cache,
     const int32_t* __restrict__ block_table, int bt_stride, const int32_t* __restrict__ token_row,

@@ -195,40 +195,55 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 }
 
 // One block per (merge task, kv head): task = {item, row_tile, first_slot, num_splits}.
+// Thread (n, j) of the 16 x 16 block first turns the splits' maxima and sums of row n into
+// weights in shared memory, then adds the weighted partial outputs for its value dims.
+#define MERGE_MAX_SPLITS 256
 __global__ void __launch_bounds__(256)
 attention_merge_kernel(const int32_t* __restrict__ tasks, const int32_t* __restrict__ item_meta,
                        int num_items, const float* __restrict__ part_o,
                        const float* __restrict__ part_ml, bf16_t* __restrict__ out,
                        int64_t out_stride, int heads, int kv_heads, int head_dim) {
+  __shared__ float weight[16][MERGE_MAX_SPLITS];
+  __shared__ float inv_denom[16];
   const int32_t* t = tasks + static_cast<int64_t>(blockIdx.x) * 4;
   const int item = t[0], row_tile = t[1], first_slot = t[2], splits = t[3];
   const int kvh = blockIdx.y;
   const int group = heads / kv_heads;
   const int q_start = item_meta[item], q_len = item_meta[num_items + item];
   const int n = threadIdx.x >> 4;        // row of the tile
-  const int lane16 = threadIdx.x & 15;
+  const int j = threadIdx.x & 15;
   const int rho = row_tile * 16 + n;
-  if (rho >= q_len * group) return;
+  const bool valid = rho < q_len * group;
+  const int64_t stride = static_cast<int64_t>(kv_heads) * 16;     // partial rows between two splits
+  const int64_t base0 = (static_cast<int64_t>(first_slot) * kv_heads + kvh) * 16 + n;
+  // maxima: 16 threads per row share the splits
+  float m = -INFINITY;
+  for (int s = j; s < splits; s += 16) {
+    const float ms = part_ml[(base0 + s * stride) * 2];
+    weight[n][s] = ms;
+    m = fmaxf(m, ms);
+  }
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, SE_WAVE));
+  float denom = 0.f;
+  for (int s = j; s < splits; s += 16) {
+    const float w = exp2f(weight[n][s] - m);
+    weight[n][s] = w;
+    denom += part_ml[(base0 + s * stride) * 2 + 1] * w;
+  }
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) denom += __shfl_xor(denom, off, SE_WAVE);
+  if (j == 0) inv_denom[n] = 1.f / denom;
+  __syncthreads();
+  if (!valid) return;
   const int token = q_start + rho / group;
   const int head = kvh * group + rho % group;
-  float m = -INFINITY;
-  for (int s = 0; s < splits; ++s) {
-    const int64_t base = (static_cast<int64_t>(first_slot + s) * kv_heads + kvh) * 16 + n;
-    m = fmaxf(m, part_ml[base * 2]);
-  }
-  float denom = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const int64_t base = (static_cast<int64_t>(first_slot + s) * kv_heads + kvh) * 16 + n;
-    denom += part_ml[base * 2 + 1] * exp2f(part_ml[base * 2] - m);
-  }
-  const float inv = 1.f / denom;
+  const float inv = inv_denom[n];
   bf16_t* o_row = out + static_cast<int64_t>(token) * out_stride + static_cast<int64_t>(head) * head_dim;
-  for (int d = lane16; d < head_dim; d += 16) {
+  for (int d = j; d < head_dim; d += 16) {
     float acc = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const int64_t base = (static_cast<int64_t>(first_slot + s) * kv_heads + kvh) * 16 + n;
-      acc += part_o[base * head_dim + d] * exp2f(part_ml[base * 2] - m);
-    }
+#pragma unroll 4
+    for (int s = 0; s < splits; ++s) acc += part_o[(base0 + s * stride) * head_dim + d] * weight[n][s];
     o_row[d] = from_float<bf16_t>(acc * inv);
   }
 }
@@ -244,7 +259,7 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
   if (head_dim % 32 || head_dim <= 0 || head_dim > 256) return SE_ERR_SHAPE;
   if (kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 8) return SE_ERR_SHAPE;
   if (q_stride % 8 || out_stride % 4) return SE_ERR_SHAPE;
-  if (num_tasks > 0 && (!part_o || !part_ml || !tasks)) return SE_ERR_SHAPE;
+  if (num_tasks > 0 && (!part_o || !part_ml || !tasks)) return SE_ERR_SHAPE;  // splits per task <= 256 (host)
   const float scale_log2e = scale * 1.4426950408889634f;
   dim3 grid((num_units + 3) / 4, kv_heads);
 #define SE_ATT(DS)                                                                                 \

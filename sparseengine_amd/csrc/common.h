@@ -85,3 +85,51 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 }
 
 enum SeDtype { SE_F32 = 0, SE_BF16 = 1 };
+
+// 16-byte vectors of storage elements
+template <typename T>
+struct Vec16;
+template <>
+struct Vec16<float> {
+  static constexpr int N = 4;
+  float4 v;
+  __device__ __forceinline__ float get(int i) const { return (&v.x)[i]; }
+  __device__ __forceinline__ void set(int i, float f) { (&v.x)[i] = f; }
+};
+template <>
+struct Vec16<bf16_t> {
+  static constexpr int N = 8;
+  uint4 v;
+  __device__ __forceinline__ float get(int i) const {
+    const uint32_t word = (&v.x)[i >> 1];
+    return __uint_as_float((i & 1) ? (word & 0xffff0000u) : (word << 16));
+  }
+  __device__ __forceinline__ void set(int i, float f) {
+    uint32_t& word = (&v.x)[i >> 1];
+    const uint32_t bits = float_to_bf16_bits(f);
+    word = (i & 1) ? ((word & 0x0000ffffu) | (bits << 16)) : ((word & 0xffff0000u) | bits);
+  }
+};
+
+// Bring n elements (n % Vec16<T>::N == 0, 16-byte aligned) into shared memory as float with a block
+// of 256 threads.  Every load is issued before the first one is used: a row is a handful of
+// vectors per thread, and a loop that waits for each load in turn costs a memory latency apiece.
+template <typename T, int MAXV>
+__device__ __forceinline__ void stage_row(const T* src, float* dst, int n) {
+  constexpr int VN = Vec16<T>::N;
+  const int nvec = n / VN;
+  Vec16<T> v[MAXV];
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) v[i].v = *reinterpret_cast<const decltype(v[i].v)*>(src + static_cast<int64_t>(idx) * VN);
+  }
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) dst[idx * VN + j] = v[i].get(j);
+    }
+  }
+}

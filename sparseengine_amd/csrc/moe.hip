@@ -137,15 +137,46 @@ __global__ void moe_align_kernel(const int32_t* __restrict__ ids, int assignment
   __syncthreads();
   for (int a = threadIdx.x; a < assignments; a += blockDim.x) atomicAdd(&counts[ids[a]], 1);
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int32_t run = 0;
-    for (int e = 0; e < experts; ++e) {
+  // exclusive prefix sum of the padded counts: every thread scans its own stretch of experts,
+  // wave 0 scans the stretch totals
+  {
+    const int per_thread = (experts + blockDim.x - 1) / blockDim.x;
+    const int first = threadIdx.x * per_thread;
+    int32_t mine = 0;
+    for (int e = first; e < first + per_thread && e < experts; ++e)
+      mine += (counts[e] + tile_rows - 1) / tile_rows * tile_rows;
+    __shared__ int32_t stretch[1024];
+    stretch[threadIdx.x] = mine;
+    __syncthreads();
+    if (threadIdx.x < SE_WAVE) {
+      // 1024 / 64 = 16 consecutive stretch totals per lane
+      const int per_lane = blockDim.x / SE_WAVE;
+      int32_t lane_total = 0;
+      for (int i = 0; i < per_lane; ++i) lane_total += stretch[threadIdx.x * per_lane + i];
+      int32_t inclusive = lane_total;
+#pragma unroll
+      for (int off = 1; off < SE_WAVE; off <<= 1) {
+        const int32_t up = __shfl_up(inclusive, off, SE_WAVE);
+        if (static_cast<int>(threadIdx.x) >= off) inclusive += up;
+      }
+      int32_t run = inclusive - lane_total;
+      for (int i = 0; i < per_lane; ++i) {
+        const int32_t v = stretch[threadIdx.x * per_lane + i];
+        stretch[threadIdx.x * per_lane + i] = run;
+        run += v;
+      }
+      if (threadIdx.x == SE_WAVE - 1) {
+        offsets[experts] = run;
+        counters[0] = run / tile_rows;
+        counters[1] = run;
+      }
+    }
+    __syncthreads();
+    int32_t run = stretch[threadIdx.x];
+    for (int e = first; e < first + per_thread && e < experts; ++e) {
       offsets[e] = run;
       run += (counts[e] + tile_rows - 1) / tile_rows * tile_rows;
     }
-    offsets[experts] = run;
-    counters[0] = run / tile_rows;
-    counters[1] = run;
   }
   __syncthreads();
   for (int e = threadIdx.x; e < experts; e += blockDim.x) {
@@ -245,16 +276,18 @@ __global__ void grouped_gemm_generic_kernel(const T* __restrict__ in, const T* _
   }
 }
 
-// out[t, c] = sum over the token's top_k slots of y[t * top_k + k, c], float accumulation in slot order
+// out[t, c] = sum over the token's top_k slots of y[t * top_k + k, c], float accumulation in slot
+// order; one thread per output element (grid: tokens x column blocks)
 template <typename T>
 __global__ void moe_sum_kernel(const T* __restrict__ y, T* __restrict__ out, int top_k,
                                int hidden) {
   const int64_t t = blockIdx.x;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-    float acc = 0.f;
-    for (int k = 0; k < top_k; ++k) acc += to_float(y[(t * top_k + k) * hidden + c]);
-    out[t * hidden + c] = from_float<T>(acc);
-  }
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= hidden) return;
+  float acc = 0.f;
+#pragma unroll 8
+  for (int k = 0; k < top_k; ++k) acc += to_float(y[(t * top_k + k) * hidden + c]);
+  out[t * hidden + c] = from_float<T>(acc);
 }
 
 // out[t, c] = silu(x[t, c]) * x[t, width + c] with the roundings of the fused expert path
@@ -322,12 +355,14 @@ int se_grouped_gemm_generic(const void* in, const void* w, void* out, const int3
 int se_moe_sum(const void* y, void* out, int tokens, int top_k, int hidden, int dtype,
                hipStream_t stream) {
   if (tokens <= 0) return SE_OK;
+  if (hidden <= 0) return SE_ERR_SHAPE;
+  dim3 grid(tokens, (hidden + 255) / 256);
   if (dtype == SE_F32)
-    moe_sum_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(y),
-                                                      static_cast<float*>(out), top_k, hidden);
+    moe_sum_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(y),
+                                                    static_cast<float*>(out), top_k, hidden);
   else
-    moe_sum_kernel<bf16_t><<<tokens, 256, 0, stream>>>(static_cast<const bf16_t*>(y),
-                                                       static_cast<bf16_t*>(out), top_k, hidden);
+    moe_sum_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(y),
+                                                     static_cast<bf16_t*>(out), top_k, hidden);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -26,31 +26,122 @@ __global__ void rms_norm_kernel(const T* x, T* residual, const W* __restrict__ w
   const int64_t in_row = rows ? rows[blockIdx.x] : blockIdx.x;
   const T* xr = x + in_row * x_stride;
   T* rr = residual ? residual + in_row * res_stride : nullptr;
+  // all loads come before any store: x, residual and out may be the same memory, and a store in
+  // the loading loop would keep the loads from overlapping each other
   float sq = 0.f;
+#pragma unroll 4
   for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
     float v = to_float(xr[c]);
-    if (rr) {
-      v += to_float(rr[c]);
-      if (write_residual) rr[c] = from_float<T>(v);
-    }
+    if (rr) v += to_float(rr[c]);
     row_cache[c] = v;
     sq += v * v;
   }
   const float total = block_sum(sq, scratch);
   const float inv = rsqrtf(total / static_cast<float>(hidden) + eps);
   T* o = out + static_cast<int64_t>(blockIdx.x) * out_stride;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x)
-    o[c] = from_float<T>(row_cache[c] * inv * to_float(weight[c]));
+#pragma unroll 4
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float v = row_cache[c];
+    if (rr && write_residual) rr[c] = from_float<T>(v);
+    o[c] = from_float<T>(v * inv * to_float(weight[c]));
+  }
+}
+
+// The same with 16-byte loads and stores, all loads of a phase issued before their first use;
+// needs hidden and the row strides to be multiples of the vector length and 16-byte alignment.
+template <typename T, typename W, int MAXV>
+__global__ void __launch_bounds__(256)
+rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* out,
+                    const int32_t* __restrict__ rows, int hidden, float eps, int64_t x_stride,
+                    int64_t res_stride, int64_t out_stride, int write_residual) {
+  extern __shared__ float row_cache[];  // hidden floats, then 16 floats for the reduction
+  float* scratch = row_cache + hidden;
+  constexpr int VN = Vec16<T>::N;
+  constexpr int WN = Vec16<W>::N;
+  constexpr int WV = VN / WN;           // weight vectors per activation vector (1, or 2 for float weights)
+  const int nvec = hidden / VN;
+  const int64_t in_row = rows ? rows[blockIdx.x] : blockIdx.x;
+  const T* xr = x + in_row * x_stride;
+  T* rr = residual ? residual + in_row * res_stride : nullptr;
+
+  Vec16<T> xv[MAXV], rv[MAXV];
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+      xv[i].v = *reinterpret_cast<const decltype(xv[i].v)*>(xr + idx * VN);
+      if (rr) rv[i].v = *reinterpret_cast<const decltype(rv[i].v)*>(rr + idx * VN);
+    }
+  }
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        float v = xv[i].get(j);
+        if (rr) v += rv[i].get(j);
+        row_cache[idx * VN + j] = v;
+        sq += v * v;
+      }
+    }
+  }
+  Vec16<W> wv[MAXV][WV];
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+#pragma unroll
+      for (int k = 0; k < WV; ++k)
+        wv[i][k].v = *reinterpret_cast<const decltype(wv[i][k].v)*>(weight + idx * VN + k * WN);
+    }
+  }
+  const float total = block_sum(sq, scratch);
+  const float inv = rsqrtf(total / static_cast<float>(hidden) + eps);
+  T* o = out + static_cast<int64_t>(blockIdx.x) * out_stride;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+      Vec16<T> ov, sv;
+#pragma unroll
+      for (int j = 0; j < VN; ++j) {
+        const float v = row_cache[idx * VN + j];
+        sv.set(j, v);
+        ov.set(j, v * inv * wv[i][j / WN].get(j % WN));
+      }
+      if (rr && write_residual) *reinterpret_cast<decltype(sv.v)*>(rr + idx * VN) = sv.v;
+      *reinterpret_cast<decltype(ov.v)*>(o + idx * VN) = ov.v;
+    }
+  }
 }
 
 template <typename T, typename W>
 static int launch_rms(const void* x, void* residual, const void* weight, void* out,
                       const int32_t* rows, int n_out, int hidden, float eps, int64_t xs, int64_t rs,
-                      int64_t os, int write_residual, hipStream_t stream) {
+                      int64_t os, int write_residual, int vector_ok, hipStream_t stream) {
   const size_t shmem = (static_cast<size_t>(hidden) + 16) * sizeof(float);
-  rms_norm_kernel<T, W><<<n_out, 256, shmem, stream>>>(
-      static_cast<const T*>(x), static_cast<T*>(residual), static_cast<const W*>(weight),
-      static_cast<T*>(out), rows, hidden, eps, xs, rs, os, write_residual);
+  constexpr int VN = Vec16<T>::N;
+  const T* xp = static_cast<const T*>(x);
+  T* rp = static_cast<T*>(residual);
+  const W* wp = static_cast<const W*>(weight);
+  T* op = static_cast<T*>(out);
+  if (vector_ok && hidden % VN == 0 && xs % VN == 0 && rs % VN == 0 && os % VN == 0) {
+    const int per_thread = (hidden / VN + 255) / 256;
+#define SE_RMS(MAXV)                                                                             \
+  rms_norm_vec_kernel<T, W, MAXV><<<n_out, 256, shmem, stream>>>(xp, rp, wp, op, rows, hidden, eps, \
+                                                                 xs, rs, os, write_residual)
+    if (per_thread <= 1) SE_RMS(1);
+    else if (per_thread <= 2) SE_RMS(2);
+    else if (per_thread <= 4) SE_RMS(4);
+    else if (per_thread <= 8) SE_RMS(8);
+    else SE_RMS(16);
+#undef SE_RMS
+  } else {
+    rms_norm_kernel<T, W><<<n_out, 256, shmem, stream>>>(xp, rp, wp, op, rows, hidden, eps, xs, rs, os,
+                                                         write_residual);
+  }
   SE_CHECK_LAUNCH();
   return SE_OK;
 }
@@ -71,23 +162,24 @@ int se_embedding(const int32_t* ids, const void* table, void* out, int tokens, i
 }
 
 // x, residual (optional), out: [*, hidden] with the given row strides (in elements).
+// vector_ok: every pointer is 16-byte aligned (the wide kernel is then used where strides allow).
 // hidden is limited by the row cache kept in shared memory.
 int se_rms_norm(const void* x, void* residual, const void* weight, void* out, const int32_t* rows,
                 int n_out, int hidden, float eps, int64_t x_stride, int64_t res_stride,
-                int64_t out_stride, int write_residual, int dtype, int weight_dtype,
+                int64_t out_stride, int write_residual, int dtype, int weight_dtype, int vector_ok,
                 hipStream_t stream) {
   if (n_out <= 0) return SE_OK;
   if (hidden <= 0 || hidden > 15360) return SE_ERR_SHAPE;
   if (dtype == SE_F32) {
     if (weight_dtype != SE_F32) return SE_ERR_SHAPE;
     return launch_rms<float, float>(x, residual, weight, out, rows, n_out, hidden, eps, x_stride,
-                                    res_stride, out_stride, write_residual, stream);
+                                    res_stride, out_stride, write_residual, vector_ok, stream);
   }
   if (weight_dtype == SE_F32)
     return launch_rms<bf16_t, float>(x, residual, weight, out, rows, n_out, hidden, eps, x_stride,
-                                     res_stride, out_stride, write_residual, stream);
+                                     res_stride, out_stride, write_residual, vector_ok, stream);
   return launch_rms<bf16_t, bf16_t>(x, residual, weight, out, rows, n_out, hidden, eps, x_stride,
-                                    res_stride, out_stride, write_residual, stream);
+                                    res_stride, out_stride, write_residual, vector_ok, stream);
 }
 
 }  // extern "C"

@@ -14,6 +14,7 @@ UNIT_FIELDS = 6      # item, row_tile, key_begin, key_end, partial_slot (-1: non
 TASK_FIELDS = 4      # item, row_tile, first_slot, num_splits
 TARGET_WAVES = 2048  # wavefronts wanted in flight (256 CUs x 4 SIMDs x 2)
 MIN_SPLIT_KEYS = 64
+MAX_SPLITS = 256      # what the merge kernel's shared memory holds
 
 
 @dataclass
@@ -33,7 +34,7 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
     units, tasks, slot = [], [], 0
     for item, (n_tiles, ctx) in enumerate(zip(tiles.tolist(), ctx_len.tolist())):
         reach = min(ctx, window + int(q_len[item])) if window else ctx     # keys a tile can read
-        splits = max(1, min(want, reach // MIN_SPLIT_KEYS))
+        splits = max(1, min(want, reach // MIN_SPLIT_KEYS, MAX_SPLITS))
         tile_ids = np.arange(n_tiles, dtype=np.int32)
         if splits == 1:
             block = np.zeros((n_tiles, UNIT_FIELDS), dtype=np.int32)

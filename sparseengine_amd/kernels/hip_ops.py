@@ -56,12 +56,12 @@ _SIGNATURES = {
     "norm": {
         "se_embedding": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "se_rms_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
-                        c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p],
+                        c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p],
     },
     "rope_kv": {
         "se_qk_norm_rope_store": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                   c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int,
-                                  c_int, c_int, c_int, c_void_p],
+                                  c_int, c_int, c_int, c_int, c_void_p],
     },
     "attention_generic": {
         "se_paged_attention_generic": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p,
@@ -188,7 +188,9 @@ class HipKernels:
         _check(_fn.get("norm", "se_rms_norm")(
             _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), n_out, hidden, float(eps),
             x.stride(0), residual.stride(0) if residual is not None else 0, out.stride(0),
-            int(bool(write_residual)), _code(x.dtype), _code(weight.dtype), _stream()), "rms_norm")
+            int(bool(write_residual)), _code(x.dtype), _code(weight.dtype),
+            int(all(t is None or t.data_ptr() % 16 == 0 for t in (x, residual, weight, out))), _stream()),
+            "rms_norm")
 
     # ------------------------------------------------------------------ attention inputs
     def qk_norm_rope_store(self, qkv, positions, cos_sin, q_weight, k_weight, eps, heads, kv_heads,
@@ -218,8 +220,9 @@ class HipKernels:
         _check(_fn.get("rope_kv", "se_qk_norm_rope_store")(
             _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(cos_sin) if rotary_dim else None,
             _ptr(q_weight), _ptr(k_weight), float(eps), tokens, heads, kv_heads, head_dim, rotary_dim,
-            _ptr(cache), _ptr(slots), page_size, int(write_kv), _code(qkv.dtype), wd, _stream()),
-            "qk_norm_rope_store")
+            _ptr(cache), _ptr(slots), page_size, int(write_kv), _code(qkv.dtype), wd,
+            int(all(t is None or t.data_ptr() % 16 == 0 for t in (qkv, q_weight, k_weight, cache, cos_sin))),
+            _stream()), "qk_norm_rope_store")
 
     def paged_attention(self, q, cache, meta, out, scale: float, window: int = 0):
         """Causal attention of every token of the step against its request's pages.
