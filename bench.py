@@ -40,6 +40,7 @@ def main() -> int:
     parser.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated")
     parser.add_argument("--kv-requests", type=int, default=64, help="requests of full context the cache is sized for")
     parser.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiling decode)")
+    parser.add_argument("--no-decode", action="store_true", help="skip the decode measurements (for profiling prefill)")
     parser.add_argument("--fake-context", action="store_true",
                         help="profiling aid, never used for reported numbers: reserve the prompts' cache pages "
                              "without computing them, so that a kernel trace holds decode steps only")
@@ -145,6 +146,8 @@ def main() -> int:
     print(f"[bench] prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
 
     # ---- decode
+    if args.no_decode:
+        return 0
     step_s, distinct, context = decode(args.batch, args.steps, args.warmup, "d")
     print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
     points = {}

@@ -20,7 +20,7 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-template <int MODE, int MB, int NB>
+template <int MODE, int MB, int NB, int U>
 __global__ void __launch_bounds__(256)
 grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
                          bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
@@ -72,21 +72,59 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // A stage is U steps of 32 along K.  Two register sets take turns: while the matrix cores work
+  // on one stage the loads of the next are already under way (the loop is memory-latency bound
+  // otherwise: one round trip per stage and wave).
   const int k_begin = wave * (K / 4);
   const int k_end = k_begin + K / 4;
+  if constexpr (U == 0) {
+    // tall tiles: registers go to accumulators; one step at a time, the compiler overlaps what it can
 #pragma unroll 2
-  for (int k = k_begin; k < k_end; k += 32) {
-    uint4 af[NBT], bf[MB];
+    for (int k = k_begin; k < k_end; k += 32) {
+      uint4 af[NBT], bf[MB];
 #pragma unroll
-    for (int nb = 0; nb < NBT; ++nb) af[nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + k);
+      for (int nb = 0; nb < NBT; ++nb) af[nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + k);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) bf[mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k);
+      for (int mb = 0; mb < MB; ++mb) bf[mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k);
 #pragma unroll
-    for (int nb = 0; nb < NBT; ++nb)
+      for (int nb = 0; nb < NBT; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            __builtin_bit_cast(bf16x8, af[nb]), __builtin_bit_cast(bf16x8, bf[mb]), acc[nb][mb], 0, 0, 0);
+        for (int mb = 0; mb < MB; ++mb)
+          acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, af[nb]), __builtin_bit_cast(bf16x8, bf[mb]), acc[nb][mb], 0, 0, 0);
+    }
+  } else {
+  constexpr int STAGE = 32 * (U == 0 ? 1 : U);
+  constexpr int UU = U == 0 ? 1 : U;
+  uint4 a0[UU][NBT], b0[UU][MB], a1[UU][NBT], b1[UU][MB];
+  auto load_stage = [&](uint4 (&af)[UU][NBT], uint4 (&bf)[UU][MB], int k) {
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+#pragma unroll
+      for (int nb = 0; nb < NBT; ++nb) af[u][nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + k + 32 * u);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) bf[u][mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k + 32 * u);
+    }
+  };
+  auto run_stage = [&](const uint4 (&af)[UU][NBT], const uint4 (&bf)[UU][MB]) {
+#pragma unroll
+    for (int u = 0; u < UU; ++u)
+#pragma unroll
+      for (int nb = 0; nb < NBT; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, af[u][nb]), __builtin_bit_cast(bf16x8, bf[u][mb]), acc[nb][mb], 0, 0, 0);
+  };
+  load_stage(a0, b0, k_begin);
+  for (int k = k_begin; k < k_end; k += 2 * STAGE) {
+    const bool more1 = k + STAGE < k_end;
+    if (more1) load_stage(a1, b1, k + STAGE);
+    run_stage(a0, b0);
+    if (!more1) break;
+    if (k + 2 * STAGE < k_end) load_stage(a0, b0, k + 2 * STAGE);
+    run_stage(a1, b1);
+  }
   }
 
   // lane (kgroup, col) holds, for i < 4, the sum for weight row 4 * kgroup + i and activation row col
@@ -145,14 +183,37 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     }
 }
 
+template <int MODE, int MB, int NB, int U>
+static void launch_u(const void* in, const void* w, void* out, const int32_t* sorted,
+                   const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
+                   int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
+  dim3 grid(N / (16 * NB), max_tiles);
+  grouped_gemm_mfma_kernel<MODE, MB, NB, U><<<grid, 256, 0, stream>>>(
+      static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
+      tile_expert, counters, route_weight, assignments, top_k, N, K);
+}
+
+// steps of 32 per stage: as many as divide a wave's quarter of K, fewer for taller tiles (registers)
 template <int MODE, int MB, int NB>
 static void launch(const void* in, const void* w, void* out, const int32_t* sorted,
                    const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
                    int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
-  dim3 grid(N / (16 * NB), max_tiles);
-  grouped_gemm_mfma_kernel<MODE, MB, NB><<<grid, 256, 0, stream>>>(
-      static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
-      tile_expert, counters, route_weight, assignments, top_k, N, K);
+  constexpr int UMAX = MB == 1 ? 4 : (MB == 2 ? 2 : 0);
+  const int quarter = K / 4;
+  if (UMAX == 0) {
+    launch_u<MODE, MB, NB, 0>(in, w, out, sorted, tile_expert, counters, route_weight, assignments, top_k,
+                              N, K, max_tiles, stream);
+    return;
+  }
+  if (UMAX >= 4 && quarter % 128 == 0)
+    launch_u<MODE, MB, NB, UMAX >= 4 ? 4 : 1>(in, w, out, sorted, tile_expert, counters, route_weight,
+                                              assignments, top_k, N, K, max_tiles, stream);
+  else if (UMAX >= 2 && quarter % 64 == 0)
+    launch_u<MODE, MB, NB, UMAX >= 2 ? 2 : 1>(in, w, out, sorted, tile_expert, counters, route_weight,
+                                              assignments, top_k, N, K, max_tiles, stream);
+  else
+    launch_u<MODE, MB, NB, 1>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
+                              top_k, N, K, max_tiles, stream);
 }
 
 // tile_rows: 16, 32 or 64 (the alignment the sorted list was built with); col_blocks: 1 or 2.

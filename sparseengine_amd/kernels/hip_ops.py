@@ -321,7 +321,7 @@ class HipKernels:
             _ptr(ws.counters), _stream()), "moe_align")
         return max_tiles
 
-    def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace):
+    def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, tile_rows=None, wide=None):
         """``out[t] = sum_k weights[t,k] * W2_e(silu(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``;
         ``w13 [E, 2I, h]`` holds gate rows then up rows, ``w2 [E, h, I]``."""
         tokens, hidden = x.shape
@@ -341,12 +341,14 @@ class HipKernels:
             # matrix-core path: tiles as tall as an expert's usual share of the step, blocks as wide
             # as still leaves enough workgroups for the whole chip
             share = assignments / min(experts, assignments)
-            tile_rows = 16 if share <= 16 else 32 if share <= 32 else 64
+            if tile_rows is None:
+                tile_rows = 16 if share <= 16 else 32 if share <= 32 else 64
             max_tiles = self.moe_align(ids, experts, ws, tile_rows)
             if max_tiles > 65535:
                 raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
             gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
-            wide = 2 if max_tiles * (inter // 32) >= 2048 else 1
+            if wide is None:
+                wide = 2 if max_tiles * (inter // 32) >= 2048 else 1
             _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                       _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
                       wide, _stream()), "moe gate-up (mfma)")

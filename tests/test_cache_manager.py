@@ -1,0 +1,162 @@
+"""The cache manager: no page lost, none held twice, none freed twice, under random orders of
+requests; pages come back at the end of a request and when a window has passed them."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from sparseengine_amd.cache.manager import CacheManager, OutOfRows
+from sparseengine_amd.cache.page_pool import OutOfPages, PageOwnershipError, PagePool
+from sparseengine_amd.parts.base import PagedKVRequest, StateRequest
+
+FULL = PagedKVRequest(2, 16, None)
+WINDOW = PagedKVRequest(2, 16, 40)
+
+
+def manager(requests, pages, rows=4, page_size=16, max_len=512, tensors=False):
+    return CacheManager(requests, max_rows=rows, max_model_len=max_len, page_size=page_size, num_pages=pages,
+                        dtype=torch.float32, device="cpu", allocate_tensors=tensors)
+
+
+def test_page_pool_ownership():
+    pool = PagePool(4)
+    a = pool.allocate(3, owner=0)
+    assert sorted(a) == [0, 1, 2] and pool.free_count == 1
+    with pytest.raises(OutOfPages):
+        pool.allocate(2, owner=1)
+    assert pool.free_count == 1                                 # a refused allocation changes nothing
+    with pytest.raises(PageOwnershipError, match="owned by row 0"):
+        pool.release([a[0]], owner=1)
+    pool.release(a[:2], owner=0)
+    with pytest.raises(PageOwnershipError, match="freed twice"):
+        pool.release([a[0]], owner=0)
+    with pytest.raises(PageOwnershipError, match="twice in one release"):
+        pool.release([a[2], a[2]], owner=0)
+    assert pool.allocate(1, owner=5) == [a[1]]                  # the page given back last is used again first
+    pool.check()
+
+
+def test_append_is_all_or_nothing_and_slots_follow_the_table():
+    m = manager({0: FULL, 1: FULL}, pages=6)
+    r0, r1 = m.admit("a"), m.admit("b")
+    alloc = m.append([(r0, 20), (r1, 5)])
+    group = m.groups[0]
+    assert m.group_of_position == {0: 0, 1: 0} and len(m.groups) == 1     # same geometry: one group, one table
+    slots = alloc.slots[0]
+    pages0 = group.table[r0, :2]
+    assert slots[:16].tolist() == [pages0[0] * 16 + i for i in range(16)]
+    assert slots[16:20].tolist() == [pages0[1] * 16 + i for i in range(4)]
+    assert slots[20:].tolist() == [group.table[r1, 0] * 16 + i for i in range(5)]
+    before = (group.table.copy(), m.row_len.copy(), group.pool.free_count)
+    with pytest.raises(OutOfPages):
+        m.append([(r0, 12), (r1, 60)])                          # 0 + 4 pages wanted, 3 free
+    assert (group.table == before[0]).all() and (m.row_len == before[1]).all() and group.pool.free_count == before[2]
+    assert m.can_append([(r0, 12), (r1, 43)]) and not m.can_append([(r0, 13), (r1, 43 + 16)])
+    m.append([(r0, 12), (r1, 43)])                              # exactly fills what is left
+    m.check_invariants()
+    with pytest.raises(ValueError, match="twice"):
+        m.append([(r0, 1), (r0, 1)])
+    m.free("a")
+    with pytest.raises(PageOwnershipError, match="holds no row"):
+        m.free("a")
+    m.free("b")
+    assert group.pool.free_count == 6 and m.num_free_rows == 4
+    m.check_invariants()
+
+
+def test_rows_run_out_and_come_back():
+    m = manager({0: FULL}, pages=8, rows=2)
+    m.admit(1); m.admit(2)
+    with pytest.raises(OutOfRows):
+        m.admit(3)
+    with pytest.raises(ValueError, match="already holds"):
+        m.admit(1)
+    m.free(1)
+    assert m.admit(3) in (0, 1)
+    short = manager({0: FULL}, pages=100, max_len=32)
+    with pytest.raises(ValueError, match="max_model_len"):
+        short.append([(short.admit("x"), 33)])
+
+
+def test_groups_have_pools_of_their_own_and_windows_give_pages_back():
+    m = manager({0: FULL, 1: WINDOW, 2: FULL, 3: WINDOW}, pages={0: 40, 1: 6})
+    assert [g.positions for g in m.groups] == [[0, 2], [1, 3]]
+    row = m.admit("r")
+    held = []
+    for step in range(30):                                      # 300 tokens through a window of 40
+        m.append([(row, 10)])
+        m.check_invariants()
+        held.append(6 - m.groups[1].pool.free_count)
+    assert m.groups[0].pool.free_count == 40 - 19               # the full group keeps ceil(300 / 16) pages
+    assert max(held) <= 4                                       # window 40 + step 10 never needs more than 4 pages of 16
+    table = m.groups[1].table[row]
+    live = np.nonzero(table >= 0)[0]
+    assert live.tolist() == list(range(int(m.groups[1].first_live[row]), 19))
+    # every key a coming query may still read is held: the next query sits at 300 and reads keys >= 261
+    assert int(m.groups[1].first_live[row]) * 16 <= 261
+    m.free("r")
+    assert m.groups[1].pool.free_count == 6
+
+
+def test_state_slots_are_zeroed_on_admission():
+    m = manager({0: FULL, 1: StateRequest((("s", (3, 2), None), ("count", (1,), torch.int32)))}, pages=4, tensors=True)
+    row = m.admit("a")
+    m.state[1]["s"][row] += 5
+    m.state[1]["count"][row] += 2
+    m.free("a")
+    m.admit("b")
+    assert float(m.state[1]["s"][m.row_of("b")].abs().sum()) == 0 and int(m.state[1]["count"][m.row_of("b")]) == 0
+    assert m.state[1]["s"].shape == (4, 3, 2) and m.state[1]["count"].dtype == torch.int32
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_every_page_accounted_for(seed):
+    rng = random.Random(seed)
+    windowed = seed % 2 == 1
+    requests = {0: FULL, 1: WINDOW if windowed else FULL, 2: StateRequest((("h", (4,), None),))}
+    m = manager(requests, pages={0: 24, 1: 9} if windowed else 24, rows=5, max_len=200, tensors=False)
+    live, next_id, reference = {}, 0, {}
+    for _ in range(600):
+        action = rng.random()
+        if action < 0.25 and m.num_free_rows:
+            live[next_id] = m.admit(next_id)
+            reference[next_id] = 0
+            next_id += 1
+        elif action < 0.85 and live:
+            chosen = rng.sample(sorted(live), rng.randint(1, len(live)))
+            items = [(live[r], rng.choice([1, 1, 2, 7, 16, 33])) for r in chosen]
+            items = [(row, n) for (row, n), r in zip(items, chosen) if reference[r] + n <= 200]
+            if not items:
+                continue
+            if m.can_append(items):
+                alloc = m.append(items)
+                for row, n in items:
+                    rid = m.row_owner[row]
+                    reference[rid] += n
+                for slots in alloc.slots.values():
+                    assert len(set(slots.tolist())) == len(slots)          # no two tokens share a slot
+            else:
+                with pytest.raises(OutOfPages):
+                    m.append(items)
+        elif live:
+            rid = rng.choice(sorted(live))
+            m.free(rid)
+            del live[rid], reference[rid]
+        m.check_invariants()
+        for rid, row in live.items():
+            assert int(m.row_len[row]) == reference[rid]
+    for rid in list(live):
+        m.free(rid)
+    m.check_invariants()
+    assert all(g.pool.free_count == g.pool.num_pages for g in m.groups) and m.num_free_rows == 5
+
+
+def test_truncate_undoes_an_append():
+    m = manager({0: FULL}, pages=5)
+    row = m.admit("a")
+    m.append([(row, 20)])
+    m.append([(row, 30)])
+    m.truncate(row, 20)
+    m.check_invariants()
+    assert m.groups[0].pool.free_count == 3 and int(m.row_len[row]) == 20

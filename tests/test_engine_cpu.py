@@ -1,0 +1,196 @@
+"""The engine's host side (batches, cache, step function, replay, scheduler, entry point) on the
+CPU: the kernel twins stand in for the HIP kernels, everything else is the product's own code.
+The kernels themselves are tested on the GPU."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+from sparseengine_amd import LLM, SamplingParams
+from sparseengine_amd.engine.replay import replay_step, replay_stream
+from sparseengine_amd.engine.runner import ModelRunner, StepEntry
+from sparseengine_amd.cache.page_pool import OutOfPages
+from sparseengine_amd.kernels.attention_work import build_attention_work
+from tests import traces
+from tests.helpers import CONFIGS, make_folder, random_tokens
+from tests.plain.minimax_m2 import PlainMiniMaxM2
+from tests.twin_kernels import TwinKernels
+
+LENGTHS = {"A": [5, 17, 31, 100, 64, 129], "B": [1, 9, 40, 100, 200]}
+
+
+@pytest.fixture(scope="module", params=["A_loud", "B_loud"])
+def model(request, tmp_path_factory):
+    key = request.param
+    folder = make_folder(tmp_path_factory.mktemp("cpu_models"), key)
+    vocab = CONFIGS[key][0]["vocab_size"]
+    requests = {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate(LENGTHS[key[0]])}
+    plain = PlainMiniMaxM2(folder)
+    return folder, requests, {rid: plain.logits(t).numpy() for rid, t in requests.items()}, plain
+
+
+def runner_for(folder, tokens, page_size=16, rows=4, dtype="float32"):
+    return ModelRunner.from_folder(folder, dtype=dtype, device="cpu", kv_page_size=page_size,
+                                   num_kvcache_tokens=-(-tokens // 64) * 64, max_num_seqs=rows, kernels=TwinKernels())
+
+
+def replay(folder, records, tokens, page_size=16):
+    runner = runner_for(folder, tokens, page_size)
+    out = {}
+    for rec in records:
+        logits = replay_step(runner, rec, None)
+        if logits is not None:
+            out[rec["step"]] = logits
+        runner.cache.check_invariants()
+    assert all(g.pool.free_count == g.pool.num_pages for g in runner.cache.groups) and runner.cache.num_free_rows == 4
+    return traces.gather(records, out)
+
+
+@pytest.mark.parametrize("mode", ["whole", "tail", "portions", "mixed"])
+def test_every_way_of_cutting_gives_the_plain_logits(model, mode):
+    folder, requests, expected, _ = model
+    if mode == "whole":
+        records, peak = traces.whole(requests), 256
+    elif mode == "tail":
+        records, peak = traces.prefill_then_decode(requests, tail=32), 256
+    elif mode == "portions":
+        records, peak = traces.changing_portions(requests, seed=1), 256
+    else:
+        records, peak = traces.mixed(requests, seed=0)
+        assert peak < sum(-(-len(t) // 64) * 64 for t in requests.values())      # pages must be used again
+    got = replay(folder, records, peak)
+    for rid, ref in expected.items():
+        assert np.abs(got[rid] - ref).max() < 2e-5 * max(1.0, np.abs(ref).max()), rid
+
+
+def test_step_refuses_what_does_not_fit_and_changes_nothing(model):
+    folder, requests, _, _ = model
+    runner = runner_for(folder, 64)
+    toks = requests["r3"]
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("big", toks[:100], [])])
+    assert not runner.cache.has_row("big") and runner.cache.num_free_rows == 4
+    runner.step([StepEntry("ok", toks[:60], [])])
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("ok", toks[60:70], []), StepEntry("other", toks[:3], [])])
+    assert int(runner.cache.row_len[runner.cache.row_of("ok")]) == 60 and not runner.cache.has_row("other")
+    with pytest.raises(ValueError, match="vocabulary"):
+        runner.step([StepEntry("ok", [10 ** 6], [])])
+    runner.cache.check_invariants()
+
+
+def test_trace_stream_writes_files_and_done_lines(model, tmp_path):
+    folder, requests, expected, _ = model
+    records, peak = traces.mixed(requests, seed=5)
+    runner = runner_for(folder, peak)
+
+    class Report(list):
+        def write(self, text): self.append(text)
+        def flush(self): pass
+    report = Report()
+    steps = replay_stream(runner, (json.dumps(r) for r in records), str(tmp_path / "out"), report=report)
+    assert steps == len(records)
+    assert [l.strip() for l in "".join(report).splitlines()] == [f"done {r['step']}" for r in records]
+    vocab = next(iter(expected.values())).shape[1]
+    logits = {r["step"]: np.fromfile(tmp_path / "out" / f"{r['step']}.f32", dtype="<f4").reshape(-1, vocab)
+              for r in records if any(e["want"] for e in r["entries"])}
+    got = traces.gather(records, logits)
+    for rid, ref in expected.items():
+        assert np.abs(got[rid] - ref).max() < 2e-5 * max(1.0, np.abs(ref).max())
+
+
+def llm(folder, **kw):
+    opts = dict(dtype="float32", num_kvcache_slots=512, kv_page_size=16, max_num_seqs_in_batch=4,
+                validate_runtime_invariants=True, _kernels=TwinKernels(), _device="cpu")
+    opts.update(kw)
+    return LLM(folder, **opts)
+
+
+def test_generate_is_the_plain_greedy_decoding(model):
+    folder, requests, _, plain = model
+    prompts = [t[:n] for t, n in zip(requests.values(), (5, 17, 31))]
+    engine = llm(folder)
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
+    assert [o["token_ids"] for o in outs] == [plain.greedy(p, 8) for p in prompts]
+    assert all(o["text"] == "" for o in outs)                       # no tokenizer in a random folder
+    with pytest.raises(ValueError, match="exceeds max_model_len"):
+        engine.add_request(prompts[0], SamplingParams(max_tokens=10 ** 6))
+    with pytest.raises(ValueError, match="unknown configuration keys"):
+        LLM(folder, not_an_option=1)
+    with pytest.raises(ValueError, match="tokenizer"):
+        engine.add_request("text", SamplingParams(max_tokens=1))
+
+
+def test_portions_beside_decodes_and_pressure_change_no_token(model):
+    folder, requests, _, plain = model
+    prompts = [t[:n] for t, n in zip(requests.values(), (5, 17, 31, 60))]
+    params = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
+    expected = [plain.greedy(p, 20) for p in prompts]
+    chunked = llm(folder, max_num_batched_tokens=16)                 # 16-token portions beside decodes
+    assert [o["token_ids"] for o in chunked.generate(prompts, params, use_tqdm=False)] == expected
+    tight = llm(folder, num_kvcache_slots=128, decode_reservation_tokens=0)   # 8 pages: somebody must be thrown out
+    assert [o["token_ids"] for o in tight.generate(prompts, params, use_tqdm=False)] == expected
+    assert tight.scheduler.total_preemptions >= 1
+    assert all(g.pool.free_count == g.pool.num_pages for g in tight.runner.cache.groups)
+
+
+def test_sampling_does_not_depend_on_the_batch(model):
+    folder, requests, _, _ = model
+    prompts = [t[:n] for t, n in zip(requests.values(), (5, 17, 31))]
+    engine = llm(folder)
+    sp = SamplingParams(temperature=0.8, top_k=50, top_p=0.9, max_tokens=12, ignore_eos=True, seed=5)
+    alone = engine.generate([prompts[1]], sp, use_tqdm=False)[0]["token_ids"]
+    others = [SamplingParams(temperature=1.3, max_tokens=9, ignore_eos=True, seed=1), sp,
+              SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True)]
+    together = engine.generate(prompts, others, use_tqdm=False)[1]["token_ids"]
+    assert alone == together and len(set(alone)) > 3
+    again = llm(folder, sampler_seed=1).generate([prompts[1]], sp, use_tqdm=False)[0]["token_ids"]
+    assert again != alone                                            # another sampler seed, another draw
+
+
+def test_penalties_logprobs_and_eos(model):
+    folder, requests, _, plain = model
+    prompt = list(requests.values())[2][:20]
+    engine = llm(folder)
+    base = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True, logprobs=3), use_tqdm=False)
+    first = base[0]["token_ids"][0]
+    stopped = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=6, eos_token_ids=[first]), use_tqdm=False)
+    assert stopped[0]["token_ids"] == [first]
+    # a strong presence penalty forbids repeating a generated token
+    pen = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True, presence_penalty=2.0,
+                                                   repetition_penalty=1.5), use_tqdm=False)[0]["token_ids"]
+    free = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True), use_tqdm=False)[0]["token_ids"]
+    assert len(set(pen)) >= len(set(free))
+    engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True, logprobs=2))
+    finished = []
+    while not engine.is_finished():
+        out, count = engine.step()
+        finished += out
+    (_, tokens, logprobs, tops), = finished
+    ref = torch.log_softmax(plain.logits(prompt)[-1], -1)
+    assert logprobs[0] == pytest.approx(float(ref[tokens[0]]), abs=1e-4)
+    assert set(tops[0]) == set(torch.topk(ref, 2).indices.tolist())
+
+
+def test_attention_work_lists_cover_every_row_and_key_once():
+    for q_len, ctx, group, kvh, window in [([1], [2049], 6, 8, 0), ([1] * 64, [2200 - i for i in range(64)], 6, 8, 0),
+                                            ([37, 23, 1], [37, 150, 301], 2, 2, 0), ([2048], [2048], 6, 8, 0),
+                                            ([1, 1], [5000, 300], 4, 1, 128), ([3], [70], 16, 1, 0)]:
+        work = build_attention_work(q_len, ctx, group, kvh, window)
+        units = work.units
+        for item, (ql, c) in enumerate(zip(q_len, ctx)):
+            mine = units[units[:, 0] == item]
+            tiles = -(-ql * group // 16)
+            assert sorted(set(mine[:, 1].tolist())) == list(range(tiles))
+            for tile in range(tiles):
+                ranges = sorted((b, e) for _, t, b, e, *_ in mine.tolist() if t == tile)
+                assert ranges[-1][1] == c and all(b % 32 == 0 for b, _ in ranges)
+                assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:]))        # no gap, no overlap
+                first = ranges[0][0]
+                assert first == 0 or (window and first <= max(0, c - ql - window + 1))
+        split = units[units[:, 4] >= 0]
+        assert sorted(split[:, 4].tolist()) == list(range(work.num_slots))
+        for item, tile, first_slot, n in work.tasks.tolist():
+            slots = sorted(u[4] for u in units.tolist() if u[0] == item and u[1] == tile)
+            assert slots == list(range(first_slot, first_slot + n)) and n <= 256
