@@ -5,13 +5,15 @@
 // written back as the new residual while the norm uses the unrounded sum.
 #include "common.h"
 
-template <typename T>
-__global__ void embedding_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
+// TT: storage of the table, T: storage of the activations (a table kept in float under a
+// bfloat16 engine is rounded on the way out)
+template <typename TT, typename T>
+__global__ void embedding_kernel(const int32_t* __restrict__ ids, const TT* __restrict__ table,
                                  T* __restrict__ out, int hidden) {
   const int64_t row = ids[blockIdx.x];
-  const T* src = table + row * hidden;
+  const TT* src = table + row * hidden;
   T* dst = out + static_cast<int64_t>(blockIdx.x) * hidden;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = src[c];
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = from_float<T>(to_float(src[c]));
 }
 
 // One block per output row.  rows == nullptr: input row = output row = blockIdx.x.
@@ -149,14 +151,19 @@ static int launch_rms(const void* x, void* residual, const void* weight, void* o
 extern "C" {
 
 int se_embedding(const int32_t* ids, const void* table, void* out, int tokens, int hidden,
-                 int dtype, hipStream_t stream) {
+                 int dtype, int table_dtype, hipStream_t stream) {
   if (tokens <= 0) return SE_OK;
-  if (dtype == SE_F32)
-    embedding_kernel<float><<<tokens, 256, 0, stream>>>(ids, static_cast<const float*>(table),
-                                                        static_cast<float*>(out), hidden);
+  if (dtype == SE_F32 && table_dtype == SE_F32)
+    embedding_kernel<float, float><<<tokens, 256, 0, stream>>>(ids, static_cast<const float*>(table),
+                                                               static_cast<float*>(out), hidden);
+  else if (dtype == SE_BF16 && table_dtype == SE_F32)
+    embedding_kernel<float, bf16_t><<<tokens, 256, 0, stream>>>(ids, static_cast<const float*>(table),
+                                                                static_cast<bf16_t*>(out), hidden);
+  else if (dtype == SE_BF16 && table_dtype == SE_BF16)
+    embedding_kernel<bf16_t, bf16_t><<<tokens, 256, 0, stream>>>(ids, static_cast<const bf16_t*>(table),
+                                                                 static_cast<bf16_t*>(out), hidden);
   else
-    embedding_kernel<bf16_t><<<tokens, 256, 0, stream>>>(ids, static_cast<const bf16_t*>(table),
-                                                         static_cast<bf16_t*>(out), hidden);
+    return SE_ERR_SHAPE;
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -54,7 +54,7 @@ def _i32(t: torch.Tensor, name: str):
 
 _SIGNATURES = {
     "norm": {
-        "se_embedding": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "se_embedding": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "se_rms_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
                         c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p],
     },
@@ -159,10 +159,11 @@ class HipKernels:
     def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor):
         _i32(ids, "ids")
         tokens, hidden = out.shape
-        _require(ids.numel() == tokens and table.shape[1] == hidden and table.dtype == out.dtype
-                 and table.is_contiguous() and out.is_contiguous(), "embedding: shape/dtype mismatch")
+        _require(ids.numel() == tokens and table.shape[1] == hidden and table.is_contiguous()
+                 and out.is_contiguous(), "embedding: shape mismatch")
+        _require(table.dtype == out.dtype or table.dtype == torch.float32, "embedding: table dtype")
         _check(_fn.get("norm", "se_embedding")(_ptr(ids), _ptr(table), _ptr(out), tokens, hidden,
-                                               _code(out.dtype), _stream()), "embedding")
+                                               _code(out.dtype), _code(table.dtype), _stream()), "embedding")
 
     def rms_norm(self, x, weight, eps: float, out, residual=None, rows=None, write_residual=True):
         """``out = norm(x (+ residual)) * weight``; with ``residual`` the rounded sum replaces it

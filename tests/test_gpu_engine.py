@@ -1,0 +1,285 @@
+"""The engine on the GPU beyond replay: long decoding, the first tokens of a sequence, greedy
+generation through the entry point, weights kept in 32-bit under a bfloat16 engine, each part
+alone, and a toy architecture (defined in the tests) with a recurrent mixer, a windowed cache
+group, a dense feed-forward, a layer that runs twice and a shared cache."""
+import os
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from tests import traces
+from tests.helpers import CONFIGS, make_folder, random_tokens
+from tests.plain import minimax_m2 as P
+from tests.plain.minimax_m2 import PlainMiniMaxM2
+
+pytestmark = pytest.mark.gpu
+
+
+def bound(dtype, ref):
+    scale = float(np.abs(ref).max())
+    return 2e-5 * max(scale, 1.0) if dtype == "float32" else 0.04 * scale
+
+
+def runner_for(folder, dtype, tokens=1024, page_size=16, rows=4):
+    from sparseengine_amd.engine.runner import ModelRunner
+    return ModelRunner.from_folder(folder, dtype=dtype, kv_page_size=page_size,
+                                   num_kvcache_tokens=-(-tokens // 64) * 64, max_num_seqs=rows)
+
+
+def replay_with_routing(runner, records):
+    from sparseengine_amd.engine.replay import replay_step
+    out, routing = {}, {}
+    for rec in records:
+        taps = {}
+        logits = replay_step(runner, rec, None, taps=taps)
+        if logits is not None:
+            out[rec["step"]] = logits
+        cursor = 0
+        for e in rec["entries"]:
+            n = len(e["tokens"])
+            layers = routing.setdefault(e["id"], [[] for _ in taps.get("router", [])])
+            for layer, (ids, _) in enumerate(taps.get("router", [])):
+                layers[layer].append(ids[cursor:cursor + n].cpu())
+            cursor += n
+    return traces.gather(records, out), {r: [torch.cat(c).long() for c in layers] for r, layers in routing.items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["B_loud", "A_loud"])
+def test_long_decoding_token_by_token(tmp_path, key, dtype):
+    """A short prompt and then hundreds of single-token steps across many pages."""
+    folder = make_folder(tmp_path, key)
+    raw = CONFIGS[key][0]
+    n = raw["max_position_embeddings"] - 6
+    tokens = random_tokens(n, raw["vocab_size"], 77)
+    records = traces.prefill_then_decode({"long": tokens}, tail=n - 3)
+    runner = runner_for(folder, dtype, tokens=n + 64)
+    got, routing = replay_with_routing(runner, records)
+    plain = PlainMiniMaxM2(folder)
+    ref = plain.logits(tokens, forced_routing=routing["long"] if dtype == "bfloat16" else None).numpy()
+    err = np.abs(got["long"] - ref).max(-1)
+    assert err.max() <= bound(dtype, ref), f"first position over the bound: {int(np.argmax(err > bound(dtype, ref)))}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(tmp_path, dtype):
+    """Positions 0, 1, 2: one key, no prefix, an almost empty page; alone and three requests at once."""
+    folder = make_folder(tmp_path, "B_loud")
+    plain = PlainMiniMaxM2(folder)
+    from sparseengine_amd.engine.runner import StepEntry
+    runner = runner_for(folder, dtype)
+    seqs = {f"s{i}": random_tokens(3, 1000, 200 + i) for i in range(3)}
+    taps = {}
+    logits = runner.step([StepEntry(r, t[:1], [0]) for r, t in seqs.items()], taps=taps).cpu().numpy()
+    for i, (r, t) in enumerate(seqs.items()):
+        forced = [ids[i:i + 1].cpu().long() for ids, _ in taps["router"]] if dtype == "bfloat16" else None
+        ref = plain.logits(t[:1], forced_routing=forced).numpy()
+        assert np.abs(logits[i] - ref[0]).max() <= bound(dtype, ref)
+    taps = {}
+    logits = runner.step([StepEntry(r, t[1:3], [0, 1]) for r, t in seqs.items()], taps=taps).cpu().numpy()
+    if dtype == "float32":
+        for i, (r, t) in enumerate(seqs.items()):
+            ref = plain.logits(t).numpy()
+            assert np.abs(logits[2 * i:2 * i + 2] - ref[1:3]).max() <= bound(dtype, ref)
+
+
+def test_greedy_generation_through_the_entry_point(tmp_path):
+    from sparseengine_amd import LLM, SamplingParams
+    folder = make_folder(tmp_path, "A_loud")
+    plain = PlainMiniMaxM2(folder)
+    prompts = [random_tokens(n, 512, 300 + n) for n in (5, 17, 31, 90)]
+    params = SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True)
+    expected = [plain.greedy(p, 24) for p in prompts]
+    llm = LLM(folder, dtype="float32", num_kvcache_slots=1024, kv_page_size=16, max_num_seqs_in_batch=4,
+              validate_runtime_invariants=True)
+    assert [o["token_ids"] for o in llm.generate(prompts, params, use_tqdm=False)] == expected
+    # portions of 16 tokens beside decodes, and a cache so small that a request is thrown out and recomputed
+    tight = LLM(folder, dtype="float32", num_kvcache_slots=192, kv_page_size=16, max_num_seqs_in_batch=4,
+                max_num_batched_tokens=16, decode_reservation_tokens=0, validate_runtime_invariants=True)
+    assert [o["token_ids"] for o in tight.generate(prompts, params, use_tqdm=False)] == expected
+    assert tight.scheduler.total_preemptions >= 1
+    # bfloat16: every generated token is, for the plain logits of its own context, as good as the best
+    # one up to bfloat16 rounding
+    half = LLM(folder, dtype="bfloat16", num_kvcache_slots=1024, kv_page_size=16, max_num_seqs_in_batch=4)
+    for prompt, out in zip(prompts, half.generate(prompts, params, use_tqdm=False)):
+        ids = out["token_ids"]
+        logits = plain.logits(prompt + ids)[len(prompt) - 1:-1]
+        chosen = logits.gather(1, torch.tensor(ids)[:, None])[:, 0]
+        assert (logits.max(-1).values - chosen).max() <= 2 * 0.04 * float(logits.abs().max())
+    # temperature sampling: the same seed gives the same tokens, alone and in a batch
+    sp = SamplingParams(temperature=0.8, top_k=40, top_p=0.95, max_tokens=12, ignore_eos=True, seed=9)
+    alone = llm.generate([prompts[1]], sp, use_tqdm=False)[0]["token_ids"]
+    mixed = llm.generate(prompts[:3], [params, sp, SamplingParams(temperature=1.2, max_tokens=7, ignore_eos=True)],
+                         use_tqdm=False)[1]["token_ids"]
+    assert alone == mixed
+
+
+def test_weights_stored_in_32_bit_stay_so_under_bfloat16(tmp_path):
+    folder = make_folder(tmp_path, "A_loud")
+    path = os.path.join(folder, "model.safetensors")
+    tensors = {k: v.float() for k, v in load_file(path).items()}         # the whole checkpoint in float32
+    save_file(tensors, path)
+    runner = runner_for(folder, "bfloat16")
+    assert all(p.dtype == torch.float32 for p in runner.params.values())
+    tokens = random_tokens(60, 512, 8)
+    records = traces.changing_portions({"r": tokens}, seed=3)
+    got, routing = replay_with_routing(runner, records)
+    ref = PlainMiniMaxM2(folder).logits(tokens, forced_routing=routing["r"]).numpy()
+    assert np.abs(got["r"] - ref).max() <= bound("bfloat16", ref)
+
+
+# ------------------------------------------------------------------ each part alone
+class Harness:
+    """A cache, a batch builder and a hand-made batch for one part."""
+
+    def __init__(self, dtype, requests=None, pages=32, page_size=16):
+        from sparseengine_amd.cache.manager import CacheManager
+        from sparseengine_amd.engine.batch import BatchBuilder
+        from sparseengine_amd.kernels.hip_ops import HipKernels
+        self.dtype = dtype
+        self.cache = CacheManager(requests or {}, max_rows=4, max_model_len=512, page_size=page_size, num_pages=pages,
+                                  dtype=dtype, device="cuda")
+        self.builder = BatchBuilder(HipKernels(), self.cache, dtype, "cuda", vocab_size=1 << 20)
+
+    def batch(self, lengths):
+        from sparseengine_amd.engine.batch import StepItem
+        items = []
+        for rid, n in lengths:
+            if not self.cache.has_row(rid):
+                self.cache.admit(rid)
+            items.append(StepItem(self.cache.row_of(rid), [0] * n, []))
+        return self.builder.build(items)
+
+
+def materialize(part, dtype, seed, scale=0.1):
+    g = torch.Generator().manual_seed(seed)
+    params = {}
+    for name, decl in part.all_param_decls().items():
+        value = torch.randn(decl.shape, generator=g) * scale
+        if "norm" in name:
+            value = 1 + value
+        params[name] = value.to(torch.float32 if decl.policy == "float32" else dtype).cuda()
+    part.bind_all(params)
+    return {k: v.float().cpu() for k, v in params.items()}
+
+
+def assert_part_close(dtype, got, ref):
+    """float32: float rounding.  bfloat16: the bound of the logits tests, 4 % of the largest value."""
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-4)
+    else:
+        assert float((got - ref).abs().max()) <= 0.04 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from sparseengine_amd.config.specs import NormSpec
+    from sparseengine_amd.parts import NORMS
+    norm = NORMS.build(NormSpec(eps=1e-3), hidden_size=200)
+    w = materialize(norm, dtype, 1)
+    h = Harness(dtype)
+    fb = h.batch([("a", 7)])
+    x = torch.randn(7, 200).to(dtype).cuda()
+    r = torch.randn(7, 200).to(dtype).cuda()
+    x0, r0 = x.float().cpu(), r.float().cpu()
+    norm.forward(fb, x, residual=r)
+    y, merged = P.add_rms_norm(x0, r0, w["weight"], 1e-3)
+    assert_part_close(dtype, x.float().cpu(), y)
+    assert_part_close(dtype, r.float().cpu(), merged)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rotary,norm,window", [(6, 2, 32, 16, "flat", None), (5, 5, 48, 48, "none", 10),
+                                                                        (8, 1, 64, 0, "flat", None)])
+def test_attention_part_in_two_portions(dtype, heads, kv_heads, head_dim, rotary, norm, window):
+    from sparseengine_amd.config.specs import AttentionSpec, NoPositionSpec, RotarySpec
+    from sparseengine_amd.parts import MIXERS
+    position = RotarySpec(rotary_dim=rotary, theta=1e4, max_position=512) if rotary else NoPositionSpec()
+    spec = AttentionSpec(num_heads=heads, num_kv_heads=kv_heads, head_dim=head_dim, scale=head_dim ** -0.5,
+                         qk_norm=norm, qk_norm_eps=1e-5, window=window, position=position)
+    mixer = MIXERS.build(spec, hidden_size=72)
+    w = materialize(mixer, dtype, 2, scale=0.2)
+    h = Harness(dtype, {0: mixer.cache_request()})
+    T, cut = 45, 29
+    x = torch.randn(T, 72).to(dtype)
+    out = torch.cat([mixer.forward(h.batch([("a", cut)]), x[:cut].cuda(), 0).float().cpu(),
+                     mixer.forward(h.batch([("a", T - cut)]), x[cut:].cuda(), 0).float().cpu()])
+    xf = x.float()
+    qkv = xf @ w["qkv"].T
+    q, k, v = qkv[:, :heads * head_dim], qkv[:, heads * head_dim:(heads + kv_heads) * head_dim], qkv[:, (heads + kv_heads) * head_dim:]
+    if norm == "flat":
+        q, k = P.flat_qk_norm(q, w["q_norm"], 1e-5), P.flat_qk_norm(k, w["k_norm"], 1e-5)
+    q, k, v = q.reshape(T, heads, head_dim), k.reshape(T, kv_heads, head_dim), v.reshape(T, kv_heads, head_dim)
+    if rotary:
+        cos, sin = P.rope_angles(torch.arange(T), rotary, 1e4)
+        q, k = P.partial_rope(q, cos, sin, rotary), P.partial_rope(k, cos, sin, rotary)
+    ref = P.causal_gqa_attention(q, k, v, head_dim ** -0.5, window=window).reshape(T, -1) @ w["o"].T
+    assert_part_close(dtype, out, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden,experts,top_k,inter,scoring,bias", [(96, 5, 5, 40, "sigmoid", True), (256, 12, 3, 128, "softmax", False)])
+def test_feed_forward_parts(dtype, hidden, experts, top_k, inter, scoring, bias):
+    from sparseengine_amd.config.specs import DenseMLPSpec, MoESpec
+    from sparseengine_amd.parts import FEED_FORWARDS
+    moe = FEED_FORWARDS.build(MoESpec(num_experts=experts, top_k=top_k, intermediate_size=inter, scoring=scoring,
+                                      selection_bias=bias, norm_topk_prob=bias, routed_scaling_factor=1.0 if bias else 2.0),
+                              hidden_size=hidden, chunk_tokens=16)       # 37 tokens: three chunks, invisible
+    w = materialize(moe, dtype, 3, scale=0.15)
+    h = Harness(dtype)
+    x = torch.randn(37, hidden).to(dtype)
+    fb = h.batch([("a", 37)])
+    fb.taps = {}
+    out = moe.forward(fb, x.cuda()).float().cpu()
+    ids = torch.cat([i for i, _ in fb.taps["router"]]).long().cpu()
+    xf = x.float()
+    scores = torch.sigmoid(xf @ w["router"].T) if scoring == "sigmoid" else torch.softmax(xf @ w["router"].T, -1)
+    wts = scores.gather(1, ids)
+    wts = wts / wts.sum(-1, keepdim=True) if bias else wts * 2.0
+    ref = P.swiglu_experts(xf, w["w13"][:, :inter], w["w13"][:, inter:], w["w2"], ids, wts)
+    assert_part_close(dtype, out, ref)
+    if dtype == torch.float32:       # the choice itself: top-k of score (+ bias)
+        sel = scores + w["router_bias"] if bias else scores
+        assert torch.equal(ids.sort(-1).values, torch.topk(sel, top_k).indices.sort(-1).values)
+    mlp = FEED_FORWARDS.build(DenseMLPSpec(intermediate_size=inter), hidden_size=hidden)
+    w = materialize(mlp, dtype, 4, scale=0.15)
+    out = mlp.forward(h.batch([("b", 37)]), x.cuda()).float().cpu()
+    gu = xf @ w["gate_up"].T
+    assert_part_close(dtype, out, (torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]) @ w["down"].T)
+
+
+# ------------------------------------------------------------------ the toy architecture
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
+    from sparseengine_amd.weights.random_weights import write_model_folder
+    from tests.toy_arch import TOY_CONFIG, PlainToy
+    folder = write_model_folder(str(tmp_path / "toy"), TOY_CONFIG, 3, {"std": 0.15})
+    plain = PlainToy(folder)
+    requests = {f"r{i}": random_tokens(n, 300, 50 + i) for i, n in enumerate([70, 9, 33, 150, 1, 64])}
+    expected = {r: plain.logits(t).numpy() for r, t in requests.items()}
+    records, peak = traces.mixed(requests, seed=1)
+    runner = runner_for(folder, dtype, tokens=peak)
+    assert [(g.request.window, g.positions) for g in runner.cache.groups] == [(None, [0, 3]), (24, [2])]
+    assert list(runner.cache.state_positions) == [1]
+    from sparseengine_amd.engine.replay import replay_step
+    out = {}
+    for rec in records:
+        logits = replay_step(runner, rec, None)
+        if logits is not None:
+            out[rec["step"]] = logits
+        runner.cache.check_invariants()
+    got = traces.gather(records, out)
+    if dtype == "float32":
+        for rid, ref in expected.items():
+            assert np.abs(got[rid] - ref).max() <= bound(dtype, ref), rid
+    else:   # routed layers may tip in bfloat16: most positions must agree, and every request's first ones
+        close = total = 0
+        for rid, ref in expected.items():
+            err = np.abs(got[rid] - ref).max(-1)
+            close += int((err <= bound(dtype, ref)).sum()); total += len(err)
+        assert close >= 0.8 * total
+    assert all(g.pool.free_count == g.pool.num_pages for g in runner.cache.groups)
+    windowed = runner.cache.groups[1]
+    assert windowed.pool.num_pages >= 4      # and a window of 24 never held more than 4 pages of 16 per request

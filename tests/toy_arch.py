@@ -1,0 +1,189 @@
+"""A toy architecture defined wholly in the tests, to show that parts, cache groups, state slots
+and the run order are general: layers differ in mixer (full attention, windowed attention, a
+recurrent mixer with state of its own) and in feed-forward (dense, routed), the schedule runs a
+layer twice and lets one position read another position's cache.  Nothing in ``sparseengine_amd``
+knows about it: it registers itself through the public registries.  It is no model of anyone's.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import ClassVar
+
+import torch
+
+from sparseengine_amd.config.registry import Architecture, WeightSource, register_architecture
+from sparseengine_amd.config.specs import (AttentionSpec, DenseMLPSpec, LayerSpec, ModelSpec, MoESpec, NoPositionSpec,
+                                           NormSpec, RotarySpec, ScheduleEntry)
+from sparseengine_amd.parts import MIXERS, ParamDecl, Part, StateRequest, build_model
+from tests.plain import minimax_m2 as P
+
+
+# ------------------------------------------------------------------ a mixer with state of its own
+@dataclass(frozen=True)
+class DecayMixerSpec:
+    kind: ClassVar[str] = "toy_decay"
+    state_size: int = 8
+    decay: float = 0.9
+
+
+class DecayMixer(Part):
+    """``s_t = decay * s_{t-1} + W_in x_t``; ``y_t = W_out s_t``; the state is float32 and per request."""
+
+    def __init__(self, spec: DecayMixerSpec, hidden_size: int):
+        self.spec, self.hidden_size = spec, hidden_size
+
+    def param_decls(self):
+        return {"w_in": ParamDecl((self.spec.state_size, self.hidden_size)),
+                "w_out": ParamDecl((self.hidden_size, self.spec.state_size))}
+
+    def cache_request(self):
+        return StateRequest((("s", (self.spec.state_size,), torch.float32),))
+
+    def forward(self, fb, x, cache_position, write_cache=True):
+        state = fb.state_view(cache_position)["s"]
+        w_in, w_out = self.params["w_in"].float(), self.params["w_out"].float()
+        out = torch.empty_like(x)
+        meta = next(iter(fb.groups.values())) if fb.groups else None
+        starts = meta.item_q_start if meta is not None else fb.toy_q_start
+        lens = meta.item_q_len if meta is not None else fb.toy_q_len
+        for row, start, n in zip(fb.item_rows_host.tolist(), starts.tolist(), lens.tolist()):
+            s = state[row].clone()
+            for t in range(start, start + n):          # a portion's tokens, in order
+                s = self.spec.decay * s + w_in @ x[t].float()
+                out[t] = (w_out @ s).to(x.dtype)
+            if write_cache:
+                state[row] = s
+        return out
+
+
+MIXERS.register("toy_decay", lambda spec, hidden_size: DecayMixer(spec, hidden_size))
+
+
+# ------------------------------------------------------------------ the architecture
+def parse(raw: dict) -> dict:
+    return raw
+
+
+def _layer_spec(cfg, layer) -> LayerSpec:
+    h = cfg["hidden_size"]
+    if layer["mixer"] == "decay":
+        mixer = DecayMixerSpec(state_size=layer["state_size"], decay=layer["decay"])
+    else:
+        rotary = (RotarySpec(rotary_dim=layer["rotary_dim"], theta=cfg["rope_theta"],
+                             max_position=cfg["max_position_embeddings"]) if layer["rotary_dim"] else NoPositionSpec())
+        mixer = AttentionSpec(num_heads=layer["heads"], num_kv_heads=layer["kv_heads"], head_dim=layer["head_dim"],
+                              scale=layer["head_dim"] ** -0.5, qk_norm="flat" if layer.get("qk_norm") else "none",
+                              qk_norm_eps=cfg["eps"], window=layer.get("window"), position=rotary)
+    if layer["ffn"] == "dense":
+        ffn = DenseMLPSpec(intermediate_size=layer["intermediate"])
+    else:
+        ffn = MoESpec(num_experts=layer["experts"], top_k=layer["top_k"], intermediate_size=layer["intermediate"],
+                      scoring=layer.get("scoring", "sigmoid"), selection_bias=layer.get("bias", True),
+                      norm_topk_prob=layer.get("normalize", True), routed_scaling_factor=layer.get("scaling", 1.0))
+    return LayerSpec(mixer=mixer, feed_forward=ffn, norm=NormSpec(eps=cfg["eps"]))
+
+
+def build_spec(cfg) -> ModelSpec:
+    layers = tuple(_layer_spec(cfg, layer) for layer in cfg["layers"])
+    schedule = tuple(ScheduleEntry(e["layer"], e.get("cache_from")) for e in cfg["schedule"])
+    return ModelSpec(architecture="ToyForCausalLM", hidden_size=cfg["hidden_size"], vocab_size=cfg["vocab_size"],
+                     layers=layers, schedule=schedule, final_norm=NormSpec(eps=cfg["eps"]),
+                     max_position=cfg["max_position_embeddings"])
+
+
+def weight_sources(cfg):
+    """Checkpoint names are the parameter paths with a ``toy.`` prefix, tensor for tensor."""
+    return [WeightSource("toy." + path, path) for path in build_model(build_spec(cfg)).all_param_decls()]
+
+
+def random_tensor(cfg, name, shape, generator, options):
+    noise = torch.randn(tuple(shape), generator=generator, dtype=torch.float32, device=generator.device)
+    if "norm" in name and name.endswith("weight"):
+        return 1.0 + 0.2 * noise
+    if name.endswith("router_bias"):
+        return 0.3 * noise
+    return noise * float(options.get("std", 0.1))
+
+
+TOY = register_architecture(Architecture(
+    name="ToyForCausalLM", model_types=("toy",), parse_config=parse, build_spec=build_spec,
+    weight_sources=weight_sources, ignored_tensor=lambda name: False, random_tensor=random_tensor,
+    stored_dtype=lambda name: "float32" if name.endswith(("router", "router_bias")) else "bfloat16",
+    config_to_dict=lambda cfg: dict(cfg)))
+
+TOY_CONFIG = dict(
+    architectures=["ToyForCausalLM"], model_type="toy", hidden_size=64, vocab_size=300, eps=1e-5, rope_theta=10000.0,
+    max_position_embeddings=1024,
+    layers=[
+        dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=16, qk_norm=True, ffn="dense", intermediate=96),
+        dict(mixer="decay", state_size=12, decay=0.8, ffn="moe", experts=6, top_k=2, intermediate=40, scoring="softmax",
+             bias=False, normalize=False, scaling=1.5),
+        dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, ffn="moe", experts=4, top_k=3,
+             intermediate=24),
+        dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, ffn="dense", intermediate=48),
+    ],
+    # layer 0 runs twice (two caches); the last position reads the cache of position 0 (same geometry)
+    schedule=[dict(layer=0), dict(layer=1), dict(layer=2), dict(layer=0), dict(layer=3, cache_from=0)])
+
+
+# ------------------------------------------------------------------ its plain implementation
+class PlainToy:
+    def __init__(self, folder: str):
+        import json, os
+        from safetensors.torch import load_file
+        self.cfg = json.load(open(os.path.join(folder, "config.json")))
+        self.w = {k[4:]: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+
+    def logits(self, tokens):
+        cfg, w = self.cfg, self.w
+        T = len(tokens)
+        pos = torch.arange(T)
+        x = w["embed.weight"][torch.as_tensor(tokens)]
+        residual = None
+        kv_of = {}
+        for position, entry in enumerate(cfg["schedule"]):
+            i, layer = entry["layer"], cfg["layers"][entry["layer"]]
+            p = f"layers.{i}."
+            if residual is None:
+                residual, u = x, P.rms_norm(x, w[p + "norm_mixer.weight"], cfg["eps"])
+            else:
+                u, residual = P.add_rms_norm(x, residual, w[p + "norm_mixer.weight"], cfg["eps"])
+            if layer["mixer"] == "decay":
+                s = torch.zeros(layer["state_size"])
+                a = torch.empty_like(u)
+                for t in range(T):
+                    s = layer["decay"] * s + w[p + "mixer.w_in"] @ u[t]
+                    a[t] = w[p + "mixer.w_out"] @ s
+            else:
+                H, Hkv, D, R = layer["heads"], layer["kv_heads"], layer["head_dim"], layer["rotary_dim"]
+                qkv = u @ w[p + "mixer.qkv"].T
+                q, k, v = qkv[:, :H * D], qkv[:, H * D:(H + Hkv) * D], qkv[:, (H + Hkv) * D:]
+                if layer.get("qk_norm"):
+                    q = P.flat_qk_norm(q, w[p + "mixer.q_norm"], cfg["eps"])
+                    k = P.flat_qk_norm(k, w[p + "mixer.k_norm"], cfg["eps"])
+                q, k, v = q.reshape(T, H, D), k.reshape(T, Hkv, D), v.reshape(T, Hkv, D)
+                if R:
+                    cos, sin = P.rope_angles(pos, R, cfg["rope_theta"])
+                    q, k = P.partial_rope(q, cos, sin, R), P.partial_rope(k, cos, sin, R)
+                if entry.get("cache_from") is not None:
+                    k, v = kv_of[entry["cache_from"]]            # reads another position's keys and values
+                else:
+                    kv_of[position] = (k, v)
+                a = P.causal_gqa_attention(q, k, v, D ** -0.5, window=layer.get("window")).reshape(T, -1) @ w[p + "mixer.o"].T
+            m, residual = P.add_rms_norm(a, residual, w[p + "norm_ffn.weight"], cfg["eps"])
+            I = layer["intermediate"]
+            if layer["ffn"] == "dense":
+                gu = m @ w[p + "ffn.gate_up"].T
+                x = (torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]) @ w[p + "ffn.down"].T
+            else:
+                logits = m @ w[p + "ffn.router"].T
+                scores = torch.softmax(logits, -1) if layer.get("scoring") == "softmax" else torch.sigmoid(logits)
+                sel = scores + w[p + "ffn.router_bias"] if layer.get("bias", True) else scores
+                ids = torch.topk(sel, layer["top_k"], dim=-1).indices
+                wts = scores.gather(1, ids)
+                if layer.get("normalize", True):
+                    wts = wts / wts.sum(-1, keepdim=True)
+                wts = wts * layer.get("scaling", 1.0)
+                x = P.swiglu_experts(m, w[p + "ffn.w13"][:, :I], w[p + "ffn.w13"][:, I:], w[p + "ffn.w2"], ids, wts)
+        y, _ = P.add_rms_norm(x, residual, w["final_norm.weight"], cfg["eps"])
+        return y @ w["head.weight"].T

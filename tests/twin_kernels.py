@@ -29,7 +29,7 @@ class TwinKernels:
 
     # ------------------------------------------------------------------ embedding / norms
     def embedding(self, ids, table, out):
-        out.copy_(table[ids.long()])
+        out.copy_(table[ids.long()])        # a float table under bfloat16 activations is rounded here
 
     def rms_norm(self, x, weight, eps, out, residual=None, rows=None, write_residual=True):
         z = x.float()
