@@ -11,6 +11,8 @@
 //       out[a, n] = silu(g) * u; g and u are rounded to bfloat16, silu is taken in float and
 //       rounded, the product is rounded.
 //   MODE 1 (down): in row = act[a]; w = w2[e], [N, K]; out[a, n] = (in . w[n]) * route_weight[a].
+//   MODE 2 (dense, few rows): out[t, n] = x[t] . w[n] for one weight matrix [N, K]; tile t holds rows
+//       16 * MB * t ...; the same streaming loop serves the skinny projections of decode steps.
 //
 // Every output element is one dot product in a fixed order of K, so a row's result does not
 // depend on its place in the tile or on what else is in the batch.
@@ -32,7 +34,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   constexpr int BN = 16 * NB;
   constexpr int NBT = MODE == 0 ? 2 * NB : NB;  // weight blocks per wave: gate blocks, then up blocks
   const int tile = blockIdx.y;
-  if (tile >= counters[0]) return;  // uniform over the block
+  if (MODE != 2 && tile >= counters[0]) return;  // uniform over the block
 
   constexpr int P = NB * MB;                   // output blocks of 16 x 16 (gate/up pairs in MODE 0)
   constexpr int PARTS = MODE == 0 ? 2 : 1;
@@ -42,9 +44,10 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 
   const int lane = threadIdx.x & (SE_WAVE - 1);
   const int wave = threadIdx.x / SE_WAVE;
-  const int expert = tile_expert[tile];
+  const int expert = MODE == 2 ? 0 : tile_expert[tile];
   const int n0 = blockIdx.x * BN;
-  if (threadIdx.x < BM) rows[threadIdx.x] = sorted[tile * BM + threadIdx.x];
+  if (threadIdx.x < BM)
+    rows[threadIdx.x] = MODE == 2 ? tile * BM + static_cast<int>(threadIdx.x) : sorted[tile * BM + threadIdx.x];
   __syncthreads();
 
   const int col = lane & 15;   // row of the weight block (A) / row of the activation block (B)
@@ -171,8 +174,10 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
           const float up = round_to<bf16_t>(total[PARTS - 1][i]);
           const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
           v = act * up;
-        } else {
+        } else if (MODE == 1) {
           v = total[0][i] * route_weight[a];
+        } else {
+          v = total[0][i];
         }
         y[i] = float_to_bf16_bits(v);
       }
@@ -214,6 +219,21 @@ static void launch(const void* in, const void* w, void* out, const int32_t* sort
   else
     launch_u<MODE, MB, NB, 1>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
                               top_k, N, K, max_tiles, stream);
+}
+
+// Dense product of a few rows: out[rows, N] = x[rows, K] . w[N, K]^T (bfloat16, float accumulate).
+extern "C" int se_skinny_gemm_mfma(const void* x, const void* w, void* out, int rows, int N, int K,
+                                   hipStream_t stream) {
+  if (rows <= 0) return SE_OK;
+  if (K <= 0 || K % 128 || N <= 0 || N % 16 || rows > 65535 * 16) return SE_ERR_SHAPE;
+  if (rows <= 16)
+    launch<2, 1, 1>(x, w, out, nullptr, nullptr, nullptr, nullptr, rows, 1, N, K, 1, stream);
+  else if (rows <= 32)
+    launch<2, 2, 1>(x, w, out, nullptr, nullptr, nullptr, nullptr, rows, 1, N, K, 1, stream);
+  else
+    launch<2, 4, 1>(x, w, out, nullptr, nullptr, nullptr, nullptr, rows, 1, N, K, (rows + 63) / 64, stream);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
 }
 
 // tile_rows: 16, 32 or 64 (the alignment the sorted list was built with); col_blocks: 1 or 2.

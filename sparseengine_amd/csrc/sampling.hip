@@ -150,6 +150,81 @@ sample_kernel(const float* __restrict__ logits, int64_t stride, int vocab,
   if (threadIdx.x == 0) out[row] = best.index;
 }
 
+// Rows without top-k / top-p are one arg-max each (of the logits, or of scaled logits plus
+// noise): many blocks per row find partial maxima over stretches of the vocabulary, one
+// wavefront per row picks among them.
+#define SAMPLE_CHUNK 4096
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_partial_kernel(const float* __restrict__ logits, int64_t stride, int vocab,
+                      const float* __restrict__ temperature, const uint64_t* __restrict__ seeds,
+                      float* __restrict__ part_value, int32_t* __restrict__ part_index, int chunks) {
+  __shared__ ArgBest arg_scratch[SAMPLE_THREADS / SE_WAVE];
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const float* l = logits + static_cast<int64_t>(row) * stride;
+  const float temp = temperature ? temperature[row] : 0.f;
+  const bool greedy = !(temp > 1e-10f);
+  const float inv_temp = greedy ? 1.f : 1.f / temp;
+  const uint64_t seed = seeds ? seeds[row] : 0ull;
+  const int begin = chunk * SAMPLE_CHUNK;
+  const int end = begin + SAMPLE_CHUNK < vocab ? begin + SAMPLE_CHUNK : vocab;
+  ArgBest best = {-INFINITY, -1};
+#pragma unroll
+  for (int j = 0; j < SAMPLE_CHUNK / SAMPLE_THREADS; ++j) {
+    const int i = begin + threadIdx.x + j * SAMPLE_THREADS;
+    if (i < end) {
+      float v = l[i];
+      if (greedy) {
+        if (v != v) v = INFINITY;
+      } else {
+        v = v * inv_temp - logf(-logf(uniform_open(seed, static_cast<uint32_t>(i))));
+      }
+      ArgBest c = {v, i};
+      best = better(best, c);
+    }
+  }
+  best = block_argbest(best, arg_scratch);
+  if (threadIdx.x == 0) {
+    part_value[row * chunks + chunk] = best.value;
+    part_index[row * chunks + chunk] = best.index;
+  }
+}
+
+__global__ void sample_final_kernel(const float* __restrict__ part_value,
+                                    const int32_t* __restrict__ part_index, int chunks,
+                                    int32_t* __restrict__ out) {
+  const int row = blockIdx.x;
+  ArgBest best = {-INFINITY, -1};
+  for (int c = threadIdx.x; c < chunks; c += SE_WAVE) {
+    ArgBest cand = {part_value[row * chunks + c], part_index[row * chunks + c]};
+    best = better(best, cand);
+  }
+#pragma unroll
+  for (int off = SE_WAVE / 2; off > 0; off >>= 1) {
+    ArgBest o;
+    o.value = __shfl_xor(best.value, off, SE_WAVE);
+    o.index = __shfl_xor(best.index, off, SE_WAVE);
+    best = better(best, o);
+  }
+  if (threadIdx.x == 0) out[row] = best.index;
+}
+
+// scratch: rows * ceil(vocab / 4096) floats and as many int32
+extern "C" int se_sample_unfiltered(const float* logits, int64_t stride, int rows, int vocab,
+                                    const float* temperature, const uint64_t* seeds,
+                                    float* part_value, int32_t* part_index, int32_t* out,
+                                    hipStream_t stream) {
+  if (rows <= 0) return SE_OK;
+  if (vocab <= 0 || !part_value || !part_index) return SE_ERR_SHAPE;
+  const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  if (chunks > 65535) return SE_ERR_SHAPE;
+  sample_partial_kernel<<<dim3(rows, chunks), SAMPLE_THREADS, 0, stream>>>(
+      logits, stride, vocab, temperature, seeds, part_value, part_index, chunks);
+  SE_CHECK_LAUNCH();
+  sample_final_kernel<<<rows, SE_WAVE, 0, stream>>>(part_value, part_index, chunks, out);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
 extern "C" int se_sample(const float* logits, int64_t stride, int rows, int vocab,
                          const float* temperature, const int32_t* top_k, const float* top_p,
                          const uint64_t* seeds, int32_t* out, hipStream_t stream) {

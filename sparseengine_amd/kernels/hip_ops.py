@@ -86,10 +86,13 @@ _SIGNATURES = {
     "moe_mfma": {
         "se_grouped_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "se_skinny_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     },
     "sampling": {
         "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p],
+        "se_sample_unfiltered": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_void_p],
     },
 }
 
@@ -154,6 +157,7 @@ class HipKernels:
             raise library.KernelLibraryError(
                 "the HIP kernels need a GPU: torch.cuda.is_available() is False")
         self._attention_partials = None      # (float32 O partials, float32 max/sum partials)
+        self._sample_partials = None         # (float32 values, int32 indices) of the partial arg-max
 
     # ------------------------------------------------------------------ embedding / norms
     def embedding(self, ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor):
@@ -370,6 +374,23 @@ class HipKernels:
         _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
                                             _stream()), "moe_sum")
 
+    SKINNY_ROWS = 64        # up to this many rows a dense product streams the weight once on MFMA
+
+    def linear(self, x, weight, out):
+        """``out = x @ weight.T``.  Few bfloat16 rows take the streaming matrix-core kernel (the BLAS
+        library's choice for such shapes reads the weights at a fraction of memory speed); everything
+        else goes to the BLAS library."""
+        rows, k = x.shape
+        n = weight.shape[0]
+        if (rows <= self.SKINNY_ROWS and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and k % 128 == 0 and n % 16 == 0 and x.is_contiguous() and weight.is_contiguous()
+                and out.is_contiguous() and out.dtype == torch.bfloat16):
+            _require(weight.shape[1] == k and out.shape == (rows, n), "linear shapes")
+            _check(_fn.get("moe_mfma", "se_skinny_gemm_mfma")(_ptr(x), _ptr(weight), _ptr(out), rows, n, k,
+                                                              _stream()), "skinny gemm")
+            return out
+        return torch.mm(x, weight.t(), out=out)
+
     def silu_mul(self, x, out):
         tokens, two_w = x.shape
         _require(x.is_contiguous() and out.is_contiguous() and out.shape == (tokens, two_w // 2)
@@ -390,6 +411,16 @@ class HipKernels:
                             ("top_p", top_p, torch.float32), ("seeds", seeds, torch.int64)):
             if t is not None:
                 _require(t.dtype == dt and t.numel() == rows and t.is_contiguous(), f"sample {name}")
+        if top_k is None and top_p is None:       # one arg-max per row: spread over many blocks
+            need = rows * (-(-vocab // 4096))
+            if self._sample_partials is None or self._sample_partials[0].numel() < need:
+                self._sample_partials = (torch.empty(need, dtype=torch.float32, device=logits.device),
+                                         torch.empty(need, dtype=torch.int32, device=logits.device))
+            _check(_fn.get("sampling", "se_sample_unfiltered")(
+                _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(seeds),
+                _ptr(self._sample_partials[0]), _ptr(self._sample_partials[1]), _ptr(out), _stream()),
+                "sample")
+            return
         _check(_fn.get("sampling", "se_sample")(
             _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
             _ptr(seeds), _ptr(out), _stream()), "sample")

@@ -51,7 +51,7 @@ class GQAAttention(Part):
     def forward(self, fb, x, cache_position: int, write_cache: bool = True):
         s, p, T = self.spec, self.params, x.shape[0]
         cache, meta = fb.kv_view(cache_position)
-        qkv = linear(x, p["qkv"], out=fb.buffer("attn.qkv", (T, self.q_width + 2 * self.kv_width)))
+        qkv = linear(x, p["qkv"], out=fb.buffer("attn.qkv", (T, self.q_width + 2 * self.kv_width)), kernels=fb.kernels)
         fb.kernels.qk_norm_rope_store(
             qkv, meta.positions, self.position.table, p.get("q_norm"), p.get("k_norm"), s.qk_norm_eps,
             s.num_heads, s.num_kv_heads, s.head_dim, self.position.rotary_dim,
@@ -61,7 +61,7 @@ class GQAAttention(Part):
         fb.kernels.paged_attention(q, cache, meta, attended, s.scale, s.window or 0)
         if fb.taps is not None:
             fb.taps.setdefault("attention_inputs", []).append(qkv.clone())
-        return linear(attended, p["o"], out=fb.buffer("attn.proj", (T, self.hidden_size)))
+        return linear(attended, p["o"], out=fb.buffer("attn.proj", (T, self.hidden_size)), kernels=fb.kernels)
 
 
 MIXERS.register("gqa_attention", lambda spec, hidden_size: GQAAttention(spec, hidden_size))

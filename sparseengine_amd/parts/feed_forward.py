@@ -93,10 +93,10 @@ class DenseMLP(Part):
 
     def forward(self, fb, x):
         T, i = x.shape[0], self.spec.intermediate_size
-        gate_up = linear(x, self.params["gate_up"], out=fb.buffer("mlp.gate_up", (T, 2 * i)))
+        gate_up = linear(x, self.params["gate_up"], out=fb.buffer("mlp.gate_up", (T, 2 * i)), kernels=fb.kernels)
         act = fb.buffer("mlp.act", (T, i))
         fb.kernels.silu_mul(gate_up, act)
-        return linear(act, self.params["down"], out=fb.buffer("ffn.out", (T, self.hidden_size)))
+        return linear(act, self.params["down"], out=fb.buffer("ffn.out", (T, self.hidden_size)), kernels=fb.kernels)
 
 
 FEED_FORWARDS.register("moe", lambda spec, hidden_size, chunk_tokens=16384: RoutedExperts(spec, hidden_size, chunk_tokens))

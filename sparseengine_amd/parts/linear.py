@@ -5,12 +5,16 @@ from __future__ import annotations
 import torch
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None, kernels=None) -> torch.Tensor:
     """``x @ weight.T``.  A weight kept in float32 under a bfloat16 engine is multiplied in
-    float32 and the product rounded to the activations' dtype."""
+    float32 and the product rounded to the activations' dtype.  ``kernels`` may offer its own
+    ``linear`` for shapes the BLAS library serves badly (a few rows against a large matrix)."""
     if weight.dtype == x.dtype:
         if out is None:
             return torch.mm(x, weight.t())
+        fast = getattr(kernels, "linear", None)
+        if fast is not None:
+            return fast(x, weight, out)
         return torch.mm(x, weight.t(), out=out)
     y = torch.mm(x.to(weight.dtype), weight.t())
     if out is None:

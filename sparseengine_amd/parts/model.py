@@ -75,7 +75,7 @@ class DecoderModel(Part):
         last = fb.buffer("model.wanted", (wanted, spec.hidden_size))
         self.final_norm.forward_rows(fb, x, residual, fb.want_index, last)
         weight = (self.head or self.embed).params["weight"]
-        logits = linear(last, weight, out=fb.buffer("model.logits", (wanted, spec.vocab_size)))
+        logits = linear(last, weight, out=fb.buffer("model.logits", (wanted, spec.vocab_size)), kernels=fb.kernels)
         return logits.to(torch.float32, copy=True)      # the caller's own tensor, not the scratch buffer
 
 

@@ -357,6 +357,14 @@ def test_sampling(hip, twin):
     hip.sample(logits, temp, top_k, top_p, seeds, out)
     twin.sample(logits, temp, top_k, top_p, seeds, ref)
     assert torch.equal(out, ref)
+    # without filters the many-block path is taken: same noise, same choice as the one-block kernel
+    big = (torch.randn(5, 20011) * 2).cuda()
+    t5 = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.3]).cuda()
+    s5 = seeds[:5].contiguous()
+    fast = torch.empty(5, dtype=torch.int32, device="cuda"); slow = torch.empty_like(fast)
+    hip.sample(big, t5, None, None, s5, fast)
+    hip.sample(big, t5, torch.zeros(5, dtype=torch.int32).cuda(), None, s5, slow)
+    assert torch.equal(fast, slow) and int(fast[0]) == int(big[0].argmax())
     # a row's draw does not depend on the rest of the batch
     one = torch.empty(1, dtype=torch.int32, device="cuda")
     for r in range(rows):
@@ -403,3 +411,15 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
         row, pos = int(meta.token_row[t]), int(meta.positions[t])
         ref = dense_attention(q[t], cache, table, row, pos, head_dim ** -0.5, 0, page)
         torch.testing.assert_close(out_h[t].float(), ref, rtol=1.6e-2, atol=1.6e-2)
+
+
+@pytest.mark.parametrize("rows,n,k", [(1, 8192, 3072), (8, 3072, 6144), (16, 256, 128), (17, 48, 256), (33, 1024, 384),
+                                      (64, 200064, 3072), (5, 50, 128), (3, 64, 96)])
+def test_skinny_linear(hip, rows, n, k):
+    """Few rows against a large matrix: the streaming kernel where its sizes fit, the library otherwise."""
+    x = randn(rows, k, dtype=torch.bfloat16, seed=1)
+    w = randn(n, k, dtype=torch.bfloat16, scale=k ** -0.5, seed=2)
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    hip.linear(x, w, out)
+    ref = x.float() @ w.float().T
+    torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1.6e-2)
