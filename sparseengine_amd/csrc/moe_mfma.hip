@@ -22,6 +22,22 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
+// Work item (tile, column block) of a block in a 1-D grid.  Consecutive block ids go to
+// different XCDs (id % 8), and every XCD has an L2 of its own: so each XCD gets one contiguous
+// stretch of the work, and the column blocks of a tile - which all read the tile's activation
+// rows - and the tiles of one expert - which read the same weights - meet in one L2.
+__device__ __forceinline__ bool xcd_work_item(int column_blocks, int num_tiles, int& tile, int& column_block) {
+  const int total = num_tiles * column_blocks;
+  const int per_xcd = (total + 7) >> 3;
+  const int xcd = blockIdx.x & 7, index = blockIdx.x >> 3;
+  if (index >= per_xcd) return false;
+  const int item = xcd * per_xcd + index;
+  if (item >= total) return false;
+  tile = item / column_blocks;
+  column_block = item % column_blocks;
+  return true;
+}
+
 template <int MODE, int MB, int NB, int U>
 __global__ void __launch_bounds__(256)
 grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
@@ -29,12 +45,12 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
                          const int32_t* __restrict__ tile_expert,
                          const int32_t* __restrict__ counters,
                          const float* __restrict__ route_weight, int assignments, int top_k, int N,
-                         int K) {
+                         int K, int max_tiles) {
   constexpr int BM = 16 * MB;
   constexpr int BN = 16 * NB;
   constexpr int NBT = MODE == 0 ? 2 * NB : NB;  // weight blocks per wave: gate blocks, then up blocks
-  const int tile = blockIdx.y;
-  if (MODE != 2 && tile >= counters[0]) return;  // uniform over the block
+  int tile, column_block;
+  if (!xcd_work_item(N / BN, MODE == 2 ? max_tiles : counters[0], tile, column_block)) return;  // uniform
 
   constexpr int P = NB * MB;                   // output blocks of 16 x 16 (gate/up pairs in MODE 0)
   constexpr int PARTS = MODE == 0 ? 2 : 1;
@@ -45,7 +61,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   const int lane = threadIdx.x & (SE_WAVE - 1);
   const int wave = threadIdx.x / SE_WAVE;
   const int expert = MODE == 2 ? 0 : tile_expert[tile];
-  const int n0 = blockIdx.x * BN;
+  const int n0 = column_block * BN;
   if (threadIdx.x < BM)
     rows[threadIdx.x] = MODE == 2 ? tile * BM + static_cast<int>(threadIdx.x) : sorted[tile * BM + threadIdx.x];
   __syncthreads();
@@ -192,10 +208,11 @@ template <int MODE, int MB, int NB, int U>
 static void launch_u(const void* in, const void* w, void* out, const int32_t* sorted,
                    const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
                    int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
-  dim3 grid(N / (16 * NB), max_tiles);
+  const int64_t items = static_cast<int64_t>(N / (16 * NB)) * max_tiles;
+  const int grid = static_cast<int>((items + 7) / 8 * 8);
   grouped_gemm_mfma_kernel<MODE, MB, NB, U><<<grid, 256, 0, stream>>>(
       static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
-      tile_expert, counters, route_weight, assignments, top_k, N, K);
+      tile_expert, counters, route_weight, assignments, top_k, N, K, max_tiles);
 }
 
 // steps of 32 per stage: as many as divide a wave's quarter of K, fewer for taller tiles (registers)
@@ -221,6 +238,179 @@ static void launch(const void* in, const void* w, void* out, const int32_t* sort
                               top_k, N, K, max_tiles, stream);
 }
 
+// ---------------------------------------------------------------------------------------- //
+// Tall tiles (an expert has dozens of rows, as in the prefill of a long prompt): the weights of a
+// tile are used by many rows, so they are staged through LDS and shared by the block's four
+// waves.  A block computes BM = 16 * MB rows x 128 weight rows (MODE 0: 64 gate + 64 up rows ->
+// 64 outputs; MODE 1: 128 outputs) in steps of 64 along K, double-buffered: the loads of the next
+// step are in flight while the matrix cores work on the current one.  Wave w owns 32 of the
+// weight rows (MODE 0: gate rows 16 w .. and the matching up rows) and all rows of the tile.
+// Each output is one dot product in the order of K, as in the streaming kernel.
+// ---------------------------------------------------------------------------------------- //
+#define TALL_BK 64
+#define TALL_LD 72          // row stride in LDS (elements): 64 + 8 keeps 16-byte reads off the same banks
+
+template <int MODE, int MB>
+__global__ void __launch_bounds__(256)
+grouped_gemm_tall_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                         bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                         const int32_t* __restrict__ tile_expert,
+                         const int32_t* __restrict__ counters,
+                         const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                         int K) {
+  constexpr int BM = 16 * MB;
+  constexpr int WROWS = 128;
+  int tile, column_block;
+  if (!xcd_work_item(N / (MODE == 0 ? 64 : 128), counters[0], tile, column_block)) return;  // uniform
+  __shared__ __attribute__((aligned(16))) uint16_t ws[2][WROWS][TALL_LD];
+  __shared__ __attribute__((aligned(16))) uint16_t xs[2][BM][TALL_LD];
+  __shared__ int32_t rows[BM];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (SE_WAVE - 1);
+  const int wave = tid / SE_WAVE;
+  const int col = lane & 15, kgroup = lane >> 4;
+  const int expert = tile_expert[tile];
+  const int out_cols = MODE == 0 ? 64 : 128;
+  const int n0 = column_block * out_cols;
+  if (tid < BM) rows[tid] = sorted[tile * BM + tid];
+  __syncthreads();
+
+  const int64_t w_rows = MODE == 0 ? 2 * static_cast<int64_t>(N) : N;
+  const bf16_t* we = w + static_cast<int64_t>(expert) * w_rows * K;
+
+  // global -> LDS assignment: a chunk is 8 elements (16 bytes), a 64-wide row has 8 chunks; thread
+  // t moves chunk t & 7 of rows (t >> 3) + 32 j.  Everything is kept in named scalars so that the
+  // loads stay in registers while they are in flight.
+  static_assert(MB == 4, "the staging below moves exactly two activation chunks per thread");
+  const int r0 = tid >> 3, kc = (tid & 7) * 8;
+  const bf16_t* wp0 = we + static_cast<int64_t>(n0 + r0) * K + kc;                  // tile rows r0, r0 + 32
+  const bf16_t* wp1 = wp0 + static_cast<int64_t>(32) * K;
+  const bf16_t* wp2 = MODE == 0 ? we + (static_cast<int64_t>(N) + n0 + r0) * K + kc  // tile rows 64 + r0, 96 + r0
+                                : wp0 + static_cast<int64_t>(64) * K;
+  const bf16_t* wp3 = wp2 + static_cast<int64_t>(32) * K;
+  const int a0 = rows[r0], a1 = rows[r0 + 32];
+  const bf16_t* xp0 = in + (a0 < assignments ? static_cast<int64_t>(MODE == 0 ? a0 / top_k : a0) : 0) * K + kc;
+  const bf16_t* xp1 = in + (a1 < assignments ? static_cast<int64_t>(MODE == 0 ? a1 / top_k : a1) : 0) * K + kc;
+  const int lds0 = r0 * TALL_LD + kc;               // element offset of the thread's first chunk
+  constexpr int LDS32 = 32 * TALL_LD;
+
+  floatx4 acc[2][MB];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // rows of the weight tile this wave multiplies: block 0 and block 1
+  const int a_row0 = MODE == 0 ? 16 * wave + col : 32 * wave + col;
+  const int a_row1 = MODE == 0 ? 64 + 16 * wave + col : 32 * wave + 16 + col;
+
+#define TALL_FETCH(S, K0)                                        \
+  S##w0 = *reinterpret_cast<const uint4*>(wp0 + (K0));           \
+  S##w1 = *reinterpret_cast<const uint4*>(wp1 + (K0));           \
+  S##w2 = *reinterpret_cast<const uint4*>(wp2 + (K0));           \
+  S##w3 = *reinterpret_cast<const uint4*>(wp3 + (K0));           \
+  S##x0 = *reinterpret_cast<const uint4*>(xp0 + (K0));           \
+  S##x1 = *reinterpret_cast<const uint4*>(xp1 + (K0));
+#define TALL_STASH(S, BUF)                                                          \
+  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0) = S##w0;                         \
+  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0 + LDS32) = S##w1;                 \
+  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0 + 2 * LDS32) = S##w2;             \
+  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0 + 3 * LDS32) = S##w3;             \
+  *reinterpret_cast<uint4*>(&xs[BUF][0][0] + lds0) = S##x0;                         \
+  *reinterpret_cast<uint4*>(&xs[BUF][0][0] + lds0 + LDS32) = S##x1;
+#define TALL_COMPUTE(BUF)                                                                              \
+  _Pragma("unroll") for (int sub = 0; sub < TALL_BK / 32; ++sub) {                                     \
+    const int ko = sub * 32 + kgroup * 8;                                                              \
+    const uint4 af0 = *reinterpret_cast<const uint4*>(&ws[BUF][a_row0][ko]);                           \
+    const uint4 af1 = *reinterpret_cast<const uint4*>(&ws[BUF][a_row1][ko]);                           \
+    _Pragma("unroll") for (int mb = 0; mb < MB; ++mb) {                                                \
+      const uint4 bf = *reinterpret_cast<const uint4*>(&xs[BUF][mb * 16 + col][ko]);                   \
+      acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af0),            \
+                                                           __builtin_bit_cast(bf16x8, bf), acc[0][mb], 0, 0, 0); \
+      acc[1][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af1),            \
+                                                           __builtin_bit_cast(bf16x8, bf), acc[1][mb], 0, 0, 0); \
+    }                                                                                                  \
+  }
+
+  // Two register sets (p, q) hold the loads of the next two steps: a load has a whole step of
+  // matrix work, and the other block of the CU, to arrive before it is written to LDS.
+  uint4 pw0, pw1, pw2, pw3, px0, px1, qw0, qw1, qw2, qw3, qx0, qx1;
+  const int steps = K / TALL_BK;     // even: K % 128 == 0
+  TALL_FETCH(p, 0)
+  TALL_FETCH(q, TALL_BK)
+  TALL_STASH(p, 0)
+  __syncthreads();
+  for (int kt = 0; kt < steps; kt += 2) {
+    // step kt: LDS buffer 0 is current, set q holds step kt + 1, set p is free
+    if (kt + 2 < steps) { TALL_FETCH(p, (kt + 2) * TALL_BK) }
+    TALL_COMPUTE(0)
+    TALL_STASH(q, 1)
+    __syncthreads();
+    // step kt + 1: buffer 1 is current, set p holds step kt + 2, set q is free
+    if (kt + 3 < steps) { TALL_FETCH(q, (kt + 3) * TALL_BK) }
+    TALL_COMPUTE(1)
+    if (kt + 2 < steps) { TALL_STASH(p, 0) }
+    __syncthreads();
+  }
+#undef TALL_FETCH
+#undef TALL_STASH
+#undef TALL_COMPUTE
+
+  // lane (kgroup, col): acc[nb][mb][i] belongs to weight row 4 * kgroup + i of block nb, tile row mb * 16 + col
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int a = rows[mb * 16 + col];
+    if (a >= assignments) continue;
+    if (MODE == 0) {
+      uint16_t y[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float gate = round_to<bf16_t>(acc[0][mb][i]);
+        const float up = round_to<bf16_t>(acc[1][mb][i]);
+        const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
+        y[i] = float_to_bf16_bits(act * up);
+      }
+      uint2 packed;
+      packed.x = static_cast<uint32_t>(y[0]) | (static_cast<uint32_t>(y[1]) << 16);
+      packed.y = static_cast<uint32_t>(y[2]) | (static_cast<uint32_t>(y[3]) << 16);
+      *reinterpret_cast<uint2*>(out + static_cast<int64_t>(a) * N + n0 + 16 * wave + 4 * kgroup) = packed;
+    } else {
+      const float rw = route_weight[a];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][0] * rw)) |
+                   (static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][1] * rw)) << 16);
+        packed.y = static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][2] * rw)) |
+                   (static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][3] * rw)) << 16);
+        *reinterpret_cast<uint2*>(out + static_cast<int64_t>(a) * N + n0 + 32 * wave + 16 * nb + 4 * kgroup) = packed;
+      }
+    }
+  }
+}
+
+// tile_rows: 64.  MODE 0 needs N % 64 == 0, MODE 1 N % 128 == 0; K % 64 == 0.
+extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, const int32_t* sorted,
+                                    const int32_t* tile_expert, const int32_t* counters,
+                                    const float* route_weight, int assignments, int top_k, int N,
+                                    int K, int max_tiles, int mode, int tile_rows, hipStream_t stream) {
+  if (assignments <= 0) return SE_OK;
+  if (K <= 0 || K % (2 * TALL_BK) || N <= 0 || N % (mode == 0 ? 64 : 128)) return SE_ERR_SHAPE;
+  if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
+  const int64_t items = static_cast<int64_t>(N / (mode == 0 ? 64 : 128)) * max_tiles;
+  const int grid = static_cast<int>((items + 7) / 8 * 8);
+#define SE_TALL(MODE, MB)                                                                          \
+  grouped_gemm_tall_kernel<MODE, MB><<<grid, 256, 0, stream>>>(                                    \
+      static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
+      tile_expert, counters, route_weight, assignments, top_k, N, K)
+  if (tile_rows == 64) { if (mode == 0) SE_TALL(0, 4); else SE_TALL(1, 4); }
+  else return SE_ERR_SHAPE;
+#undef SE_TALL
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
 // Dense product of a few rows: out[rows, N] = x[rows, K] . w[N, K]^T (bfloat16, float accumulate).
 extern "C" int se_skinny_gemm_mfma(const void* x, const void* w, void* out, int rows, int N, int K,
                                    hipStream_t stream) {
@@ -244,7 +434,7 @@ extern "C" int se_grouped_gemm_mfma(const void* in, const void* w, void* out, co
                                     hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
   if (K <= 0 || K % 128 || N <= 0 || N % (16 * col_blocks)) return SE_ERR_SHAPE;
-  if (max_tiles <= 0 || max_tiles > 65535) return SE_ERR_SHAPE;
+  if (max_tiles <= 0 || max_tiles > (1 << 22)) return SE_ERR_SHAPE;
   if (mode != 0 && mode != 1) return SE_ERR_SHAPE;
 #define SE_CASE(MB, NB)                                                                             \
   if (tile_rows == 16 * MB && col_blocks == NB) {                                                   \

@@ -87,6 +87,8 @@ _SIGNATURES = {
         "se_grouped_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "se_skinny_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "se_grouped_gemm_tall": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "sampling": {
         "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -127,7 +129,7 @@ def moe_tile_bounds(assignments: int, experts: int, tile_rows: int) -> tuple[int
 class MoeWorkspace:
     """Scratch tensors of the expert pipeline, sized for a largest number of tokens."""
 
-    TILE_ROWS = (16, 32, 64)      # alignments the expert kernels may ask for
+    TILE_ROWS = (16, 32, 64, 96, 128)      # alignments the expert kernels may ask for
 
     def __init__(self, max_tokens: int, top_k: int, experts: int, hidden: int, intermediate: int,
                  dtype: torch.dtype, device):
@@ -326,7 +328,7 @@ class HipKernels:
             _ptr(ws.counters), _stream()), "moe_align")
         return max_tiles
 
-    def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, tile_rows=None, wide=None):
+    def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, tile_rows=None, wide=None, tall=None):
         """``out[t] = sum_k weights[t,k] * W2_e(silu(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``;
         ``w13 [E, 2I, h]`` holds gate rows then up rows, ``w2 [E, h, I]``."""
         tokens, hidden = x.shape
@@ -347,10 +349,25 @@ class HipKernels:
             # as still leaves enough workgroups for the whole chip
             share = assignments / min(experts, assignments)
             if tile_rows is None:
-                tile_rows = 16 if share <= 16 else 32 if share <= 32 else 64
+                tile_rows = 16 if share <= 16 else 64
+            if tall is None:
+                tall = share > 16          # many rows per expert: the weights go through LDS and are shared
+            if tall:
+                tile_rows = 64
             max_tiles = self.moe_align(ids, experts, ws, tile_rows)
             if max_tiles > 65535:
                 raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
+            if tall:
+                gt = _fn.get("moe_mfma", "se_grouped_gemm_tall")
+                _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                          _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
+                          _stream()), "moe gate-up (tall)")
+                _check(gt(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                          _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
+                          tile_rows, _stream()), "moe down (tall)")
+                _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
+                                                    _stream()), "moe_sum")
+                return
             gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
             if wide is None:
                 wide = 2 if max_tiles * (inter // 32) >= 2048 else 1
