@@ -32,6 +32,21 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
          (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
 }
 
+// Eight consecutive keys of one value dim; those after `last_key` are made zero: slots past a
+// request's last key hold whatever an earlier owner of the page left (possibly not finite).
+__device__ __forceinline__ uint4 zero_keys_beyond(uint4 v, int first_key, int last_key) {
+  const int keep = last_key - first_key + 1;   // keys 0 .. keep - 1 of the eight stay
+  auto word = [&](uint32_t w, int k) {
+    const uint32_t m = (2 * k < keep ? 0x0000ffffu : 0u) | (2 * k + 1 < keep ? 0xffff0000u : 0u);
+    return w & m;
+  };
+  v.x = word(v.x, 0);
+  v.y = word(v.y, 1);
+  v.z = word(v.z, 2);
+  v.w = word(v.w, 3);
+  return v;
+}
+
 template <int DSTEPS>  // head_dim = 32 * DSTEPS
 __global__ void __launch_bounds__(256)
 paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
@@ -93,82 +108,125 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   for (int db = 0; db < DBLOCKS; ++db) o[db] = floatx4{0.f, 0.f, 0.f, 0.f};
   float run_max = -INFINITY, run_sum = 0.f;
 
-  for (int k0 = k_first; k0 < key_end; k0 += 32) {
-    // ---- scores of 32 keys x 16 rows
-    floatx4 s[2];
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      s[b] = floatx4{0.f, 0.f, 0.f, 0.f};
-      int key = k0 + 8 * (n >> 2) + (n & 3) + 4 * b;
-      if (key > last_key) key = last_key;           // reads stay inside the request's pages
-      const int page = table[key / page_size];
-      const bf16_t* k_row = cache + (static_cast<int64_t>(page) * 2) * plane + kvh * head_span +
-                            static_cast<int64_t>(key % page_size) * D + g * 8;
-#pragma unroll
-      for (int ds = 0; ds < DSTEPS; ++ds) {
-        const uint4 kf = *reinterpret_cast<const uint4*>(k_row + ds * 32);
-        s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
-                                                       __builtin_bit_cast(bf16x8, qf[ds]), s[b], 0, 0, 0);
-      }
-    }
-    // lane (g, n): s[b][i] is the score of key k0 + 8 g + 4 b + i for row n
-    float p[8];
-    float tile_max = -INFINITY;
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + 8 * g + 4 * b + i;
-        const bool masked = key > pos || (window > 0 && key <= pos - window);
-        const float v = masked ? -INFINITY : s[b][i] * scale_log2e;
-        p[b * 4 + i] = v;
-        tile_max = fmaxf(tile_max, v);
-      }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, SE_WAVE));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, SE_WAVE));
-    const float new_max = fmaxf(run_max, tile_max);
-    const float ref = (new_max == -INFINITY) ? 0.f : new_max;   // a row with no key yet
-    const float alpha = exp2f(run_max - ref);
-    float tile_sum = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      p[j] = exp2f(p[j] - ref);
-      tile_sum += p[j];
-    }
-    tile_sum += __shfl_xor(tile_sum, 16, SE_WAVE);
-    tile_sum += __shfl_xor(tile_sum, 32, SE_WAVE);
-    run_sum = run_sum * alpha + tile_sum;
-    run_max = new_max;
-#pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) o[db] *= alpha;
+  // One step = 32 keys.  Two register sets (A, B) take turns: while the matrix cores and the
+  // softmax work on one step, the key and value operands of the next are already being loaded,
+  // and the page ids of the step after that are looked up.  Without this every step costs two
+  // memory round trips (keys, then values) and the kernel is bound by latency, not by bandwidth.
+  auto page_of_keys = [&](int k0) {     // page of the lane's two key rows (both lie in one group of 8)
+    int key = k0 + 8 * (n >> 2);
+    if (key > last_key) key = last_key;
+    return table[key / page_size];
+  };
+  auto page_of_values = [&](int k0) {   // page of the lane's eight consecutive keys
+    int key = k0 + 8 * g;
+    if (key > last_key) key = last_key & ~7;
+    return table[key / page_size];
+  };
 
-    uint4 pf;
-    pf.x = pack_bf16x2(p[0], p[1]);
-    pf.y = pack_bf16x2(p[2], p[3]);
-    pf.z = pack_bf16x2(p[4], p[5]);
-    pf.w = pack_bf16x2(p[6], p[7]);
+#define ATT_LOAD(KF, VF, K0, PK, PV)                                                              \
+  {                                                                                               \
+    _Pragma("unroll") for (int b = 0; b < 2; ++b) {                                               \
+      int key = (K0) + 8 * (n >> 2) + (n & 3) + 4 * b;                                            \
+      if (key > last_key) key = last_key; /* reads stay inside the request's pages */            \
+      const bf16_t* k_row = cache + (static_cast<int64_t>(PK) * 2) * plane + kvh * head_span +    \
+                            static_cast<int64_t>(key % page_size) * D + g * 8;                    \
+      _Pragma("unroll") for (int ds = 0; ds < DSTEPS; ++ds)                                       \
+          KF[b][ds] = *reinterpret_cast<const uint4*>(k_row + ds * 32);                           \
+    }                                                                                             \
+    int vkey = (K0) + 8 * g;                                                                      \
+    if (vkey > last_key) vkey = last_key & ~7;                                                    \
+    const bf16_t* v_col = cache + (static_cast<int64_t>(PV) * 2 + 1) * plane + kvh * head_span +  \
+                          static_cast<int64_t>(n) * page_size + (vkey % page_size);               \
+    _Pragma("unroll") for (int db = 0; db < DBLOCKS; ++db)                                        \
+        VF[db] = *reinterpret_cast<const uint4*>(v_col + static_cast<int64_t>(db) * 16 * page_size); \
+  }
 
-    // ---- values: lane (g, n) reads value dim db * 16 + n at keys k0 + 8 g .. + 7
-    int vkey = k0 + 8 * g;
-    const bool beyond = vkey + 7 > last_key;        // only in the request's last step
-    if (vkey > last_key) vkey = last_key & ~7;
-    const int vpage = table[vkey / page_size];
-    const bf16_t* v_col = cache + (static_cast<int64_t>(vpage) * 2 + 1) * plane + kvh * head_span +
-                          static_cast<int64_t>(n) * page_size + (vkey % page_size);
-#pragma unroll
-    for (int db = 0; db < DBLOCKS; ++db) {
-      uint4 vf = *reinterpret_cast<const uint4*>(v_col + static_cast<int64_t>(db) * 16 * page_size);
-      if (beyond) {
-        // slots past the request's last key hold whatever an earlier owner left: make them zero
-        uint32_t* w32 = &vf.x;
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (vkey + j > last_key) w32[j >> 1] &= (j & 1) ? 0x0000ffffu : 0xffff0000u;
+#define ATT_COMPUTE(KF, VF, K0)                                                                   \
+  {                                                                                               \
+    floatx4 s[2];                                                                                 \
+    _Pragma("unroll") for (int b = 0; b < 2; ++b) {                                               \
+      s[b] = floatx4{0.f, 0.f, 0.f, 0.f};                                                         \
+      _Pragma("unroll") for (int ds = 0; ds < DSTEPS; ++ds)                                       \
+          s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, KF[b][ds]),   \
+                                                         __builtin_bit_cast(bf16x8, qf[ds]), s[b], 0, 0, 0); \
+    }                                                                                             \
+    /* lane (g, n): s[b][i] is the score of key K0 + 8 g + 4 b + i for row n */                   \
+    float p[8];                                                                                   \
+    float tile_max = -INFINITY;                                                                   \
+    _Pragma("unroll") for (int b = 0; b < 2; ++b)                                                 \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                             \
+        const int key = (K0) + 8 * g + 4 * b + i;                                                 \
+        const bool masked = key > pos || (window > 0 && key <= pos - window);                     \
+        const float v = masked ? -INFINITY : s[b][i] * scale_log2e;                               \
+        p[b * 4 + i] = v;                                                                         \
+        tile_max = fmaxf(tile_max, v);                                                            \
+      }                                                                                           \
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, SE_WAVE));                                \
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, SE_WAVE));                                \
+    const float new_max = fmaxf(run_max, tile_max);                                               \
+    const float ref = (new_max == -INFINITY) ? 0.f : new_max; /* a row with no key yet */         \
+    const float alpha = exp2f(run_max - ref);                                                     \
+    float tile_sum = 0.f;                                                                         \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                               \
+      p[j] = exp2f(p[j] - ref);                                                                   \
+      tile_sum += p[j];                                                                           \
+    }                                                                                             \
+    tile_sum += __shfl_xor(tile_sum, 16, SE_WAVE);                                                \
+    tile_sum += __shfl_xor(tile_sum, 32, SE_WAVE);                                                \
+    run_sum = run_sum * alpha + tile_sum;                                                         \
+    run_max = new_max;                                                                            \
+    _Pragma("unroll") for (int db = 0; db < DBLOCKS; ++db) o[db] *= alpha;                        \
+    uint4 pf;                                                                                     \
+    pf.x = pack_bf16x2(p[0], p[1]);                                                               \
+    pf.y = pack_bf16x2(p[2], p[3]);                                                               \
+    pf.z = pack_bf16x2(p[4], p[5]);                                                               \
+    pf.w = pack_bf16x2(p[6], p[7]);                                                               \
+    /* values: lane (g, n) holds value dim db * 16 + n at keys K0 + 8 g .. + 7 */                 \
+    int vkey = (K0) + 8 * g;                                                                      \
+    const bool beyond = vkey + 7 > last_key; /* only in the request's last step */                \
+    if (vkey > last_key) vkey = last_key & ~7;                                                    \
+    _Pragma("unroll") for (int db = 0; db < DBLOCKS; ++db) {                                      \
+      uint4 vf = VF[db];                                                                          \
+      if (beyond) vf = zero_keys_beyond(vf, vkey, last_key);                                      \
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),             \
+                                                     __builtin_bit_cast(bf16x8, pf), o[db], 0, 0, 0); \
+    }                                                                                             \
+  }
+
+  if (k_first < key_end) {
+    uint4 kfA[2][DSTEPS], vfA[DBLOCKS];
+    if constexpr (DSTEPS <= 4) {
+      uint4 kfB[2][DSTEPS], vfB[DBLOCKS];
+      int pk = page_of_keys(k_first), pv = page_of_values(k_first);
+      ATT_LOAD(kfA, vfA, k_first, pk, pv)
+      pk = page_of_keys(k_first + 32);
+      pv = page_of_values(k_first + 32);
+      for (int k0 = k_first; k0 < key_end; k0 += 64) {
+        const bool second = k0 + 32 < key_end;
+        if (second) {
+          ATT_LOAD(kfB, vfB, k0 + 32, pk, pv)
+          pk = page_of_keys(k0 + 64);
+          pv = page_of_values(k0 + 64);
+        }
+        ATT_COMPUTE(kfA, vfA, k0)
+        if (!second) break;
+        if (k0 + 64 < key_end) {
+          ATT_LOAD(kfA, vfA, k0 + 64, pk, pv)
+          pk = page_of_keys(k0 + 96);
+          pv = page_of_values(k0 + 96);
+        }
+        ATT_COMPUTE(kfB, vfB, k0 + 32)
       }
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
-                                                     __builtin_bit_cast(bf16x8, pf), o[db], 0, 0, 0);
+    } else {   // large heads: one register set; keys and values of a step are still loaded together
+      for (int k0 = k_first; k0 < key_end; k0 += 32) {
+        const int pk = page_of_keys(k0), pv = page_of_values(k0);
+        ATT_LOAD(kfA, vfA, k0, pk, pv)
+        ATT_COMPUTE(kfA, vfA, k0)
+      }
     }
   }
+#undef ATT_LOAD
+#undef ATT_COMPUTE
 
   // lane (g, n): o[db][i] is value dim db * 16 + 4 g + i of row n
   if (slot < 0) {
@@ -190,6 +248,229 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     if (g == 0) {
       part_ml[base * 2] = run_max;
       part_ml[base * 2 + 1] = run_sum;
+    }
+  }
+}
+
+// Prompt portions: the same product with the keys and values of a step shared by a whole block.
+// A block of four wavefronts takes 4 * RT consecutive row tiles of one request and one kv head
+// (wave w the tiles first + w * RT ...), brings each step of 32 keys into shared memory once
+// (two buffers: the loads of the next step are in flight while this one is computed) and every
+// wave reads its operands from there, each operand feeding RT products.  The per-wave kernel above
+// reads every key once per 16 rows, which binds a long prompt to the L2's bandwidth.
+//
+// Shared layout: keys in operand order (row b * 16 + m holds key 8 * (m / 4) + m % 4 + 4 * b of
+// the step), row stride D + 8 elements; values [dim][32 keys], row stride 40 elements: the 16
+// lanes of a quarter wave then touch 16 different groups of four banks.
+// A unit is {item, first_tile, key_begin, key_end, -, -}; it always writes the output itself.
+template <int DSTEPS, int RT>
+__global__ void __launch_bounds__(256)
+paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
+                             const bf16_t* __restrict__ cache,
+                             const int32_t* __restrict__ block_table, int bt_stride,
+                             const int32_t* __restrict__ item_meta, int num_items,
+                             const int32_t* __restrict__ units, bf16_t* __restrict__ out,
+                             int64_t out_stride, int heads, int kv_heads, int page_size,
+                             float scale_log2e, int window) {
+  constexpr int D = 32 * DSTEPS;
+  constexpr int DBLOCKS = 2 * DSTEPS;
+  constexpr int KS = D + 8;                       // key row stride in shared memory (elements)
+  constexpr int VS = 40;                          // value row stride
+  constexpr int VECS = 128 * DSTEPS;              // 16-byte vectors of a step's keys (and of its values)
+  constexpr int LOADS = (VECS + 255) / 256;
+  __shared__ __align__(16) bf16_t k_lds[2][32 * KS];
+  __shared__ __align__(16) bf16_t v_lds[2][D * VS];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (SE_WAVE - 1);
+  const int wave = tid / SE_WAVE;
+  const int n = lane & 15;
+  const int g = lane >> 4;
+  const int kvh = blockIdx.x % kv_heads;   // units come longest first: all kv heads of one, then the next
+  const int group = heads / kv_heads;
+
+  const int32_t* u = units + static_cast<int64_t>(blockIdx.x / kv_heads) * UNIT_FIELDS;
+  const int item = u[0], first_tile = u[1], key_begin = u[2];
+  int key_end = u[3];
+  const int q_start = item_meta[item], q_len = item_meta[num_items + item],
+            ctx_len = item_meta[2 * num_items + item];
+  const int rows_total = q_len * group;
+  const int pos0 = ctx_len - q_len;
+  const int last_key = ctx_len - 1;
+
+  // the block's rows bound the keys that are loaded; the wave's rows bound what it computes
+  const int block_last_row = min((first_tile + 4 * RT) * 16, rows_total) - 1;
+  key_end = min(key_end, pos0 + block_last_row / group + 1);
+  int k_first = key_begin;
+  if (window > 0) {
+    const int lowest = pos0 + (first_tile * 16) / group - window + 1;
+    if (lowest > k_first) k_first = lowest & ~31;
+  }
+  const int tile0 = first_tile + wave * RT;
+  const bool wave_active = tile0 * 16 < rows_total;
+  const int wave_last_row = min((tile0 + RT) * 16, rows_total) - 1;
+  const int wave_hi = wave_active ? pos0 + wave_last_row / group : -1;          // largest position
+  const int wave_lo = wave_active ? pos0 + (tile0 * 16) / group : 0;            // smallest position
+
+  int token[RT], head[RT], pos[RT];
+  bool row_valid[RT];
+  uint4 qf[RT][DSTEPS];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int rho = (tile0 + rt) * 16 + n;
+    row_valid[rt] = rho < rows_total;
+    const int rho_c = row_valid[rt] ? rho : rows_total - 1;   // padding rows repeat the last row
+    const int q_idx = rho_c / group;
+    head[rt] = kvh * group + rho_c % group;
+    token[rt] = q_start + q_idx;
+    pos[rt] = pos0 + q_idx;
+    const bf16_t* q_row = q + static_cast<int64_t>(token[rt]) * q_stride +
+                          static_cast<int64_t>(head[rt]) * D + g * 8;
+#pragma unroll
+    for (int ds = 0; ds < DSTEPS; ++ds) qf[rt][ds] = *reinterpret_cast<const uint4*>(q_row + ds * 32);
+  }
+
+  const int32_t* table = block_table + static_cast<int64_t>(item) * bt_stride;
+  const int64_t head_span = static_cast<int64_t>(page_size) * D;
+  const int64_t plane = static_cast<int64_t>(kv_heads) * head_span;
+  const bf16_t* cache_head = cache + kvh * head_span;
+
+  floatx4 o[RT][DBLOCKS];
+  float run_max[RT], run_sum[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    run_max[rt] = -INFINITY;
+    run_sum[rt] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) o[rt][db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  uint4 kr[LOADS], vr[LOADS];   // a step's vectors on their way from the cache to shared memory
+
+#define TILED_FETCH(K0)                                                                            \
+  _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                              \
+    const int idx = tid + 256 * i;                                                                 \
+    if (VECS % 256 == 0 || idx < VECS) {                                                           \
+      int key = (K0) + idx / (4 * DSTEPS);                                                         \
+      if (key > last_key) key = last_key; /* reads stay inside the request's pages */             \
+      const int kpage = table[key / page_size];                                                    \
+      kr[i] = *reinterpret_cast<const uint4*>(cache_head + (static_cast<int64_t>(kpage) * 2) * plane + \
+                                              static_cast<int64_t>(key % page_size) * D +          \
+                                              (idx % (4 * DSTEPS)) * 8);                           \
+      int vkey = (K0) + 8 * (idx & 3);                                                             \
+      if (vkey > last_key) vkey = last_key & ~7;                                                   \
+      const int vpage = table[vkey / page_size];                                                   \
+      vr[i] = *reinterpret_cast<const uint4*>(cache_head + (static_cast<int64_t>(vpage) * 2 + 1) * plane + \
+                                              static_cast<int64_t>(idx >> 2) * page_size +         \
+                                              (vkey % page_size));                                 \
+    }                                                                                              \
+  }
+
+#define TILED_STASH(BUF, K0)                                                                       \
+  _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                              \
+    const int idx = tid + 256 * i;                                                                 \
+    if (VECS % 256 == 0 || idx < VECS) {                                                           \
+      const int kk = idx / (4 * DSTEPS);                                                           \
+      const int krow = ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3);                            \
+      *reinterpret_cast<uint4*>(&k_lds[BUF][krow * KS + (idx % (4 * DSTEPS)) * 8]) = kr[i];        \
+      uint4 vv = vr[i];                                                                            \
+      const int vkey = (K0) + 8 * (idx & 3);                                                       \
+      if (vkey + 7 > last_key) vv = zero_keys_beyond(vv, vkey, last_key);                          \
+      *reinterpret_cast<uint4*>(&v_lds[BUF][(idx >> 2) * VS + (idx & 3) * 8]) = vv;                \
+    }                                                                                              \
+  }
+
+  if (k_first < key_end) {
+    TILED_FETCH(k_first)
+    TILED_STASH(0, k_first)
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = k_first; k0 < key_end; k0 += 32, buf ^= 1) {
+      const bool more = k0 + 32 < key_end;
+      if (more) { TILED_FETCH(k0 + 32) }
+      if (k0 <= wave_hi && (window <= 0 || k0 + 31 > wave_lo - window)) {
+        floatx4 s[RT][2];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ds = 0; ds < DSTEPS; ++ds)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const uint4 kf = *reinterpret_cast<const uint4*>(&k_lds[buf][(b * 16 + n) * KS + ds * 32 + g * 8]);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
+                                                                 __builtin_bit_cast(bf16x8, qf[rt][ds]),
+                                                                 s[rt][b], 0, 0, 0);
+          }
+        // lane (g, n): s[rt][b][i] is the score of key k0 + 8 g + 4 b + i for row n of tile rt
+        uint4 pf[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          float p[8];
+          float tile_max = -INFINITY;
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = k0 + 8 * g + 4 * b + i;
+              const bool masked = key > pos[rt] || (window > 0 && key <= pos[rt] - window);
+              const float v = masked ? -INFINITY : s[rt][b][i] * scale_log2e;
+              p[b * 4 + i] = v;
+              tile_max = fmaxf(tile_max, v);
+            }
+          tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, SE_WAVE));
+          tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, SE_WAVE));
+          const float new_max = fmaxf(run_max[rt], tile_max);
+          const float ref = (new_max == -INFINITY) ? 0.f : new_max;  // a row with no key yet
+          const float alpha = exp2f(run_max[rt] - ref);
+          float tile_sum = 0.f;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            p[j] = exp2f(p[j] - ref);
+            tile_sum += p[j];
+          }
+          tile_sum += __shfl_xor(tile_sum, 16, SE_WAVE);
+          tile_sum += __shfl_xor(tile_sum, 32, SE_WAVE);
+          run_sum[rt] = run_sum[rt] * alpha + tile_sum;
+          run_max[rt] = new_max;
+#pragma unroll
+          for (int db = 0; db < DBLOCKS; ++db) o[rt][db] *= alpha;
+          pf[rt].x = pack_bf16x2(p[0], p[1]);
+          pf[rt].y = pack_bf16x2(p[2], p[3]);
+          pf[rt].z = pack_bf16x2(p[4], p[5]);
+          pf[rt].w = pack_bf16x2(p[6], p[7]);
+        }
+#pragma unroll
+        for (int db = 0; db < DBLOCKS; ++db) {
+          const uint4 vf = *reinterpret_cast<const uint4*>(&v_lds[buf][(db * 16 + n) * VS + g * 8]);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
+                                                               __builtin_bit_cast(bf16x8, pf[rt]),
+                                                               o[rt][db], 0, 0, 0);
+        }
+      }
+      // the other buffer was last read in the previous step, which every wave has left
+      if (more) { TILED_STASH(buf ^ 1, k0 + 32) }
+      __syncthreads();
+    }
+  }
+#undef TILED_FETCH
+#undef TILED_STASH
+
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    if (!row_valid[rt] || !wave_active) continue;
+    const float inv = 1.f / run_sum[rt];
+    bf16_t* o_row = out + static_cast<int64_t>(token[rt]) * out_stride +
+                    static_cast<int64_t>(head[rt]) * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < DBLOCKS; ++db) {
+      uint2 packed;
+      packed.x = pack_bf16x2(o[rt][db][0] * inv, o[rt][db][1] * inv);
+      packed.y = pack_bf16x2(o[rt][db][2] * inv, o[rt][db][3] * inv);
+      *reinterpret_cast<uint2*>(o_row + db * 16) = packed;
     }
   }
 }
@@ -281,5 +562,37 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
         kv_heads, head_dim);
     SE_CHECK_LAUNCH();
   }
+  return SE_OK;
+}
+
+// Prompt portions through shared memory: units are {item, first_tile, key_begin, key_end, -, -},
+// each covering `tiles_per_block` (8) row tiles; head_dim % 32 == 0, head_dim <= 128.
+extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const void* cache,
+                                        const int32_t* block_table, int bt_stride,
+                                        const int32_t* item_meta, int num_items,
+                                        const int32_t* units, int num_units, void* out,
+                                        int64_t out_stride, int heads, int kv_heads, int head_dim,
+                                        int page_size, float scale, int window,
+                                        int tiles_per_block, hipStream_t stream) {
+  if (num_units <= 0) return SE_OK;
+  if (head_dim % 32 || head_dim <= 0 || head_dim > 128) return SE_ERR_SHAPE;
+  if (kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 8) return SE_ERR_SHAPE;
+  if (q_stride % 8 || out_stride % 4 || tiles_per_block != 8) return SE_ERR_SHAPE;
+  const float scale_log2e = scale * 1.4426950408889634f;
+  if (static_cast<int64_t>(num_units) * kv_heads > 0x7fffffff) return SE_ERR_SHAPE;
+  dim3 grid(num_units * kv_heads);
+#define SE_ATT(DS)                                                                                 \
+  case DS:                                                                                         \
+    paged_attention_tiled_kernel<DS, 2><<<grid, 256, 0, stream>>>(                                 \
+        static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(cache), block_table,  \
+        bt_stride, item_meta, num_items, units, static_cast<bf16_t*>(out), out_stride, heads,     \
+        kv_heads, page_size, scale_log2e, window);                                                 \
+    break;
+  switch (head_dim / 32) {
+    SE_ATT(1) SE_ATT(2) SE_ATT(3) SE_ATT(4)
+    default: return SE_ERR_SHAPE;
+  }
+#undef SE_ATT
+  SE_CHECK_LAUNCH();
   return SE_OK;
 }

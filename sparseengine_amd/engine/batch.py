@@ -144,7 +144,8 @@ class BatchBuilder:
             from ..kernels.attention_work import build_attention_work
             for group in cache.groups:
                 for ratio, window in sorted(self.attention_shapes.get(group.index, ())):
-                    work = build_attention_work(q_len, ctx_len, ratio, group.request.kv_heads, window)
+                    work = build_attention_work(q_len, ctx_len, ratio, group.request.kv_heads, window,
+                                                head_dim=group.request.head_dim)
                     works.append((group.index, (ratio, window), work, len(parts)))
                     parts += [work.units.reshape(-1), work.tasks.reshape(-1)]
         total = sum(p.size for p in parts)
@@ -183,5 +184,5 @@ class BatchBuilder:
         for group_index, key, work, at in works:
             fb.groups[group_index].work[key] = (view(at, work.units.shape), work.units.shape[0],
                                                 view(at + 1, work.tasks.shape), work.tasks.shape[0],
-                                                work.num_slots)
+                                                work.num_slots, work.tiles_per_block)
         return fb

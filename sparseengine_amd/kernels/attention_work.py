@@ -1,8 +1,10 @@
-"""Work list of the matrix-core attention kernel (host side, numpy).
+"""Work list of the matrix-core attention kernels (host side, numpy).
 
 For one step and one (query heads per kv head) ratio: the rows of every item are cut into tiles
-of 16; when the step has too few tiles to fill the chip, every tile's keys are cut into equal
-ranges (multiples of 32 keys) and a merge task per tile combines them.
+of 16.  A step with enough tiles to fill the chip (prompt portions) goes to the kernel that shares
+keys and values through shared memory: a unit is a run of ``TILES_PER_BLOCK`` tiles of one item.
+A step with few tiles (decoding) goes to the kernel with one wavefront per unit: every tile's keys
+are cut into equal ranges (multiples of 32 keys) and a merge task per tile combines them.
 """
 from __future__ import annotations
 
@@ -15,6 +17,8 @@ TASK_FIELDS = 4      # item, row_tile, first_slot, num_splits
 TARGET_WAVES = 2048  # wavefronts wanted in flight (256 CUs x 4 SIMDs x 2)
 MIN_SPLIT_KEYS = 64
 MAX_SPLITS = 256      # what the merge kernel's shared memory holds
+TILES_PER_BLOCK = 8   # row tiles of one block of the shared-memory kernel
+TILED_MAX_HEAD_DIM = 128
 
 
 @dataclass
@@ -22,15 +26,34 @@ class AttentionWork:
     units: np.ndarray        # int32 [num_units, UNIT_FIELDS]
     tasks: np.ndarray        # int32 [num_tasks, TASK_FIELDS]
     num_slots: int
+    tiles_per_block: int = 0  # 0: units are (tile, key range) for one wavefront each; else runs of tiles for a block
 
 
 def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int = 0,
-                         target_waves: int = TARGET_WAVES) -> AttentionWork:
+                         target_waves: int = TARGET_WAVES, head_dim: int = 0) -> AttentionWork:
+    """``head_dim``: 0 keeps every step on the one-wavefront kernel (callers that do not know it)."""
     q_len = np.asarray(q_len, dtype=np.int64)
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
     tiles = (q_len * group + 15) // 16
     waves = int(tiles.sum()) * kv_heads
     want = 1 if waves >= target_waves else -(-target_waves // max(waves, 1))
+    if want == 1 and head_dim and head_dim % 32 == 0 and head_dim <= TILED_MAX_HEAD_DIM:
+        blocks = []
+        pos0 = ctx_len - q_len
+        for item, (n_tiles, ctx) in enumerate(zip(tiles.tolist(), ctx_len.tolist())):
+            first = np.arange(0, n_tiles, TILES_PER_BLOCK, dtype=np.int32)
+            block = np.zeros((first.size, UNIT_FIELDS), dtype=np.int32)
+            block[:, 0], block[:, 1], block[:, 2], block[:, 3], block[:, 4] = item, first, 0, ctx, -1
+            blocks.append(block)
+        units = np.concatenate(blocks) if blocks else np.zeros((0, UNIT_FIELDS), np.int32)
+        # longest first: a block's work grows with the position of its rows, and the blocks that are
+        # started last decide when the kernel ends
+        reach = pos0[units[:, 0]] + ((units[:, 1].astype(np.int64) + TILES_PER_BLOCK) * 16 - 1) // group
+        keys = np.minimum(reach + 1, ctx_len[units[:, 0]])
+        if window:
+            keys = np.minimum(keys, window + TILES_PER_BLOCK * 16 // group + 1)
+        units = units[np.argsort(-keys, kind="stable")]
+        return AttentionWork(units, np.zeros((0, TASK_FIELDS), np.int32), 0, TILES_PER_BLOCK)
     units, tasks, slot = [], [], 0
     for item, (n_tiles, ctx) in enumerate(zip(tiles.tolist(), ctx_len.tolist())):
         reach = min(ctx, window + int(q_len[item])) if window else ctx     # keys a tile can read

@@ -72,6 +72,11 @@ _SIGNATURES = {
         "se_paged_attention_mfma": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                     c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+        # q, q_stride, cache, block_table, bt_stride, item_meta, num_items, units, num_units, out,
+        # out_stride, heads, kv_heads, head_dim, page_size, scale, window, tiles_per_block, stream
+        "se_paged_attention_tiled": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                     c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int,
+                                     c_float, c_int, c_int, c_void_p],
     },
     "moe": {
         "se_router_topk": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -271,12 +276,23 @@ class HipKernels:
         work = None if getattr(meta, "work", None) is None else meta.work.get((group, window))
         if work is None:                      # not prepared by the batch builder: build it here
             from .attention_work import build_attention_work
-            host = build_attention_work(meta.item_q_len, meta.item_ctx_len, group, kv_heads, window)
+            host = build_attention_work(meta.item_q_len, meta.item_ctx_len, group, kv_heads, window,
+                                        head_dim=head_dim)
             work = (torch.from_numpy(host.units).to(q.device), host.units.shape[0],
-                    torch.from_numpy(host.tasks).to(q.device), host.tasks.shape[0], host.num_slots)
+                    torch.from_numpy(host.tasks).to(q.device), host.tasks.shape[0], host.num_slots,
+                    host.tiles_per_block)
             if getattr(meta, "work", None) is not None:
                 meta.work[(group, window)] = work
-        units, num_units, tasks, num_tasks, num_slots = work
+        units, num_units, tasks, num_tasks, num_slots, tiles_per_block = work
+        num_items = meta.item_meta.shape[1]
+        _require(meta.item_meta.dtype == torch.int32 and meta.item_meta.is_contiguous(), "item_meta layout")
+        if tiles_per_block:                   # prompt portions: keys and values shared by a block
+            _check(_fn.get("attention_mfma", "se_paged_attention_tiled")(
+                _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
+                _ptr(meta.item_meta), num_items, _ptr(units), num_units, _ptr(out), out.stride(0), heads,
+                kv_heads, head_dim, page_size, float(scale), window, tiles_per_block, _stream()),
+                "paged_attention (tiled)")
+            return
         part_o = part_ml = None
         if num_slots:
             need = num_slots * kv_heads * 16
@@ -287,8 +303,6 @@ class HipKernels:
             if part_ml.numel() < need * 2:
                 part_ml = torch.empty(need * 2, dtype=torch.float32, device=q.device)
                 self._attention_partials = (part_o, part_ml)
-        num_items = meta.item_meta.shape[1]
-        _require(meta.item_meta.dtype == torch.int32 and meta.item_meta.is_contiguous(), "item_meta layout")
         _check(_fn.get("attention_mfma", "se_paged_attention_mfma")(
             _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
             _ptr(meta.item_meta), num_items, _ptr(units), num_units, _ptr(tasks) if num_tasks else None,

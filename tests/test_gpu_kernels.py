@@ -413,6 +413,38 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
         torch.testing.assert_close(out_h[t].float(), ref, rtol=1.6e-2, atol=1.6e-2)
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page,window,lens,q_lens", [
+    (48, 8, 128, 64, 0, [900, 1300, 301], [900, 411, 1]),        # a whole prompt, a portion on a prefix, a decoded token
+    (32, 16, 96, 16, 0, [800, 500], [800, 300]),
+    (16, 8, 64, 32, 70, [1500, 900], [1500, 600]),               # window shorter than the portions
+    (8, 8, 32, 8, 0, [4200], [4200]),
+    (48, 8, 128, 64, 0, [2048 + 17], [2048 + 17]),
+    (12, 2, 128, 16, 300, [5000, 3000], [4100, 2001])])
+def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, page, window, lens, q_lens):
+    """Steps with many rows: blocks share each step's keys and values through shared memory."""
+    dtype = torch.bfloat16
+    cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=heads + head_dim)
+    # a page's slots past a request's end may hold anything an earlier owner left, even NaN
+    last_page = int(table[0, (lens[0] - 1) // page])
+    if lens[0] % page:
+        cache[last_page, 0, :, lens[0] % page:, :] = float("nan")
+        cache[last_page, 1].view(kv_heads, head_dim, page)[:, :, lens[0] % page:] = float("nan")
+    meta = make_meta(table, lens, q_lens)
+    T = sum(q_lens)
+    q = randn(T, heads, head_dim, dtype=dtype, seed=3)
+    scale = head_dim ** -0.5
+    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device="cuda")
+    out_t = torch.empty_like(out_h)
+    hip.paged_attention(q, cache, meta, out_h, scale, window)
+    assert meta.work[(heads // kv_heads, window)][5] == 8, "expected the shared-memory kernel"
+    twin.paged_attention(q, cache, meta, out_t, scale, window)
+    torch.testing.assert_close(out_h, out_t, **tol(dtype))
+    for t in sorted({0, 1, 15, 16, q_lens[0] - 1, min(q_lens[0], T - 1), T // 2, T - 1}):
+        row, pos = int(meta.token_row[t]), int(meta.positions[t])
+        ref = dense_attention(q[t], cache, table, row, pos, scale, window, page)
+        torch.testing.assert_close(out_h[t].float(), ref, **tol(dtype))
+
+
 @pytest.mark.parametrize("rows,n,k", [(1, 8192, 3072), (8, 3072, 6144), (16, 256, 128), (17, 48, 256), (33, 1024, 384),
                                       (64, 200064, 3072), (5, 50, 128), (3, 64, 96)])
 def test_skinny_linear(hip, rows, n, k):
