@@ -1,6 +1,7 @@
-// Paged causal GQA attention on the matrix cores (bfloat16) for gfx950: one kernel for portions
-// of prompts and for single decoded tokens, with split keys where a step has too few rows to
-// fill the chip, and a merge kernel for the splits.
+// Paged causal GQA attention on the matrix cores (bfloat16) for gfx950.  Two kernels share one
+// formulation: one wavefront per unit, with split keys and a merge kernel, for steps with few rows
+// (decoding, short portions); blocks that share keys and values through shared memory for steps
+// with many rows (prompt portions).  The host's work list decides which one a step takes.
 //
 // A *row* is one (query token, query head) pair.  For one request and one kv head the rows
 // (q_len * group of them, ordered token-major) are cut into tiles of 16; a work unit is one tile
@@ -254,16 +255,102 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 
 // Prompt portions: the same product with the keys and values of a step shared by a whole block.
 // A block of four wavefronts takes 4 * RT consecutive row tiles of one request and one kv head
-// (wave w the tiles first + w * RT ...), brings each step of 32 keys into shared memory once
-// (two buffers: the loads of the next step are in flight while this one is computed) and every
-// wave reads its operands from there, each operand feeding RT products.  The per-wave kernel above
-// reads every key once per 16 rows, which binds a long prompt to the L2's bandwidth.
+// (wave w the tiles first + w * RT ...).  Each step of 32 keys is brought into shared memory once,
+// by loads that go from the cache straight into shared memory (no register in between), NS - 1
+// steps ahead of the step that is being computed; every wave reads its operands from there and
+// each operand feeds RT products.  The one-wavefront kernel above reads every key once per 16
+// rows, which binds a long prompt to the L2's bandwidth and to the latency of each step's loads.
 //
-// Shared layout: keys in operand order (row b * 16 + m holds key 8 * (m / 4) + m % 4 + 4 * b of
-// the step), row stride D + 8 elements; values [dim][32 keys], row stride 40 elements: the 16
-// lanes of a quarter wave then touch 16 different groups of four banks.
+// Such a load writes lane l's 16 bytes at (wave-uniform base) + 16 l, so shared memory holds
+// *operands*: one chunk of 1024 bytes per (key block b, 32 dims ds) and per 16 value dims db, in
+// which lane l's piece is exactly what lane l feeds the matrix core.  Reads are then conflict-free.
+// The compiler does not see these writes; the waits for them (vmcnt) are placed by hand, and the
+// barrier is a bare s_barrier: the usual fence would wait for every load in flight.
+// The request's page ids for the block's keys are copied to shared memory first (at most
+// TILED_MAX_PAGES), so that no load in the loop depends on another.
 // A unit is {item, first_tile, key_begin, key_end, -, -}; it always writes the output itself.
-template <int DSTEPS, int RT>
+#define TILED_MAX_PAGES 2048
+#define TILED_ROW_TILES 2   // row tiles per wavefront: 8 per block
+#define TILED_STAGES 3      // steps of keys in shared memory at a time
+
+// m0 (the destination's base) is set and used inside one statement; naming it as clobbered draws a
+// warning about reserved registers that does not apply here.
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void load16_to_lds(const void* src, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)   // the base is the same in all lanes
+               : "memory", "m0");
+}
+
+// Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 that share a row: two register swaps
+// between halves and between rows of 16 lanes instead of trips through the shared-memory crossbar.
+__device__ __forceinline__ float quad_max(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const uint32_t w = __float_as_uint(v);
+  const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_sum(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const uint32_t w = __float_as_uint(v);
+  const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2_rne(float lo, float hi) {   // one v_cvt_pk_bf16_f32
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{lo, hi}, bf16x2));
+}
+
+// Online softmax of one step for the wave's RT tiles (float, base 2).  The reference maximum of a
+// row is only raised when the step's maximum exceeds it by more than SOFTMAX_SLACK (probabilities
+// may then reach 2^SLACK, which float sums and bfloat16 operands hold as well as values below 1):
+// the rescaling of the accumulators, the costly part, becomes rare.  A row's sum is kept per
+// lane and added up over its four lanes at the end.
+#define SOFTMAX_SLACK 8.f
+#define TILED_SOFTMAX(MASKED)                                                                      \
+  _Pragma("unroll") for (int rt = 0; rt < RT; ++rt) {                                              \
+    float v[8];                                                                                    \
+    _Pragma("unroll") for (int b = 0; b < 2; ++b)                                                  \
+      _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                              \
+        float x = s[rt][b][i];                                                                     \
+        if (MASKED) {                                                                              \
+          const int key = k0 + 8 * g + 4 * b + i;                                                  \
+          if (key > pos[rt] || (window > 0 && key <= pos[rt] - window)) x = -INFINITY;             \
+        }                                                                                          \
+        v[b * 4 + i] = x;                                                                          \
+      }                                                                                            \
+    float m = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])),                                   \
+                    fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));                                  \
+    m = quad_max(m) * scale_log2e; /* scale > 0: the maximum commutes with it */                   \
+    const bool grow = m > run_max[rt] + SOFTMAX_SLACK || (run_max[rt] == -INFINITY && m > -INFINITY); \
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(grow) != 0, 0)) {                             \
+      const float alpha = grow ? __builtin_amdgcn_exp2f(run_max[rt] - m) : 1.f;                    \
+      if (grow) run_max[rt] = m;                                                                   \
+      run_sum[rt] *= alpha;                                                                        \
+      _Pragma("unroll") for (int db = 0; db < DBLOCKS; ++db) o[rt][db] *= alpha;                   \
+    }                                                                                              \
+    /* a row whose keys are all masked so far has no reference yet; its probabilities are 0 */     \
+    const float ref = (MASKED && run_max[rt] == -INFINITY) ? 0.f : run_max[rt];                    \
+    float sum = 0.f;                                                                               \
+    _Pragma("unroll") for (int j = 0; j < 8; ++j) {                                                \
+      v[j] = __builtin_amdgcn_exp2f(fmaf(v[j], scale_log2e, -ref));                                \
+      sum += v[j];                                                                                 \
+    }                                                                                              \
+    run_sum[rt] += sum;                                                                            \
+    pf[rt].x = pack_bf16x2_rne(v[0], v[1]);                                                        \
+    pf[rt].y = pack_bf16x2_rne(v[2], v[3]);                                                        \
+    pf[rt].z = pack_bf16x2_rne(v[4], v[5]);                                                        \
+    pf[rt].w = pack_bf16x2_rne(v[6], v[7]);                                                        \
+  }
+
+template <int DSTEPS, int RT, int NS>
 __global__ void __launch_bounds__(256)
 paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                              const bf16_t* __restrict__ cache,
@@ -274,12 +361,9 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                              float scale_log2e, int window) {
   constexpr int D = 32 * DSTEPS;
   constexpr int DBLOCKS = 2 * DSTEPS;
-  constexpr int KS = D + 8;                       // key row stride in shared memory (elements)
-  constexpr int VS = 40;                          // value row stride
-  constexpr int VECS = 128 * DSTEPS;              // 16-byte vectors of a step's keys (and of its values)
-  constexpr int LOADS = (VECS + 255) / 256;
-  __shared__ __align__(16) bf16_t k_lds[2][32 * KS];
-  __shared__ __align__(16) bf16_t v_lds[2][D * VS];
+  constexpr int CHUNKS = 4 * DSTEPS;              // per step: 2 * DSTEPS of keys, then 2 * DSTEPS of values
+  __shared__ __align__(16) uint4 stage[NS][CHUNKS][64];
+  __shared__ int32_t page_ids[TILED_MAX_PAGES];
 
   const int tid = threadIdx.x;
   const int lane = tid & (SE_WAVE - 1);
@@ -312,6 +396,16 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   const int wave_hi = wave_active ? pos0 + wave_last_row / group : -1;          // largest position
   const int wave_lo = wave_active ? pos0 + (tile0 * 16) / group : 0;            // smallest position
 
+  const int32_t* table = block_table + static_cast<int64_t>(item) * bt_stride;
+  const int kmax = key_end - 1;                    // loads are clamped to the block's last key
+  // The page ids of the block's keys, as many as fit; a longer range is brought in window by
+  // window as the steps reach it (a very long context on small pages).
+  int window_base = k_first / page_size;          // first page held in page_ids
+  const int last_page = kmax / page_size;
+  if (k_first < key_end) {
+    const int pages = min(last_page - window_base + 1, TILED_MAX_PAGES);
+    for (int i = tid; i < pages; i += 256) page_ids[i] = table[window_base + i];
+  }
   int token[RT], head[RT], pos[RT];
   bool row_valid[RT];
   uint4 qf[RT][DSTEPS];
@@ -330,7 +424,6 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     for (int ds = 0; ds < DSTEPS; ++ds) qf[rt][ds] = *reinterpret_cast<const uint4*>(q_row + ds * 32);
   }
 
-  const int32_t* table = block_table + static_cast<int64_t>(item) * bt_stride;
   const int64_t head_span = static_cast<int64_t>(page_size) * D;
   const int64_t plane = static_cast<int64_t>(kv_heads) * head_span;
   const bf16_t* cache_head = cache + kvh * head_span;
@@ -344,51 +437,71 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) o[rt][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
+  __syncthreads();   // page ids are in place
+  // The query operands must have arrived before the loop: a wait for them inside it would also
+  // wait for the loads into shared memory that were issued just before.
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ds = 0; ds < DSTEPS; ++ds)
+      asm volatile("" : "+v"(qf[rt][ds].x), "+v"(qf[rt][ds].y), "+v"(qf[rt][ds].z), "+v"(qf[rt][ds].w));
 
-  uint4 kr[LOADS], vr[LOADS];   // a step's vectors on their way from the cache to shared memory
+  // Waves 0 and 1 bring the two key blocks of a step, waves 2 and 3 one half of the value dims each.
+  const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&stage[0][0][0]));
+  auto issue = [&](int step) {
+    const int k0 = k_first + 32 * step;
+    const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS) * 1024u;
+    if (wave < 2) {
+      int key = k0 + 8 * (n >> 2) + (n & 3) + 4 * wave;
+      if (key > kmax) key = kmax;
+      const int page = page_ids[key / page_size - window_base];
+      const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2) * plane +
+                          static_cast<int64_t>(key % page_size) * D + g * 8;
+#pragma unroll
+      for (int ds = 0; ds < DSTEPS; ++ds)
+        load16_to_lds(src + ds * 32, dst + static_cast<uint32_t>(wave * DSTEPS + ds) * 1024u);
+    } else {
+      const int half = wave - 2;
+      int vkey = k0 + 8 * g;
+      if (vkey > kmax) vkey = kmax & ~7;
+      const int page = page_ids[vkey / page_size - window_base];
+      const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2 + 1) * plane +
+                          static_cast<int64_t>(half * DSTEPS * 16 + n) * page_size + (vkey % page_size);
+#pragma unroll
+      for (int j = 0; j < DSTEPS; ++j)
+        load16_to_lds(src + static_cast<int64_t>(j) * 16 * page_size,
+                      dst + static_cast<uint32_t>(2 * DSTEPS + half * DSTEPS + j) * 1024u);
+    }
+  };
 
-#define TILED_FETCH(K0)                                                                            \
-  _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                              \
-    const int idx = tid + 256 * i;                                                                 \
-    if (VECS % 256 == 0 || idx < VECS) {                                                           \
-      int key = (K0) + idx / (4 * DSTEPS);                                                         \
-      if (key > last_key) key = last_key; /* reads stay inside the request's pages */             \
-      const int kpage = table[key / page_size];                                                    \
-      kr[i] = *reinterpret_cast<const uint4*>(cache_head + (static_cast<int64_t>(kpage) * 2) * plane + \
-                                              static_cast<int64_t>(key % page_size) * D +          \
-                                              (idx % (4 * DSTEPS)) * 8);                           \
-      int vkey = (K0) + 8 * (idx & 3);                                                             \
-      if (vkey > last_key) vkey = last_key & ~7;                                                   \
-      const int vpage = table[vkey / page_size];                                                   \
-      vr[i] = *reinterpret_cast<const uint4*>(cache_head + (static_cast<int64_t>(vpage) * 2 + 1) * plane + \
-                                              static_cast<int64_t>(idx >> 2) * page_size +         \
-                                              (vkey % page_size));                                 \
-    }                                                                                              \
-  }
-
-#define TILED_STASH(BUF, K0)                                                                       \
-  _Pragma("unroll") for (int i = 0; i < LOADS; ++i) {                                              \
-    const int idx = tid + 256 * i;                                                                 \
-    if (VECS % 256 == 0 || idx < VECS) {                                                           \
-      const int kk = idx / (4 * DSTEPS);                                                           \
-      const int krow = ((kk >> 2) & 1) * 16 + (kk >> 3) * 4 + (kk & 3);                            \
-      *reinterpret_cast<uint4*>(&k_lds[BUF][krow * KS + (idx % (4 * DSTEPS)) * 8]) = kr[i];        \
-      uint4 vv = vr[i];                                                                            \
-      const int vkey = (K0) + 8 * (idx & 3);                                                       \
-      if (vkey + 7 > last_key) vv = zero_keys_beyond(vv, vkey, last_key);                          \
-      *reinterpret_cast<uint4*>(&v_lds[BUF][(idx >> 2) * VS + (idx & 3) * 8]) = vv;                \
-    }                                                                                              \
-  }
-
-  if (k_first < key_end) {
-    TILED_FETCH(k_first)
-    TILED_STASH(0, k_first)
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = k_first; k0 < key_end; k0 += 32, buf ^= 1) {
-      const bool more = k0 + 32 < key_end;
-      if (more) { TILED_FETCH(k0 + 32) }
+  const int nsteps = (key_end - k_first + 31) / 32;
+  if (nsteps > 0) {
+#pragma unroll
+    for (int j = 0; j < NS - 1; ++j)
+      if (j < nsteps) issue(j);
+    for (int step = 0; step < nsteps; ++step) {
+      const int k0 = k_first + 32 * step;
+      // this step's data: all but the loads of the NS - 2 steps after it must have come back
+      if (step + NS - 2 < nsteps) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | ((NS - 2) * DSTEPS));     // vmcnt((NS - 2) * DSTEPS)
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                           // vmcnt(0)
+      }
+      __builtin_amdgcn_s_barrier();   // everyone's part of the step is in; everyone has left step - 1
+      asm volatile("" ::: "memory");
+      if (step + NS - 1 < nsteps) {
+        const int k_next = k_first + 32 * (step + NS - 1);
+        if (min(k_next + 31, kmax) / page_size >= window_base + TILED_MAX_PAGES) {
+          // nobody reads page_ids between the barrier above and its own issue below
+          window_base = k_next / page_size;
+          const int pages = min(last_page - window_base + 1, TILED_MAX_PAGES);
+          for (int i = tid; i < pages; i += 256) page_ids[i] = table[window_base + i];
+          __syncthreads();
+        }
+        issue(step + NS - 1);   // into the buffer that step - 1 has used
+      }
       if (k0 <= wave_hi && (window <= 0 || k0 + 31 > wave_lo - window)) {
+        const uint4(*buf)[64] = stage[step % NS];
         floatx4 s[RT][2];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -396,54 +509,30 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
         for (int ds = 0; ds < DSTEPS; ++ds)
 #pragma unroll
           for (int b = 0; b < 2; ++b) {
-            const uint4 kf = *reinterpret_cast<const uint4*>(&k_lds[buf][(b * 16 + n) * KS + ds * 32 + g * 8]);
+            const uint4 kf = buf[b * DSTEPS + ds][lane];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
               s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
                                                                  __builtin_bit_cast(bf16x8, qf[rt][ds]),
                                                                  s[rt][b], 0, 0, 0);
           }
-        // lane (g, n): s[rt][b][i] is the score of key k0 + 8 g + 4 b + i for row n of tile rt
+        // lane (g, n): s[rt][b][i] is the score of key k0 + 8 g + 4 b + i for row n of tile rt.
+        // Most steps lie wholly inside every row's range of keys and need no mask.
         uint4 pf[RT];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          float p[8];
-          float tile_max = -INFINITY;
-#pragma unroll
-          for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int key = k0 + 8 * g + 4 * b + i;
-              const bool masked = key > pos[rt] || (window > 0 && key <= pos[rt] - window);
-              const float v = masked ? -INFINITY : s[rt][b][i] * scale_log2e;
-              p[b * 4 + i] = v;
-              tile_max = fmaxf(tile_max, v);
-            }
-          tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, SE_WAVE));
-          tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, SE_WAVE));
-          const float new_max = fmaxf(run_max[rt], tile_max);
-          const float ref = (new_max == -INFINITY) ? 0.f : new_max;  // a row with no key yet
-          const float alpha = exp2f(run_max[rt] - ref);
-          float tile_sum = 0.f;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            p[j] = exp2f(p[j] - ref);
-            tile_sum += p[j];
-          }
-          tile_sum += __shfl_xor(tile_sum, 16, SE_WAVE);
-          tile_sum += __shfl_xor(tile_sum, 32, SE_WAVE);
-          run_sum[rt] = run_sum[rt] * alpha + tile_sum;
-          run_max[rt] = new_max;
-#pragma unroll
-          for (int db = 0; db < DBLOCKS; ++db) o[rt][db] *= alpha;
-          pf[rt].x = pack_bf16x2(p[0], p[1]);
-          pf[rt].y = pack_bf16x2(p[2], p[3]);
-          pf[rt].z = pack_bf16x2(p[4], p[5]);
-          pf[rt].w = pack_bf16x2(p[6], p[7]);
+        if (k0 + 31 > wave_lo || (window > 0 && k0 <= wave_hi - window)) {
+          TILED_SOFTMAX(1)
+        } else {
+          TILED_SOFTMAX(0)
         }
+        // the block's last step may hold slots past the request's last key: whatever an earlier owner
+        // of the page left there, possibly not finite.  The loader's clamping is repeated here.
+        const bool tail = k0 + 31 > kmax;
+        int vkey = k0 + 8 * g;
+        if (vkey > kmax) vkey = kmax & ~7;
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db) {
-          const uint4 vf = *reinterpret_cast<const uint4*>(&v_lds[buf][(db * 16 + n) * VS + g * 8]);
+          uint4 vf = buf[2 * DSTEPS + db][lane];
+          if (tail) vf = zero_keys_beyond(vf, vkey, last_key);
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt)
             o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
@@ -451,18 +540,15 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                                                                o[rt][db], 0, 0, 0);
         }
       }
-      // the other buffer was last read in the previous step, which every wave has left
-      if (more) { TILED_STASH(buf ^ 1, k0 + 32) }
-      __syncthreads();
+      asm volatile("" ::: "memory");
     }
   }
-#undef TILED_FETCH
-#undef TILED_STASH
 
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
+    const float total = quad_sum(run_sum[rt]);   // every lane takes part
     if (!row_valid[rt] || !wave_active) continue;
-    const float inv = 1.f / run_sum[rt];
+    const float inv = 1.f / total;
     bf16_t* o_row = out + static_cast<int64_t>(token[rt]) * out_stride +
                     static_cast<int64_t>(head[rt]) * D + 4 * g;
 #pragma unroll
@@ -577,13 +663,13 @@ extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const v
   if (num_units <= 0) return SE_OK;
   if (head_dim % 32 || head_dim <= 0 || head_dim > 128) return SE_ERR_SHAPE;
   if (kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 8) return SE_ERR_SHAPE;
-  if (q_stride % 8 || out_stride % 4 || tiles_per_block != 8) return SE_ERR_SHAPE;
+  if (q_stride % 8 || out_stride % 4 || tiles_per_block != 4 * TILED_ROW_TILES) return SE_ERR_SHAPE;
   const float scale_log2e = scale * 1.4426950408889634f;
   if (static_cast<int64_t>(num_units) * kv_heads > 0x7fffffff) return SE_ERR_SHAPE;
   dim3 grid(num_units * kv_heads);
 #define SE_ATT(DS)                                                                                 \
   case DS:                                                                                         \
-    paged_attention_tiled_kernel<DS, 2><<<grid, 256, 0, stream>>>(                                 \
+    paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES><<<grid, 256, 0, stream>>>(          \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(cache), block_table,  \
         bt_stride, item_meta, num_items, units, static_cast<bf16_t*>(out), out_stride, heads,     \
         kv_heads, page_size, scale_log2e, window);                                                 \

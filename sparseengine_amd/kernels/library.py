@@ -27,6 +27,16 @@ HIPCC_FLAGS = [
     "-O3", f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC", "-std=c++17", "-Wno-pass-failed",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# Per source.  The attention kernels keep their accumulators in ordinary vector registers: left to
+# itself the compiler parks them in the accumulation registers and copies all of them to and fro
+# in every step of the key loop, which costs more instructions than the step's own arithmetic.
+EXTRA_FLAGS = {
+    "attention_mfma": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
+def _flags(name: str) -> list[str]:
+    return HIPCC_FLAGS + EXTRA_FLAGS.get(name, [])
 
 
 class KernelLibraryError(RuntimeError):
@@ -35,7 +45,7 @@ class KernelLibraryError(RuntimeError):
 
 def _digest(name: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(_flags(name)).encode())
     for path in [CSRC / f"{name}.hip"] + sorted(CSRC.glob("*.h")):
         h.update(path.name.encode())
         h.update(path.read_bytes())
@@ -102,7 +112,7 @@ def build(names=None, force: bool = False, verbose: bool = True) -> dict[str, Pa
         out_dir = out_dir or _writable_dir()
         target = out_dir / f"{name}.{_digest(name)}.so"
         partial = out_dir / f".{name}.{os.getpid()}.tmp.so"
-        cmd = [hipcc, *HIPCC_FLAGS, "-o", str(partial), str(CSRC / f"{name}.hip")]
+        cmd = [hipcc, *_flags(name), "-o", str(partial), str(CSRC / f"{name}.hip")]
         proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         jobs.append((name, proc, partial, target))
     if jobs and verbose:

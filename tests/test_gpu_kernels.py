@@ -419,7 +419,8 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     (16, 8, 64, 32, 70, [1500, 900], [1500, 600]),               # window shorter than the portions
     (8, 8, 32, 8, 0, [4200], [4200]),
     (48, 8, 128, 64, 0, [2048 + 17], [2048 + 17]),
-    (12, 2, 128, 16, 300, [5000, 3000], [4100, 2001])])
+    (12, 2, 128, 16, 300, [5000, 3000], [4100, 2001]),
+    (8, 8, 32, 8, 0, [17000], [4100])])                          # more pages than the kernel keeps ids of at once
 def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, page, window, lens, q_lens):
     """Steps with many rows: blocks share each step's keys and values through shared memory."""
     dtype = torch.bfloat16
