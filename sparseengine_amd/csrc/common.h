@@ -57,16 +57,93 @@ __device__ __forceinline__ float round_to(float v) {
   return to_float(from_float<T>(v));
 }
 
+// Exchange steps of a reduction over the 64 lanes of a wavefront, all inside the vector unit:
+// neighbours within four lanes, mirrors within 8 and 16 lanes (after the earlier steps all lanes
+// of a group hold the same value, so a mirror is as good as an exchange), then swaps between
+// rows of 16 and between halves.  Shuffles through the shared-memory crossbar cost a memory
+// latency apiece, and a reduction is six of them in a row.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, false));
+}
+#define SE_DPP_XOR1 0xB1          // quad_perm [1, 0, 3, 2]
+#define SE_DPP_XOR2 0x4E          // quad_perm [2, 3, 0, 1]
+#define SE_DPP_HALF_MIRROR 0x141  // lane i <-> 7 - i within 8
+#define SE_DPP_MIRROR 0x140       // lane i <-> 15 - i within 16
+
+__device__ __forceinline__ uint32_t word_of(float v) { return __float_as_uint(v); }
+__device__ __forceinline__ uint32_t word_of(int v) { return static_cast<uint32_t>(v); }
+__device__ __forceinline__ void word_to(uint32_t w, float& v) { v = __uint_as_float(w); }
+__device__ __forceinline__ void word_to(uint32_t w, int& v) { v = static_cast<int>(w); }
+
+// `op(a, b)` must be commutative and associative up to rounding; every lane gets the result.
+// T is float or int.
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_reduce(T v, Op op) {
+  T o;
+  word_to(dpp_move<SE_DPP_XOR1>(word_of(v)), o);
+  v = op(v, o);
+  word_to(dpp_move<SE_DPP_XOR2>(word_of(v)), o);
+  v = op(v, o);
+  word_to(dpp_move<SE_DPP_HALF_MIRROR>(word_of(v)), o);
+  v = op(v, o);
+  word_to(dpp_move<SE_DPP_MIRROR>(word_of(v)), o);
+  v = op(v, o);
+  const auto rows = __builtin_amdgcn_permlane16_swap(word_of(v), word_of(v), false, false);
+  word_to(rows[0], v);
+  word_to(rows[1], o);
+  v = op(v, o);
+  const auto halves = __builtin_amdgcn_permlane32_swap(word_of(v), word_of(v), false, false);
+  word_to(halves[0], v);
+  word_to(halves[1], o);
+  return op(v, o);
+}
+
+// The same for a (value, index) pair.  `take_other(v, i, ov, oi)` says whether the other pair
+// wins; it must order distinct pairs strictly, so that both sides of an exchange agree.
+template <typename Better>
+__device__ __forceinline__ void wave_reduce_pair(float& v, int& i, Better take_other) {
+  auto step = [&](float ov, int oi) {
+    if (take_other(v, i, ov, oi)) {
+      v = ov;
+      i = oi;
+    }
+  };
+#define SE_PAIR_DPP(CTRL) \
+  step(__uint_as_float(dpp_move<CTRL>(__float_as_uint(v))), static_cast<int>(dpp_move<CTRL>(static_cast<uint32_t>(i))))
+  SE_PAIR_DPP(SE_DPP_XOR1);
+  SE_PAIR_DPP(SE_DPP_XOR2);
+  SE_PAIR_DPP(SE_DPP_HALF_MIRROR);
+  SE_PAIR_DPP(SE_DPP_MIRROR);
+#undef SE_PAIR_DPP
+  {
+    const uint32_t a = __float_as_uint(v), b = static_cast<uint32_t>(i);
+    const auto va = __builtin_amdgcn_permlane16_swap(a, a, false, false);
+    const auto ia = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+    v = __uint_as_float(va[0]);
+    i = static_cast<int>(ia[0]);
+    step(__uint_as_float(va[1]), static_cast<int>(ia[1]));
+  }
+  {
+    const uint32_t a = __float_as_uint(v), b = static_cast<uint32_t>(i);
+    const auto va = __builtin_amdgcn_permlane32_swap(a, a, false, false);
+    const auto ia = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+    v = __uint_as_float(va[0]);
+    i = static_cast<int>(ia[0]);
+    step(__uint_as_float(va[1]), static_cast<int>(ia[1]));
+  }
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = SE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, SE_WAVE);
-  return v;
+  return wave_reduce(v, [](float a, float b) { return a + b; });
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = SE_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, SE_WAVE));
-  return v;
+  return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); });
+}
+
+__device__ __forceinline__ int wave_sum(int v) {
+  return wave_reduce(v, [](int a, int b) { return a + b; });
 }
 
 // Sum over a whole block of up to 1024 threads; every thread gets the result.
@@ -111,22 +188,24 @@ struct Vec16<bf16_t> {
   }
 };
 
-// Bring n elements (n % Vec16<T>::N == 0, 16-byte aligned) into shared memory as float with a block
-// of 256 threads.  Every load is issued before the first one is used: a row is a handful of
-// vectors per thread, and a loop that waits for each load in turn costs a memory latency apiece.
+// Bring n elements (n % Vec16<T>::N == 0, 16-byte aligned, n <= MAXV * 256 vectors) into shared
+// memory as float with a block of at least 256 threads.  Every load is issued before the first one
+// is used: a row is a handful of vectors per thread, and a loop that waits for each load in turn
+// costs a memory latency apiece.
 template <typename T, int MAXV>
 __device__ __forceinline__ void stage_row(const T* src, float* dst, int n) {
   constexpr int VN = Vec16<T>::N;
   const int nvec = n / VN;
+  const int threads = blockDim.x;
   Vec16<T> v[MAXV];
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
-    const int idx = threadIdx.x + i * 256;
+    const int idx = threadIdx.x + i * threads;
     if (idx < nvec) v[i].v = *reinterpret_cast<const decltype(v[i].v)*>(src + static_cast<int64_t>(idx) * VN);
   }
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
-    const int idx = threadIdx.x + i * 256;
+    const int idx = threadIdx.x + i * threads;
     if (idx < nvec) {
 #pragma unroll
       for (int j = 0; j < VN; ++j) dst[idx * VN + j] = v[i].get(j);

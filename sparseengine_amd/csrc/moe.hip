@@ -11,6 +11,7 @@
 
 #define ROUTER_MAX_PER_LANE 16  // experts <= 64 * 16
 
+template <int PER_LANE>  // experts <= 64 * PER_LANE
 __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t stride,
                                    const float* __restrict__ bias, int32_t* __restrict__ ids,
                                    float* __restrict__ weights, int tokens, int experts, int top_k,
@@ -20,10 +21,10 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
   if (token >= tokens) return;  // whole waves leave together; no block barrier below
   const float* row = logits + static_cast<int64_t>(token) * stride;
 
-  float score[ROUTER_MAX_PER_LANE], sel[ROUTER_MAX_PER_LANE];
+  float score[PER_LANE], sel[PER_LANE];
   float row_max = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < PER_LANE; ++i) {
     const int e = i * SE_WAVE + lane;
     score[i] = e < experts ? row[e] : -INFINITY;
     row_max = fmaxf(row_max, score[i]);
@@ -32,22 +33,22 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
     row_max = wave_max(row_max);
     float part = 0.f;
 #pragma unroll
-    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+    for (int i = 0; i < PER_LANE; ++i) {
       const int e = i * SE_WAVE + lane;
       score[i] = e < experts ? expf(score[i] - row_max) : 0.f;
       part += score[i];
     }
     const float denom = wave_sum(part);
 #pragma unroll
-    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) score[i] /= denom;
+    for (int i = 0; i < PER_LANE; ++i) score[i] /= denom;
   } else {
 #pragma unroll
-    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) score[i] = 1.f / (1.f + expf(-score[i]));
+    for (int i = 0; i < PER_LANE; ++i) score[i] = 1.f / (1.f + expf(-score[i]));
   }
   uint32_t taken = 0;     // bit i: element i of this lane is chosen
   uint32_t excluded = 0;  // bit i: element i does not exist
 #pragma unroll
-  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < PER_LANE; ++i) {
     const int e = i * SE_WAVE + lane;
     if (e < experts) {
       float s = score[i] + (bias ? bias[e] : 0.f);
@@ -63,7 +64,7 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
     float best = -INFINITY;
     int best_idx = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+    for (int i = 0; i < PER_LANE; ++i) {
       if ((taken | excluded) & (1u << i)) continue;
       const int e = i * SE_WAVE + lane;
       if (best_idx == 0x7fffffff || sel[i] > best) {
@@ -71,27 +72,18 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
         best_idx = e;
       }
     }
-#pragma unroll
-    for (int off = SE_WAVE / 2; off > 0; off >>= 1) {
-      const float other = __shfl_xor(best, off, SE_WAVE);
-      const int other_idx = __shfl_xor(best_idx, off, SE_WAVE);
-      const bool take_other =
-          other_idx != 0x7fffffff &&
-          (best_idx == 0x7fffffff || other > best || (other == best && other_idx < best_idx));
-      if (take_other) {
-        best = other;
-        best_idx = other_idx;
-      }
-    }
+    wave_reduce_pair(best, best_idx, [](float v, int i, float ov, int oi) {
+      return oi != 0x7fffffff && (i == 0x7fffffff || ov > v || (ov == v && oi < i));
+    });
     if ((best_idx & (SE_WAVE - 1)) == lane) taken |= 1u << (best_idx / SE_WAVE);
     threshold = best;
   }
   // output order: strictly greater than the threshold by index, then the chosen ties by index
   int greater_before = 0, ties_before = 0;
-  int my_slot[ROUTER_MAX_PER_LANE];
+  int my_slot[PER_LANE];
   const uint64_t lower_lanes = (lane == 0) ? 0ull : (~0ull >> (SE_WAVE - lane));
 #pragma unroll
-  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < PER_LANE; ++i) {
     const bool chosen = taken & (1u << i);
     const bool greater = chosen && sel[i] > threshold;
     const bool tie = chosen && !greater;
@@ -104,11 +96,11 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
   }
   float part = 0.f;
 #pragma unroll
-  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i)
+  for (int i = 0; i < PER_LANE; ++i)
     if (taken & (1u << i)) part += score[i];
   const float total = wave_sum(part);
 #pragma unroll
-  for (int i = 0; i < ROUTER_MAX_PER_LANE; ++i) {
+  for (int i = 0; i < PER_LANE; ++i) {
     if (!(taken & (1u << i))) continue;
     const int slot = my_slot[i] >= 0 ? my_slot[i] : greater_before + (-my_slot[i] - 1);
     ids[static_cast<int64_t>(token) * top_k + slot] = i * SE_WAVE + lane;
@@ -311,9 +303,14 @@ int se_router_topk(const float* logits, int64_t stride, const float* bias, int32
   if (experts <= 0 || experts > SE_WAVE * ROUTER_MAX_PER_LANE) return SE_ERR_SHAPE;
   if (top_k <= 0 || top_k > experts) return SE_ERR_SHAPE;
   const int waves = 4;
-  router_topk_kernel<<<(tokens + waves - 1) / waves, waves * SE_WAVE, 0, stream>>>(
-      logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize,
-      scaling);
+  const dim3 grid((tokens + waves - 1) / waves);
+  if (experts <= SE_WAVE * 4) {
+    router_topk_kernel<4><<<grid, waves * SE_WAVE, 0, stream>>>(
+        logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize, scaling);
+  } else {
+    router_topk_kernel<ROUTER_MAX_PER_LANE><<<grid, waves * SE_WAVE, 0, stream>>>(
+        logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize, scaling);
+  }
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -13,6 +13,20 @@
 // token's slot is page * page_size + offset; negative slots are skipped.
 #include "common.h"
 
+// the storage value whose widening to float is `v`, bit for bit (NaN payloads included)
+template <typename T>
+__device__ __forceinline__ T narrow_exact(float v);
+template <>
+__device__ __forceinline__ float narrow_exact<float>(float v) {
+  return v;
+}
+template <>
+__device__ __forceinline__ bf16_t narrow_exact<bf16_t>(float v) {
+  bf16_t r;
+  r.bits = static_cast<uint16_t>(__float_as_uint(v) >> 16);
+  return r;
+}
+
 template <typename T, typename W>
 __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
                                           const int32_t* __restrict__ positions,
@@ -27,6 +41,13 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
   extern __shared__ float row[];
   __shared__ float scratch[16];
   const int token = blockIdx.x;
+  // With few tokens the block is 1024 threads wide: a thread then has one vector, and every load
+  // it needs is in flight at once.
+  const int first = threadIdx.x;
+  const int stride = blockDim.x;
+  // what the later phases need from small tables is asked for before the row itself
+  const int position = positions[token];
+  const int slot = write_kv ? slots[token] : -1;
   T* src = qkv + static_cast<int64_t>(token) * row_stride;
   const int q_width = heads * head_dim;
   const int k_width = kv_heads * head_dim;
@@ -60,9 +81,8 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
   }
 
   const int half = rotary_dim / 2;
-  const float* cs = cos_sin + static_cast<int64_t>(positions[token]) * rotary_dim;
+  const float* cs = cos_sin + static_cast<int64_t>(position) * rotary_dim;
   int64_t k_dst = -1, v_dst = -1;
-  const int slot = write_kv ? slots[token] : -1;
   if (slot >= 0) {
     const int64_t page = slot / page_size;
     const int64_t off = slot % page_size;
@@ -76,7 +96,7 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
     // the rotary boundaries (head_dim, rotary_dim / 2 are multiples of the vector length)
     constexpr int WN = Vec16<W>::N;
     constexpr int WV = VN / WN;
-    for (int vi = threadIdx.x; vi < (q_width + k_width) / VN; vi += blockDim.x) {
+    for (int vi = first; vi < (q_width + k_width) / VN; vi += stride) {
       const int c0 = vi * VN;
       const bool is_q = c0 < q_width;
       const int base = is_q ? 0 : q_width;
@@ -127,7 +147,7 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
     }
   } else {
   // one thread per element of q and k: normed value, then the rotation with its partner
-  for (int c = threadIdx.x; c < q_width + k_width; c += blockDim.x) {
+  for (int c = first; c < q_width + k_width; c += stride) {
     const bool is_q = c < q_width;
     const int local = is_q ? c : c - q_width;
     const int d = local % head_dim;
@@ -156,10 +176,12 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
   }
   }
   if (v_dst >= 0) {
-    const T* v = src + q_width + k_width;      // bit-exact copy: from memory, not from the float staging
-    for (int c = threadIdx.x; c < k_width; c += blockDim.x) {
+    // the staged floats are the stored values widened; narrowing them again gives back the same bits
+    const float* v = row + q_width + k_width;
+    for (int c = first; c < k_width; c += stride) {
       const int head = c / head_dim, d = c % head_dim;
-      cache[v_dst + static_cast<int64_t>(head) * page_size * head_dim + static_cast<int64_t>(d) * page_size] = v[c];
+      cache[v_dst + static_cast<int64_t>(head) * page_size * head_dim + static_cast<int64_t>(d) * page_size] =
+          narrow_exact<T>(v[c]);
     }
   }
 }
@@ -174,7 +196,9 @@ static int launch(void* qkv, int64_t row_stride, const int32_t* positions, const
   const int vector_path = vector_ok && head_dim % VN == 0 && (rotary_dim / 2) % VN == 0 && row_stride % VN == 0 &&
                           (rotary_dim / 2) % 4 == 0 && (Vec16<W>::N <= VN);
   const size_t shmem = static_cast<size_t>(heads + 2 * kv_heads) * head_dim * sizeof(float);
-  qk_norm_rope_store_kernel<T, W><<<tokens, 256, shmem, stream>>>(
+  // few tokens: wide blocks, so that the step is not a handful of long-running narrow ones
+  const int threads = tokens < 128 ? 1024 : 256;
+  qk_norm_rope_store_kernel<T, W><<<tokens, threads, shmem, stream>>>(
       static_cast<T*>(qkv), row_stride, positions, cos_sin, static_cast<const W*>(qw),
       static_cast<const W*>(kw), eps, heads, kv_heads, head_dim, rotary_dim, static_cast<T*>(cache),
       slots, page_size, write_kv, vector_path);

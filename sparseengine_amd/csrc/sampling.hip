@@ -39,14 +39,18 @@ __device__ __forceinline__ ArgBest better(ArgBest a, ArgBest b) {
   return a;
 }
 
+// larger value, lower index among equals, over the wavefront; every lane gets the result
+__device__ __forceinline__ ArgBest wave_argbest(ArgBest v) {
+  wave_reduce_pair(v.value, v.index, [](float av, int ai, float bv, int bi) {
+    if (bi < 0) return false;
+    if (ai < 0) return true;
+    return bv > av || (bv == av && bi < ai);
+  });
+  return v;
+}
+
 __device__ ArgBest block_argbest(ArgBest v, ArgBest* scratch) {
-#pragma unroll
-  for (int off = SE_WAVE / 2; off > 0; off >>= 1) {
-    ArgBest o;
-    o.value = __shfl_xor(v.value, off, SE_WAVE);
-    o.index = __shfl_xor(v.index, off, SE_WAVE);
-    v = better(v, o);
-  }
+  v = wave_argbest(v);
   const int lane = threadIdx.x & (SE_WAVE - 1), wave = threadIdx.x / SE_WAVE;
   __syncthreads();
   if (lane == 0) scratch[wave] = v;
@@ -59,8 +63,7 @@ __device__ ArgBest block_argbest(ArgBest v, ArgBest* scratch) {
 __device__ float block_sum_f(float v, float* scratch) { return block_sum(v, scratch); }
 
 __device__ int block_sum_i(int v, int* scratch) {
-#pragma unroll
-  for (int off = SE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, SE_WAVE);
+  v = wave_sum(v);
   const int lane = threadIdx.x & (SE_WAVE - 1), wave = threadIdx.x / SE_WAVE;
   __syncthreads();
   if (lane == 0) scratch[wave] = v;
@@ -198,13 +201,7 @@ __global__ void sample_final_kernel(const float* __restrict__ part_value,
     ArgBest cand = {part_value[row * chunks + c], part_index[row * chunks + c]};
     best = better(best, cand);
   }
-#pragma unroll
-  for (int off = SE_WAVE / 2; off > 0; off >>= 1) {
-    ArgBest o;
-    o.value = __shfl_xor(best.value, off, SE_WAVE);
-    o.index = __shfl_xor(best.index, off, SE_WAVE);
-    best = better(best, o);
-  }
+  best = wave_argbest(best);
   if (threadIdx.x == 0) out[row] = best.index;
 }
 
