@@ -2,10 +2,11 @@
 //
 // Work is a list of tiles of BM = 16 * MB sorted assignments that share one expert (see
 // moe_align in moe.hip).  A workgroup of four wavefronts computes BN = 16 * NB output columns of
-// one tile; the four wavefronts split the reduction dimension K into quarters, each streaming
-// its quarter of the expert's weight rows straight from memory into MFMA operands
+// one tile; the wavefronts split the reduction dimension K into equal parts (quarters, or more
+// for the dense products of a step with few rows, which have few blocks), each streaming
+// its part of the expert's weight rows straight from memory into MFMA operands
 // (v_mfma_f32_16x16x32_bf16: weights are the A operand, the tile's activation rows the B
-// operand), and the four partial tiles are summed through LDS before the epilogue.
+// operand), and the partial tiles are summed through LDS before the epilogue.
 //
 //   MODE 0 (gate-up + SwiGLU): in row = x[a / top_k]; w = w13[e] = [gate rows; up rows], [2N, K];
 //       out[a, n] = silu(g) * u; g and u are rounded to bfloat16, silu is taken in float and
@@ -38,8 +39,8 @@ __device__ __forceinline__ bool xcd_work_item(int column_blocks, int num_tiles, 
   return true;
 }
 
-template <int MODE, int MB, int NB, int U>
-__global__ void __launch_bounds__(256)
+template <int MODE, int MB, int NB, int U, int KW = 4>   // KW wavefronts split K
+__global__ void __launch_bounds__(64 * KW)
 grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
                          bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
                          const int32_t* __restrict__ tile_expert,
@@ -54,8 +55,8 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 
   constexpr int P = NB * MB;                   // output blocks of 16 x 16 (gate/up pairs in MODE 0)
   constexpr int PARTS = MODE == 0 ? 2 : 1;
-  // block p is finished by wave p % 4; the other three waves leave their partial sums here
-  __shared__ floatx4 partial[P][3][PARTS][SE_WAVE];
+  // block p is finished by wave p % KW; the other waves leave their partial sums here
+  __shared__ floatx4 partial[P][KW - 1][PARTS][SE_WAVE];
   __shared__ int32_t rows[BM];
 
   const int lane = threadIdx.x & (SE_WAVE - 1);
@@ -94,8 +95,8 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   // A stage is U steps of 32 along K.  Two register sets take turns: while the matrix cores work
   // on one stage the loads of the next are already under way (the loop is memory-latency bound
   // otherwise: one round trip per stage and wave).
-  const int k_begin = wave * (K / 4);
-  const int k_end = k_begin + K / 4;
+  const int k_begin = wave * (K / KW);
+  const int k_end = k_begin + K / KW;
   if constexpr (U == 0) {
     // tall tiles: registers go to accumulators; one step at a time, the compiler overlaps what it can
 #pragma unroll 2
@@ -152,9 +153,9 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const int p = nb * MB + mb;
-      const int owner = p & 3;
+      const int owner = p % KW;
       if (wave != owner) {
-        const int slot = ((wave - owner + 4) & 3) - 1;
+        const int slot = ((wave - owner + KW) % KW) - 1;
 #pragma unroll
         for (int part = 0; part < PARTS; ++part) partial[p][slot][part][lane] = acc[part * NB + nb][mb];
       }
@@ -166,17 +167,17 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const int p = nb * MB + mb;
-      if ((p & 3) != wave) continue;
+      if ((p % KW) != wave) continue;
       floatx4 total[PARTS];
 #pragma unroll
       for (int part = 0; part < PARTS; ++part) {
         total[part] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {  // the quarters of K are always added in the same order
+        for (int s = 0; s < KW; ++s) {  // the parts of K are always added in the same order
           if (s == wave)
             total[part] += acc[part * NB + nb][mb];
           else
-            total[part] += partial[p][((s - wave + 4) & 3) - 1][part][lane];
+            total[part] += partial[p][((s - wave + KW) % KW) - 1][part][lane];
         }
       }
       const int a = rows[mb * 16 + col];
@@ -412,16 +413,49 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 }
 
 // Dense product of a few rows: out[rows, N] = x[rows, K] . w[N, K]^T (bfloat16, float accumulate).
+// A projection has only N / 16 blocks, far fewer than an expert layer: K is split over as many
+// wavefronts per block (up to 16) as it takes to put a few thousand of them in flight.
+template <int MB, int KW, int U>
+static void launch_dense(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
+                         hipStream_t stream) {
+  const int64_t items = static_cast<int64_t>(N / 16) * tiles;
+  const int grid = static_cast<int>((items + 7) / 8 * 8);
+  grouped_gemm_mfma_kernel<2, MB, 1, U, KW><<<grid, 64 * KW, 0, stream>>>(
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), nullptr,
+      nullptr, nullptr, nullptr, rows, 1, N, K, tiles);
+}
+
+template <int MB>
+static void dense_by_split(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
+                           hipStream_t stream) {
+  // steps of 32 per stage of the kernel's loop; with one weight block per wave even 64 rows leave
+  // registers for two stages in flight
+  constexpr int UMAX = MB == 1 ? 4 : 2;
+  constexpr int STAGE = 32 * UMAX;
+  const int64_t blocks = static_cast<int64_t>(N / 16) * tiles;
+  int kw = 4;
+  while (kw < 16 && blocks * kw < 3072 && K % (2 * kw * STAGE) == 0) kw *= 2;
+  if (K % (kw * STAGE) == 0) {
+    if (kw == 4) launch_dense<MB, 4, UMAX>(x, w, out, rows, N, K, tiles, stream);
+    else if (kw == 8) launch_dense<MB, 8, UMAX>(x, w, out, rows, N, K, tiles, stream);
+    else launch_dense<MB, 16, UMAX>(x, w, out, rows, N, K, tiles, stream);
+  } else if (UMAX >= 2 && K % (4 * 64) == 0) {
+    launch_dense<MB, 4, UMAX >= 2 ? 2 : 1>(x, w, out, rows, N, K, tiles, stream);
+  } else {   // K % 128 == 0 always holds here
+    launch_dense<MB, 4, 1>(x, w, out, rows, N, K, tiles, stream);
+  }
+}
+
 extern "C" int se_skinny_gemm_mfma(const void* x, const void* w, void* out, int rows, int N, int K,
                                    hipStream_t stream) {
   if (rows <= 0) return SE_OK;
   if (K <= 0 || K % 128 || N <= 0 || N % 16 || rows > 65535 * 16) return SE_ERR_SHAPE;
   if (rows <= 16)
-    launch<2, 1, 1>(x, w, out, nullptr, nullptr, nullptr, nullptr, rows, 1, N, K, 1, stream);
+    dense_by_split<1>(x, w, out, rows, N, K, 1, stream);
   else if (rows <= 32)
-    launch<2, 2, 1>(x, w, out, nullptr, nullptr, nullptr, nullptr, rows, 1, N, K, 1, stream);
+    dense_by_split<2>(x, w, out, rows, N, K, 1, stream);
   else
-    launch<2, 4, 1>(x, w, out, nullptr, nullptr, nullptr, nullptr, rows, 1, N, K, (rows + 63) / 64, stream);
+    dense_by_split<4>(x, w, out, rows, N, K, (rows + 63) / 64, stream);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -405,7 +405,11 @@ class HipKernels:
         _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
                                             _stream()), "moe_sum")
 
-    SKINNY_ROWS = 64        # up to this many rows a dense product streams the weight once on MFMA
+    # Up to this many rows a dense product streams the weight once on MFMA.  Measured on MI355X at
+    # 8192 x 3072 and 200064 x 3072: 8 rows 12.5 / 225 us against the library's 26 / 376; 32 rows
+    # 20 / 400 against 23 / 381; from 48 rows on the library wins (the kernel's activation loads
+    # then outweigh its weight loads).
+    SKINNY_ROWS = 32
 
     def linear(self, x, weight, out):
         """``out = x @ weight.T``.  Few bfloat16 rows take the streaming matrix-core kernel (the BLAS
