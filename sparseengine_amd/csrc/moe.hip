@@ -110,6 +110,56 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
 }
 
 // ---------------------------------------------------------------------------------------- //
+// Router logits of a step with few tokens: logits[t, e] = x[t] . w[e], float accumulate from
+// float weights; the activations are widened as they are read (no float copy of x, no library
+// call whose launch and set-up cost more than the product).  One wavefront per expert; a lane
+// takes 8 consecutive k out of every 512 and keeps the sums of up to ROUTER_TOKEN_GROUP tokens.
+// Requires K % 8 == 0 and 16-byte aligned rows.
+// ---------------------------------------------------------------------------------------- //
+#define ROUTER_TOKEN_GROUP 8
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+router_logits_kernel(const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+                     float* __restrict__ logits, int64_t out_stride, int tokens, int experts, int K) {
+  const int lane = threadIdx.x & (SE_WAVE - 1);
+  const int expert = blockIdx.x * 4 + threadIdx.x / SE_WAVE;
+  if (expert >= experts) return;   // whole waves leave together; there is no block barrier below
+  constexpr int XV = 8 / Vec16<T>::N;            // 16-byte vectors of 8 activations
+  const float* w_row = w + static_cast<int64_t>(expert) * K;
+  for (int t0 = 0; t0 < tokens; t0 += ROUTER_TOKEN_GROUP) {
+    float acc[ROUTER_TOKEN_GROUP];
+#pragma unroll
+    for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g) acc[g] = 0.f;
+#pragma unroll 2
+    for (int k = lane * 8; k < K; k += SE_WAVE * 8) {
+      const float4 w0 = *reinterpret_cast<const float4*>(w_row + k);
+      const float4 w1 = *reinterpret_cast<const float4*>(w_row + k + 4);
+      Vec16<T> xv[ROUTER_TOKEN_GROUP][XV];
+#pragma unroll
+      for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g) {
+        const int t = min(t0 + g, tokens - 1);     // rows past the end repeat the last one
+        const T* xr = x + static_cast<int64_t>(t) * x_stride + k;
+#pragma unroll
+        for (int v = 0; v < XV; ++v)
+          xv[g][v].v = *reinterpret_cast<const decltype(xv[g][v].v)*>(xr + v * Vec16<T>::N);
+      }
+      const float wk[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+      for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          acc[g] = fmaf(xv[g][j / Vec16<T>::N].get(j % Vec16<T>::N), wk[j], acc[g]);
+    }
+#pragma unroll
+    for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g) {
+      const float total = wave_sum(acc[g]);
+      if (lane == 0 && t0 + g < tokens) logits[static_cast<int64_t>(t0 + g) * out_stride + expert] = total;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------- //
 // Group the A = tokens * top_k assignments by expert.  Every expert's run is padded to a
 // multiple of `tile_rows`; padding entries hold A.  One block does the whole job.
 //   sorted[capacity]      assignment ids in expert order (capacity >= A + experts*(tile_rows-1))
@@ -311,6 +361,23 @@ int se_router_topk(const float* logits, int64_t stride, const float* bias, int32
     router_topk_kernel<ROUTER_MAX_PER_LANE><<<grid, waves * SE_WAVE, 0, stream>>>(
         logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize, scaling);
   }
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+// logits[tokens, experts] (float) = x[tokens, K] (dtype) . w[experts, K]^T (float), for few tokens
+int se_router_logits(const void* x, int64_t x_stride, const float* w, float* logits,
+                     int64_t out_stride, int tokens, int experts, int K, int dtype,
+                     hipStream_t stream) {
+  if (tokens <= 0) return SE_OK;
+  if (experts <= 0 || K <= 0 || K % 8 || x_stride % 8) return SE_ERR_SHAPE;
+  const dim3 grid((experts + 3) / 4);
+  if (dtype == SE_F32)
+    router_logits_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x), x_stride, w, logits,
+                                                          out_stride, tokens, experts, K);
+  else
+    router_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, w,
+                                                           logits, out_stride, tokens, experts, K);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -81,6 +81,8 @@ _SIGNATURES = {
     "moe": {
         "se_router_topk": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                            c_int, c_int, c_float, c_void_p],
+        "se_router_logits": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
+                             c_void_p],
         "se_moe_align": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_grouped_gemm_generic": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -310,6 +312,25 @@ class HipKernels:
             page_size, float(scale), window, _stream()), "paged_attention (mfma)")
 
     # ------------------------------------------------------------------ mixture of experts
+    ROUTER_KERNEL_TOKENS = 16   # up to this many tokens the router's product is one small kernel
+
+    def router_logits(self, x, weight, out):
+        """``out[T, experts] = x @ weight.T`` in float32 from float32 weights.  Few tokens take a
+        kernel that widens the activations as it reads them; more go to the BLAS library."""
+        tokens, k = x.shape
+        experts = weight.shape[0]
+        _require(weight.dtype == torch.float32 and weight.is_contiguous() and weight.shape[1] == k,
+                 "router weight must be float32 [experts, hidden]")
+        _require(out.dtype == torch.float32 and out.shape == (tokens, experts) and out.stride(1) == 1,
+                 "router logits must be float32 [tokens, experts]")
+        if (tokens <= self.ROUTER_KERNEL_TOKENS and k % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0
+                and x.dtype in (torch.bfloat16, torch.float32)):
+            _check(_fn.get("moe", "se_router_logits")(
+                _ptr(x), x.stride(0), _ptr(weight), _ptr(out), out.stride(0), tokens, experts, k,
+                _code(x.dtype), _stream()), "router_logits")
+            return out
+        return torch.mm(x.float(), weight.t(), out=out)
+
     def router_topk(self, logits, bias, top_k: int, ids, weights, scoring="sigmoid", normalize=True,
                     scaling: float = 1.0):
         tokens, experts = logits.shape

@@ -60,7 +60,7 @@ class RoutedExperts(Part):
 
     def _forward_chunk(self, fb, x, out):
         s, p, T = self.spec, self.params, x.shape[0]
-        logits = torch.mm(x.float(), p["router"].t(), out=fb.buffer("moe.logits", (T, s.num_experts), torch.float32))
+        logits = fb.kernels.router_logits(x, p["router"], fb.buffer("moe.logits", (T, s.num_experts), torch.float32))
         ids = fb.buffer("moe.ids", (T, s.top_k), torch.int32)
         weights = fb.buffer("moe.weights", (T, s.top_k), torch.float32)
         fb.kernels.router_topk(logits, p.get("router_bias"), s.top_k, ids, weights, scoring=s.scoring,

@@ -217,6 +217,22 @@ def test_paged_attention_finds_one_far_key(hip, dtype):
             torch.testing.assert_close(got, value, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,experts,k", [(1, 256, 3072), (8, 256, 3072), (16, 7, 200), (13, 30, 1032), (40, 16, 64)])
+def test_router_logits_are_float_products(hip, dtype, tokens, experts, k):
+    """Few tokens take the small kernel (activations widened on the fly), more the library."""
+    x = randn(tokens, k, dtype=dtype, seed=3)
+    w = randn(experts, k, dtype=torch.float32, scale=k ** -0.5, seed=4)
+    out = torch.empty(tokens, experts, dtype=torch.float32, device="cuda")
+    hip.router_logits(x, w, out)
+    ref = (x.double() @ w.double().T).float()
+    torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
+    # a view with a row stride (the engine hands over slices of larger buffers)
+    wide = randn(tokens, k + 8, dtype=dtype, seed=5)
+    hip.router_logits(wide[:, :k], w, out)
+    torch.testing.assert_close(out, (wide[:, :k].double() @ w.double().T).float(), rtol=1e-5, atol=1e-5)
+
+
 def test_router_matches_library_topk(hip, twin):
     torch.manual_seed(27)
     for tokens, experts, k in [(4096, 256, 8), (33, 8, 2), (17, 16, 4), (5, 100, 7), (3, 1, 1), (9, 1000, 16)]:

@@ -98,6 +98,9 @@ class TwinKernels:
             out[t] = o.reshape(-1).to(dt)
 
     # ------------------------------------------------------------------ mixture of experts
+    def router_logits(self, x, weight, out):
+        return torch.mm(x.float(), weight.t(), out=out)
+
     def router_topk(self, logits, bias, top_k, ids, weights, scoring="sigmoid", normalize=True, scaling=1.0):
         s = torch.sigmoid(logits) if scoring == "sigmoid" else torch.softmax(logits, -1)
         sel = s + bias if bias is not None else s.clone()
