@@ -31,7 +31,15 @@ def _ptr(t: torch.Tensor | None):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """Handle of the current device's current stream.  A decode step makes a few hundred launches;
+    the tensor library's public accessor builds a stream object for each call and costs as much
+    as a small kernel runs, its raw accessor does not."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 

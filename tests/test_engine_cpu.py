@@ -194,3 +194,26 @@ def test_attention_work_lists_cover_every_row_and_key_once():
         for item, tile, first_slot, n in work.tasks.tolist():
             slots = sorted(u[4] for u in units.tolist() if u[0] == item and u[1] == tile)
             assert slots == list(range(first_slot, first_slot + n)) and n <= 256
+
+
+def test_block_work_lists_for_many_rows_cover_every_tile_once_longest_first():
+    """Steps with enough rows to fill the chip take blocks of consecutive tiles and no splits."""
+    from sparseengine_amd.kernels.attention_work import TILES_PER_BLOCK
+    for q_len, ctx, group, kvh, window in [([2048], [2048], 6, 8, 0), ([900, 411, 1], [900, 1300, 301], 6, 8, 0),
+                                            ([1500, 600], [1500, 900], 2, 8, 70)]:
+        work = build_attention_work(q_len, ctx, group, kvh, window, head_dim=128)
+        assert work.tiles_per_block == TILES_PER_BLOCK and work.num_slots == 0 and len(work.tasks) == 0
+        reach = []
+        for item, (ql, c) in enumerate(zip(q_len, ctx)):
+            mine = work.units[work.units[:, 0] == item]
+            tiles = -(-ql * group // 16)
+            assert sorted(mine[:, 1].tolist()) == list(range(0, tiles, TILES_PER_BLOCK))
+            assert (mine[:, 2] == 0).all() and (mine[:, 3] == c).all() and (mine[:, 4] == -1).all()
+        for item, first, *_ in work.units.tolist():
+            last_row = min((first + TILES_PER_BLOCK) * 16, q_len[item] * group) - 1
+            keys = ctx[item] - q_len[item] + last_row // group + 1
+            reach.append(min(keys, window + TILES_PER_BLOCK * 16 // group + 1) if window else keys)
+        assert reach == sorted(reach, reverse=True)
+    # a head size the block kernel does not take, and a step with few rows, keep the per-wavefront list
+    assert build_attention_work([2048], [2048], 6, 8, 0, head_dim=160).tiles_per_block == 0
+    assert build_attention_work([8], [300], 6, 8, 0, head_dim=128).tiles_per_block == 0
