@@ -26,7 +26,9 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-#define UNIT_FIELDS 6  // item, row_tile, key_begin, key_end, partial_slot (-1: writes out), unused
+// A unit carries what its wavefront needs to start (one 32-byte record, no second look-up):
+#define UNIT_FIELDS 8  // item, row_tile, key_begin, key_end, partial_slot (-1: writes out), q_start, q_len, ctx_len
+#define TASK_FIELDS 6  // item, row_tile, first_slot, num_splits, q_start, q_len
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return static_cast<uint32_t>(float_to_bf16_bits(lo)) |
@@ -53,7 +55,6 @@ __global__ void __launch_bounds__(256)
 paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                             const bf16_t* __restrict__ cache,
                             const int32_t* __restrict__ block_table, int bt_stride,
-                            const int32_t* __restrict__ item_meta, int num_items,
                             const int32_t* __restrict__ units, int num_units,
                             bf16_t* __restrict__ out, int64_t out_stride,
                             float* __restrict__ part_o, float* __restrict__ part_ml, int heads,
@@ -68,11 +69,11 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   const int kvh = blockIdx.y;
   const int group = heads / kv_heads;
 
-  const int32_t* u = units + static_cast<int64_t>(unit) * UNIT_FIELDS;
-  const int item = u[0], row_tile = u[1], key_begin = u[2], slot = u[4];
-  int key_end = u[3];
-  const int q_start = item_meta[item], q_len = item_meta[num_items + item],
-            ctx_len = item_meta[2 * num_items + item];
+  const int4* u = reinterpret_cast<const int4*>(units + static_cast<int64_t>(unit) * UNIT_FIELDS);
+  const int4 u0 = u[0], u1 = u[1];
+  const int item = u0.x, row_tile = u0.y, key_begin = u0.z, slot = u1.x;
+  int key_end = u0.w;
+  const int q_start = u1.y, q_len = u1.z, ctx_len = u1.w;
   const int rows_total = q_len * group;
 
   const int rho = row_tile * 16 + n;
@@ -268,7 +269,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 // barrier is a bare s_barrier: the usual fence would wait for every load in flight.
 // The request's page ids for the block's keys are copied to shared memory first (at most
 // TILED_MAX_PAGES), so that no load in the loop depends on another.
-// A unit is {item, first_tile, key_begin, key_end, -, -}; it always writes the output itself.
+// A unit is {item, first_tile, key_begin, key_end, -, q_start, q_len, ctx_len}; it always writes the
+// output itself.
 #define TILED_MAX_PAGES 2048
 #define TILED_ROW_TILES 2   // row tiles per wavefront: 8 per block
 #define TILED_STAGES 3      // steps of keys in shared memory at a time
@@ -355,7 +357,6 @@ __global__ void __launch_bounds__(256)
 paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                              const bf16_t* __restrict__ cache,
                              const int32_t* __restrict__ block_table, int bt_stride,
-                             const int32_t* __restrict__ item_meta, int num_items,
                              const int32_t* __restrict__ units, bf16_t* __restrict__ out,
                              int64_t out_stride, int heads, int kv_heads, int page_size,
                              float scale_log2e, int window) {
@@ -376,8 +377,7 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   const int32_t* u = units + static_cast<int64_t>(blockIdx.x / kv_heads) * UNIT_FIELDS;
   const int item = u[0], first_tile = u[1], key_begin = u[2];
   int key_end = u[3];
-  const int q_start = item_meta[item], q_len = item_meta[num_items + item],
-            ctx_len = item_meta[2 * num_items + item];
+  const int q_start = u[5], q_len = u[6], ctx_len = u[7];
   const int rows_total = q_len * group;
   const int pos0 = ctx_len - q_len;
   const int last_key = ctx_len - 1;
@@ -561,63 +561,81 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   }
 }
 
-// One block per (merge task, kv head): task = {item, row_tile, first_slot, num_splits}.
-// Thread (n, j) of the 16 x 16 block first turns the splits' maxima and sums of row n into
-// weights in shared memory, then adds the weighted partial outputs for its value dims.
+// One block per (merge task, kv head): task = {item, row_tile, first_slot, num_splits, q_start, q_len}.
+// Thread (n, j) of the 16 x 16 block first turns the splits' maxima and sums of row n into weights
+// in shared memory; then every thread owns float4 pieces of the tile's 16 x head_dim output and
+// adds the weighted partial outputs, eight splits' loads in flight at a time.
 #define MERGE_MAX_SPLITS 256
 __global__ void __launch_bounds__(256)
-attention_merge_kernel(const int32_t* __restrict__ tasks, const int32_t* __restrict__ item_meta,
-                       int num_items, const float* __restrict__ part_o,
+attention_merge_kernel(const int32_t* __restrict__ tasks, const float* __restrict__ part_o,
                        const float* __restrict__ part_ml, bf16_t* __restrict__ out,
                        int64_t out_stride, int heads, int kv_heads, int head_dim) {
   __shared__ float weight[16][MERGE_MAX_SPLITS];
   __shared__ float inv_denom[16];
-  const int32_t* t = tasks + static_cast<int64_t>(blockIdx.x) * 4;
-  const int item = t[0], row_tile = t[1], first_slot = t[2], splits = t[3];
+  const int32_t* t = tasks + static_cast<int64_t>(blockIdx.x) * TASK_FIELDS;
+  const int row_tile = t[1], first_slot = t[2], splits = t[3], q_start = t[4], q_len = t[5];
   const int kvh = blockIdx.y;
   const int group = heads / kv_heads;
-  const int q_start = item_meta[item], q_len = item_meta[num_items + item];
-  const int n = threadIdx.x >> 4;        // row of the tile
-  const int j = threadIdx.x & 15;
-  const int rho = row_tile * 16 + n;
-  const bool valid = rho < q_len * group;
   const int64_t stride = static_cast<int64_t>(kv_heads) * 16;     // partial rows between two splits
-  const int64_t base0 = (static_cast<int64_t>(first_slot) * kv_heads + kvh) * 16 + n;
-  // maxima: 16 threads per row share the splits
-  float m = -INFINITY;
-  for (int s = j; s < splits; s += 16) {
-    const float ms = part_ml[(base0 + s * stride) * 2];
-    weight[n][s] = ms;
-    m = fmaxf(m, ms);
-  }
+  const int64_t tile_base = (static_cast<int64_t>(first_slot) * kv_heads + kvh) * 16;
+  {
+    const int n = threadIdx.x >> 4;        // row of the tile
+    const int j = threadIdx.x & 15;        // 16 threads per row share the splits
+    const int64_t base0 = tile_base + n;
+    float m = -INFINITY;
+    for (int s = j; s < splits; s += 16) {
+      const float ms = part_ml[(base0 + s * stride) * 2];
+      weight[n][s] = ms;
+      m = fmaxf(m, ms);
+    }
 #pragma unroll
-  for (int off = 8; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, SE_WAVE));
-  float denom = 0.f;
-  for (int s = j; s < splits; s += 16) {
-    const float w = exp2f(weight[n][s] - m);
-    weight[n][s] = w;
-    denom += part_ml[(base0 + s * stride) * 2 + 1] * w;
-  }
+    for (int off = 8; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, SE_WAVE));
+    float denom = 0.f;
+    for (int s = j; s < splits; s += 16) {
+      const float w = exp2f(weight[n][s] - m);
+      weight[n][s] = w;
+      denom += part_ml[(base0 + s * stride) * 2 + 1] * w;
+    }
 #pragma unroll
-  for (int off = 8; off > 0; off >>= 1) denom += __shfl_xor(denom, off, SE_WAVE);
-  if (j == 0) inv_denom[n] = 1.f / denom;
+    for (int off = 8; off > 0; off >>= 1) denom += __shfl_xor(denom, off, SE_WAVE);
+    if (j == 0) inv_denom[n] = 1.f / denom;
+  }
   __syncthreads();
-  if (!valid) return;
-  const int token = q_start + rho / group;
-  const int head = kvh * group + rho % group;
-  const float inv = inv_denom[n];
-  bf16_t* o_row = out + static_cast<int64_t>(token) * out_stride + static_cast<int64_t>(head) * head_dim;
-  for (int d = j; d < head_dim; d += 16) {
-    float acc = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < splits; ++s) acc += part_o[(base0 + s * stride) * head_dim + d] * weight[n][s];
-    o_row[d] = from_float<bf16_t>(acc * inv);
+  const int vecs_per_row = head_dim / 4;
+  for (int piece = threadIdx.x; piece < 16 * vecs_per_row; piece += 256) {
+    const int n = piece / vecs_per_row, d4 = (piece % vecs_per_row) * 4;
+    const int rho = row_tile * 16 + n;
+    if (rho >= q_len * group) continue;
+    const float* src = part_o + (tile_base + n) * head_dim + d4;
+    float4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+      float4 v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (s0 + i < splits) v[i] = *reinterpret_cast<const float4*>(src + (s0 + i) * stride * head_dim);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (s0 + i < splits) {   // the splits are always added in the order of their key ranges
+          const float w = weight[n][s0 + i];
+          acc.x += v[i].x * w;
+          acc.y += v[i].y * w;
+          acc.z += v[i].z * w;
+          acc.w += v[i].w * w;
+        }
+    }
+    const float inv = inv_denom[n];
+    const int token = q_start + rho / group;
+    const int head = kvh * group + rho % group;
+    uint2 packed;
+    packed.x = pack_bf16x2(acc.x * inv, acc.y * inv);
+    packed.y = pack_bf16x2(acc.z * inv, acc.w * inv);
+    *reinterpret_cast<uint2*>(out + static_cast<int64_t>(token) * out_stride +
+                              static_cast<int64_t>(head) * head_dim + d4) = packed;
   }
 }
 
 extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const void* cache,
                                        const int32_t* block_table, int bt_stride,
-                                       const int32_t* item_meta, int num_items,
                                        const int32_t* units, int num_units, const int32_t* tasks,
                                        int num_tasks, void* out, int64_t out_stride, float* part_o,
                                        float* part_ml, int heads, int kv_heads, int head_dim,
@@ -633,7 +651,7 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
   case DS:                                                                                         \
     paged_attention_mfma_kernel<DS><<<grid, 256, 0, stream>>>(                                     \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(cache), block_table,  \
-        bt_stride, item_meta, num_items, units, num_units, static_cast<bf16_t*>(out), out_stride, \
+        bt_stride, units, num_units, static_cast<bf16_t*>(out), out_stride,                       \
         part_o, part_ml, heads, kv_heads, page_size, scale_log2e, window);                        \
     break;
   switch (head_dim / 32) {
@@ -644,7 +662,7 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
   SE_CHECK_LAUNCH();
   if (num_tasks > 0) {
     attention_merge_kernel<<<dim3(num_tasks, kv_heads), 256, 0, stream>>>(
-        tasks, item_meta, num_items, part_o, part_ml, static_cast<bf16_t*>(out), out_stride, heads,
+        tasks, part_o, part_ml, static_cast<bf16_t*>(out), out_stride, heads,
         kv_heads, head_dim);
     SE_CHECK_LAUNCH();
   }
@@ -655,7 +673,6 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
 // each covering `tiles_per_block` (8) row tiles; head_dim % 32 == 0, head_dim <= 128.
 extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const void* cache,
                                         const int32_t* block_table, int bt_stride,
-                                        const int32_t* item_meta, int num_items,
                                         const int32_t* units, int num_units, void* out,
                                         int64_t out_stride, int heads, int kv_heads, int head_dim,
                                         int page_size, float scale, int window,
@@ -671,7 +688,7 @@ extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const v
   case DS:                                                                                         \
     paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES><<<grid, 256, 0, stream>>>(          \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(cache), block_table,  \
-        bt_stride, item_meta, num_items, units, static_cast<bf16_t*>(out), out_stride, heads,     \
+        bt_stride, units, static_cast<bf16_t*>(out), out_stride, heads,                           \
         kv_heads, page_size, scale_log2e, window);                                                 \
     break;
   switch (head_dim / 32) {

@@ -136,7 +136,8 @@ class BatchBuilder:
             width = max(1, -(-int(ctx_len.max()) // cache.page_size))
             tables[group.index] = np.ascontiguousarray(group.table[rows, :width])
 
-        parts = [token_ids, positions, token_item, rows, q_start, q_len, ctx_len, want]
+        item_meta_host = np.stack([q_start, q_len, ctx_len]).astype(np.int32)      # one part: [3, items]
+        parts = [token_ids, positions, token_item, rows, item_meta_host.reshape(-1), want]
         for group in cache.groups:
             parts += [allocation.slots[group.index], tables[group.index].reshape(-1)]
         works = []
@@ -148,7 +149,8 @@ class BatchBuilder:
                                                 head_dim=group.request.head_dim)
                     works.append((group.index, (ratio, window), work, len(parts)))
                     parts += [work.units.reshape(-1), work.tasks.reshape(-1)]
-        total = sum(p.size for p in parts)
+        # every part starts on a 16-byte boundary: kernels read records of four ints at once
+        total = sum(-(-p.size // 4) * 4 for p in parts)
         if self._copied is not None:
             self._copied.synchronize()  # the last step's copy has left the pinned buffer
         host, dev = self._buffers(total)
@@ -157,7 +159,7 @@ class BatchBuilder:
         for p in parts:
             host_np[cursor:cursor + p.size] = p.reshape(-1)
             offsets.append(cursor)
-            cursor += p.size
+            cursor += -(-p.size // 4) * 4
         dev[:total].copy_(host[:total], non_blocking=True)
         if self.device.type == "cuda":
             self._copied = torch.cuda.Event()
@@ -171,13 +173,12 @@ class BatchBuilder:
         fb.num_tokens, fb.num_items = T, B
         fb.token_ids, fb.positions, fb.token_item = view(0), view(1), view(2)
         fb.item_rows, fb.item_rows_host = view(3), rows
-        fb.want_index = view(7)
-        # q_start, q_len, ctx_len lie next to each other: one [3, items] device view
-        item_meta = dev[offsets[4]:offsets[4] + 3 * B].view(3, B)
+        fb.want_index = view(5)
+        item_meta = view(4, (3, B))
         for gi, group in enumerate(cache.groups):
             fb.groups[group.index] = GroupMeta(
-                block_table=view(8 + 2 * gi + 1, tables[group.index].shape),
-                token_row=fb.token_item, positions=fb.positions, slots=view(8 + 2 * gi),
+                block_table=view(6 + 2 * gi + 1, tables[group.index].shape),
+                token_row=fb.token_item, positions=fb.positions, slots=view(6 + 2 * gi),
                 page_size=cache.page_size, item_q_start=q_start, item_q_len=q_len,
                 item_ctx_len=ctx_len, item_meta=item_meta, max_ctx_len=int(ctx_len.max()),
                 max_q_len=int(q_len.max()))

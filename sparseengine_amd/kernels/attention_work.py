@@ -12,10 +12,14 @@ from dataclasses import dataclass
 
 import numpy as np
 
-UNIT_FIELDS = 6      # item, row_tile, key_begin, key_end, partial_slot (-1: none), unused
-TASK_FIELDS = 4      # item, row_tile, first_slot, num_splits
-TARGET_WAVES = 2048  # wavefronts wanted in flight (256 CUs x 4 SIMDs x 2)
-MIN_SPLIT_KEYS = 64
+UNIT_FIELDS = 8      # item, row_tile, key_begin, key_end, partial_slot (-1: none), q_start, q_len, ctx_len
+TASK_FIELDS = 6      # item, row_tile, first_slot, num_splits, q_start, q_len
+# Measured on MI355X (48:8 heads of 128, pages of 64): 8 requests x 2048 keys take 20.5 us with 16
+# ranges of 128 keys each against 23.8 us with 32 of 64; 8 x 8192 keys 48 us against 61; 4 x 131072
+# keys 361 us (5.9 TB/s) against 423; 64 requests x 2048 keys 97 us unsplit against 117 us in 4 ranges.
+TARGET_WAVES = 1024    # wavefronts wanted in flight when keys are split (256 CUs x 4 SIMDs)
+NO_SPLIT_WAVES = 512   # from this many tiles x kv heads on, every tile keeps all its keys
+MIN_SPLIT_KEYS = 128
 MAX_SPLITS = 256      # what the merge kernel's shared memory holds
 TILES_PER_BLOCK = 8   # row tiles of one block of the shared-memory kernel
 TILED_MAX_HEAD_DIM = 128
@@ -34,16 +38,21 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
     """``head_dim``: 0 keeps every step on the one-wavefront kernel (callers that do not know it)."""
     q_len = np.asarray(q_len, dtype=np.int64)
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
+    q_start = np.concatenate(([0], np.cumsum(q_len)[:-1]))      # items' tokens lie one after the other
     tiles = (q_len * group + 15) // 16
     waves = int(tiles.sum()) * kv_heads
-    want = 1 if waves >= target_waves else -(-target_waves // max(waves, 1))
-    if want == 1 and head_dim and head_dim % 32 == 0 and head_dim <= TILED_MAX_HEAD_DIM:
+    want = 1 if waves >= min(NO_SPLIT_WAVES, target_waves) else -(-target_waves // max(waves, 1))
+    # blocks of TILES_PER_BLOCK tiles pay off when items have many rows (prompt portions), not for a
+    # large batch of single tokens
+    many_rows = int(tiles.sum()) >= 4 * len(tiles) and waves >= 2 * NO_SPLIT_WAVES
+    if want == 1 and many_rows and head_dim and head_dim % 32 == 0 and head_dim <= TILED_MAX_HEAD_DIM:
         blocks = []
         pos0 = ctx_len - q_len
         for item, (n_tiles, ctx) in enumerate(zip(tiles.tolist(), ctx_len.tolist())):
             first = np.arange(0, n_tiles, TILES_PER_BLOCK, dtype=np.int32)
             block = np.zeros((first.size, UNIT_FIELDS), dtype=np.int32)
             block[:, 0], block[:, 1], block[:, 2], block[:, 3], block[:, 4] = item, first, 0, ctx, -1
+            block[:, 5], block[:, 6], block[:, 7] = q_start[item], q_len[item], ctx
             blocks.append(block)
         units = np.concatenate(blocks) if blocks else np.zeros((0, UNIT_FIELDS), np.int32)
         # longest first: a block's work grows with the position of its rows, and the blocks that are
@@ -62,6 +71,7 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
         if splits == 1:
             block = np.zeros((n_tiles, UNIT_FIELDS), dtype=np.int32)
             block[:, 0], block[:, 1], block[:, 2], block[:, 3], block[:, 4] = item, tile_ids, 0, ctx, -1
+            block[:, 5], block[:, 6], block[:, 7] = q_start[item], q_len[item], ctx
             units.append(block)
             continue
         first_key = max(0, ctx - reach) // 32 * 32
@@ -74,10 +84,12 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
         block[:, :, 2] = begins[None, :]
         block[:, :, 3] = np.minimum(begins + chunk, ctx)[None, :]
         block[:, :, 4] = slot + np.arange(n_tiles * splits, dtype=np.int32).reshape(n_tiles, splits)
+        block[:, :, 5], block[:, :, 6], block[:, :, 7] = q_start[item], q_len[item], ctx
         units.append(block.reshape(-1, UNIT_FIELDS))
         task = np.zeros((n_tiles, TASK_FIELDS), dtype=np.int32)
         task[:, 0], task[:, 1], task[:, 3] = item, tile_ids, splits
         task[:, 2] = slot + tile_ids * splits
+        task[:, 4], task[:, 5] = q_start[item], q_len[item]
         tasks.append(task)
         slot += n_tiles * splits
     return AttentionWork(np.concatenate(units) if units else np.zeros((0, UNIT_FIELDS), np.int32),

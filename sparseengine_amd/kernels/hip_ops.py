@@ -77,14 +77,15 @@ _SIGNATURES = {
                                        c_int, c_float, c_int, c_int, c_void_p],
     },
     "attention_mfma": {
-        "se_paged_attention_mfma": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int,
-                                    c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_void_p,
-                                    c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
-        # q, q_stride, cache, block_table, bt_stride, item_meta, num_items, units, num_units, out,
-        # out_stride, heads, kv_heads, head_dim, page_size, scale, window, tiles_per_block, stream
-        "se_paged_attention_tiled": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int,
-                                     c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int,
-                                     c_float, c_int, c_int, c_void_p],
+        # q, q_stride, cache, block_table, bt_stride, units, num_units, tasks, num_tasks, out, out_stride,
+        # part_o, part_ml, heads, kv_heads, head_dim, page_size, scale, window, stream
+        "se_paged_attention_mfma": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p,
+                                    c_int, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                    c_float, c_int, c_void_p],
+        # q, q_stride, cache, block_table, bt_stride, units, num_units, out, out_stride, heads, kv_heads,
+        # head_dim, page_size, scale, window, tiles_per_block, stream
+        "se_paged_attention_tiled": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p,
+                                     c_int64, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
     },
     "moe": {
         "se_router_topk": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -294,14 +295,11 @@ class HipKernels:
             if getattr(meta, "work", None) is not None:
                 meta.work[(group, window)] = work
         units, num_units, tasks, num_tasks, num_slots, tiles_per_block = work
-        num_items = meta.item_meta.shape[1]
-        _require(meta.item_meta.dtype == torch.int32 and meta.item_meta.is_contiguous(), "item_meta layout")
         if tiles_per_block:                   # prompt portions: keys and values shared by a block
             _check(_fn.get("attention_mfma", "se_paged_attention_tiled")(
                 _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
-                _ptr(meta.item_meta), num_items, _ptr(units), num_units, _ptr(out), out.stride(0), heads,
-                kv_heads, head_dim, page_size, float(scale), window, tiles_per_block, _stream()),
-                "paged_attention (tiled)")
+                _ptr(units), num_units, _ptr(out), out.stride(0), heads, kv_heads, head_dim, page_size,
+                float(scale), window, tiles_per_block, _stream()), "paged_attention (tiled)")
             return
         part_o = part_ml = None
         if num_slots:
@@ -315,9 +313,9 @@ class HipKernels:
                 self._attention_partials = (part_o, part_ml)
         _check(_fn.get("attention_mfma", "se_paged_attention_mfma")(
             _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
-            _ptr(meta.item_meta), num_items, _ptr(units), num_units, _ptr(tasks) if num_tasks else None,
-            num_tasks, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim,
-            page_size, float(scale), window, _stream()), "paged_attention (mfma)")
+            _ptr(units), num_units, _ptr(tasks) if num_tasks else None, num_tasks, _ptr(out), out.stride(0),
+            _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim, page_size, float(scale), window,
+            _stream()), "paged_attention (mfma)")
 
     # ------------------------------------------------------------------ mixture of experts
     ROUTER_KERNEL_TOKENS = 16   # up to this many tokens the router's product is one small kernel

@@ -191,9 +191,13 @@ def test_attention_work_lists_cover_every_row_and_key_once():
                 assert first == 0 or (window and first <= max(0, c - ql - window + 1))
         split = units[units[:, 4] >= 0]
         assert sorted(split[:, 4].tolist()) == list(range(work.num_slots))
-        for item, tile, first_slot, n in work.tasks.tolist():
+        starts = [sum(q_len[:i]) for i in range(len(q_len))]
+        for u in units.tolist():              # every unit carries its item's place, length and context
+            assert u[5:] == [starts[u[0]], q_len[u[0]], ctx[u[0]]]
+        for item, tile, first_slot, n, q_start, ql in work.tasks.tolist():
             slots = sorted(u[4] for u in units.tolist() if u[0] == item and u[1] == tile)
             assert slots == list(range(first_slot, first_slot + n)) and n <= 256
+            assert (q_start, ql) == (starts[item], q_len[item])
 
 
 def test_block_work_lists_for_many_rows_cover_every_tile_once_longest_first():

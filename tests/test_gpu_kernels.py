@@ -422,7 +422,7 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     q = randn(T, heads, head_dim, dtype=dtype, seed=2)
     out_h = torch.empty(T, heads * head_dim, dtype=dtype, device="cuda")
     hip.paged_attention(q, cache, meta, out_h, head_dim ** -0.5, 0)
-    assert meta.work[(heads // kv_heads, 0)][3] > 0 or batch * q_len > 100, "expected split units"
+    assert meta.work[(heads // kv_heads, 0)][3] > 0 or batch * q_len >= 64, "expected split units"
     for t in sorted({0, T // 2, T - 1}):
         row, pos = int(meta.token_row[t]), int(meta.positions[t])
         ref = dense_attention(q[t], cache, table, row, pos, head_dim ** -0.5, 0, page)
