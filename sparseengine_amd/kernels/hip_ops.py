@@ -252,7 +252,9 @@ class HipKernels:
 
         ``q``: ``[T, heads, head_dim]`` view (token stride free, heads dense); ``cache``:
         ``[pages, 2, kv_heads, page_size, head_dim]``; ``meta``: an object with ``block_table``
-        (int32 ``[rows, max_pages]``), ``token_row`` and ``positions`` (int32 ``[T]``);
+        (int32 ``[items, max_pages]``), ``token_row`` and ``positions`` (int32 ``[T]``) and, for the
+        matrix-core kernels, the items' lengths on the host (``item_q_len``, ``item_ctx_len``) and
+        optionally prepared work lists (``work``);
         ``out``: ``[T, heads * head_dim]``."""
         tokens, heads, head_dim = q.shape
         kv_heads, page_size = cache.shape[2], cache.shape[3]
@@ -269,7 +271,7 @@ class HipKernels:
             raise KernelShapeError(f"attention: {heads} heads do not divide into {kv_heads} kv heads")
         window = int(window or 0)
         if (q.dtype == torch.bfloat16 and head_dim % 32 == 0 and head_dim <= 256 and page_size % 8 == 0
-                and getattr(meta, "item_meta", None) is not None):
+                and getattr(meta, "item_q_len", None) is not None):      # the step's items are known
             return self._paged_attention_mfma(q, cache, meta, out, scale, window)
         if head_dim % 8 or head_dim > 512:
             raise KernelShapeError(f"attention: head_dim {head_dim} must be a multiple of 8, at most 512")
