@@ -273,7 +273,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 // output itself.
 #define TILED_MAX_PAGES 2048
 #define TILED_ROW_TILES 2   // row tiles per wavefront: 8 per block
-#define TILED_STAGES 3      // steps of keys in shared memory at a time
+#define TILED_STAGES 4      // steps of keys in shared memory at a time
 
 // m0 (the destination's base) is set and used inside one statement; naming it as clobbered draws a
 // warning about reserved registers that does not apply here.
@@ -287,13 +287,25 @@ __device__ __forceinline__ void load16_to_lds(const void* src, uint32_t lds_addr
 
 // Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 that share a row: two register swaps
 // between halves and between rows of 16 lanes instead of trips through the shared-memory crossbar.
+// The library's fmaxf quiets signalling NaNs first, one more instruction per operand; scores are
+// products of finite numbers or -inf, so the bare instructions do.
+__device__ __forceinline__ float max_bare(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float max3_bare(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 __device__ __forceinline__ float quad_max(float v) {
   const uint32_t u = __float_as_uint(v);
   const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  v = max_bare(__uint_as_float(a[0]), __uint_as_float(a[1]));
   const uint32_t w = __float_as_uint(v);
   const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  return max_bare(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float quad_sum(float v) {
   const uint32_t u = __float_as_uint(v);
@@ -328,8 +340,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2_rne(float lo, float hi) {   // o
         }                                                                                          \
         v[b * 4 + i] = x;                                                                          \
       }                                                                                            \
-    float m = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])),                                   \
-                    fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));                                  \
+    float m = max_bare(max3_bare(v[0], v[1], v[2]), max3_bare(max3_bare(v[3], v[4], v[5]), v[6], v[7])); \
     m = quad_max(m) * scale_log2e; /* scale > 0: the maximum commutes with it */                   \
     const bool grow = m > run_max[rt] + SOFTMAX_SLACK || (run_max[rt] == -INFINITY && m > -INFINITY); \
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(grow) != 0, 0)) {                             \
@@ -363,12 +374,15 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   constexpr int D = 32 * DSTEPS;
   constexpr int DBLOCKS = 2 * DSTEPS;
   constexpr int CHUNKS = 4 * DSTEPS;              // per step: 2 * DSTEPS of keys, then 2 * DSTEPS of values
-  __shared__ __align__(16) uint4 stage[NS][CHUNKS][64];
-  __shared__ int32_t page_ids[TILED_MAX_PAGES];
+  // dynamic: NS stages of CHUNKS x 64 vectors, then TILED_MAX_PAGES page ids (more than a block's
+  // static allowance when NS = 4 and head_dim = 128)
+  extern __shared__ __align__(16) uint4 tiled_shared[];
+  uint4(*stage)[CHUNKS][64] = reinterpret_cast<uint4(*)[CHUNKS][64]>(tiled_shared);
+  int32_t* page_ids = reinterpret_cast<int32_t*>(tiled_shared + NS * CHUNKS * 64);
 
   const int tid = threadIdx.x;
   const int lane = tid & (SE_WAVE - 1);
-  const int wave = tid / SE_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SE_WAVE);   // known to be the same in all lanes
   const int n = lane & 15;
   const int g = lane >> 4;
   const int kvh = blockIdx.x % kv_heads;   // units come longest first: all kv heads of one, then the next
@@ -401,6 +415,7 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   // The page ids of the block's keys, as many as fit; a longer range is brought in window by
   // window as the steps reach it (a very long context on small pages).
   int window_base = k_first / page_size;          // first page held in page_ids
+  int window_end = (window_base + TILED_MAX_PAGES) * page_size;   // first key whose page is not held
   const int last_page = kmax / page_size;
   if (k_first < key_end) {
     const int pages = min(last_page - window_base + 1, TILED_MAX_PAGES);
@@ -446,32 +461,37 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     for (int ds = 0; ds < DSTEPS; ++ds)
       asm volatile("" : "+v"(qf[rt][ds].x), "+v"(qf[rt][ds].y), "+v"(qf[rt][ds].z), "+v"(qf[rt][ds].w));
 
-  // Waves 0 and 1 bring the two key blocks of a step, waves 2 and 3 one half of the value dims each.
+  // Waves 0 and 1 bring the two key blocks of a step, waves 2 and 3 one half of the value dims each:
+  // wave w fills chunks w * DSTEPS ... of a stage.  Steps are issued in order, so a lane follows its
+  // key's page and place in the page by adding 32 (no division in the loop); a key past the block's
+  // last one is replaced by that one (values: by its group of eight).
   const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&stage[0][0][0]));
+  const bool loads_keys = wave < 2;
+  const int lane_key = loads_keys ? 8 * (n >> 2) + (n & 3) + 4 * wave : 8 * g;
+  const int clamp_key = loads_keys ? kmax : (kmax & ~7);
+  const int clamp_page = clamp_key / page_size, clamp_off = clamp_key % page_size;
+  int next_key = k_first + lane_key;                     // the lane's key of the next step to be issued
+  int next_page = next_key / page_size, next_off = next_key % page_size;
+  const int64_t lane_base = loads_keys ? g * 8
+                                       : plane + static_cast<int64_t>((wave - 2) * DSTEPS * 16 + n) * page_size;
+  const int off_scale = loads_keys ? D : 1;
+  const int64_t load_stride = loads_keys ? 32 : static_cast<int64_t>(16) * page_size;
   auto issue = [&](int step) {
-    const int k0 = k_first + 32 * step;
-    const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS) * 1024u;
-    if (wave < 2) {
-      int key = k0 + 8 * (n >> 2) + (n & 3) + 4 * wave;
-      if (key > kmax) key = kmax;
-      const int page = page_ids[key / page_size - window_base];
-      const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2) * plane +
-                          static_cast<int64_t>(key % page_size) * D + g * 8;
+    const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS + wave * DSTEPS) * 1024u;
+    const bool over = next_key > kmax;
+    const int page = page_ids[(over ? clamp_page : next_page) - window_base];
+    const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2) * plane + lane_base +
+                        static_cast<int64_t>(over ? clamp_off : next_off) * off_scale;
 #pragma unroll
-      for (int ds = 0; ds < DSTEPS; ++ds)
-        load16_to_lds(src + ds * 32, dst + static_cast<uint32_t>(wave * DSTEPS + ds) * 1024u);
-    } else {
-      const int half = wave - 2;
-      int vkey = k0 + 8 * g;
-      if (vkey > kmax) vkey = kmax & ~7;
-      const int page = page_ids[vkey / page_size - window_base];
-      const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2 + 1) * plane +
-                          static_cast<int64_t>(half * DSTEPS * 16 + n) * page_size + (vkey % page_size);
+    for (int j = 0; j < DSTEPS; ++j) load16_to_lds(src + j * load_stride, dst + static_cast<uint32_t>(j) * 1024u);
+    next_key += 32;
+    next_off += 32;
 #pragma unroll
-      for (int j = 0; j < DSTEPS; ++j)
-        load16_to_lds(src + static_cast<int64_t>(j) * 16 * page_size,
-                      dst + static_cast<uint32_t>(2 * DSTEPS + half * DSTEPS + j) * 1024u);
-    }
+    for (int i = 0; i < 4; ++i)          // pages hold at least 8 keys
+      if (next_off >= page_size) {
+        next_off -= page_size;
+        ++next_page;
+      }
   };
 
   const int nsteps = (key_end - k_first + 31) / 32;
@@ -491,9 +511,10 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
       asm volatile("" ::: "memory");
       if (step + NS - 1 < nsteps) {
         const int k_next = k_first + 32 * (step + NS - 1);
-        if (min(k_next + 31, kmax) / page_size >= window_base + TILED_MAX_PAGES) {
+        if (min(k_next + 31, kmax) >= window_end) {
           // nobody reads page_ids between the barrier above and its own issue below
           window_base = k_next / page_size;
+          window_end = (window_base + TILED_MAX_PAGES) * page_size;
           const int pages = min(last_page - window_base + 1, TILED_MAX_PAGES);
           for (int i = tid; i < pages; i += 256) page_ids[i] = table[window_base + i];
           __syncthreads();
@@ -526,18 +547,29 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
         }
         // the block's last step may hold slots past the request's last key: whatever an earlier owner
         // of the page left there, possibly not finite.  The loader's clamping is repeated here.
-        const bool tail = k0 + 31 > kmax;
-        int vkey = k0 + 8 * g;
-        if (vkey > kmax) vkey = kmax & ~7;
+        // Two copies of the loop: folded into one, the masking would be paid in every step.
+        if (__builtin_expect(k0 + 31 > kmax, 0)) {
+          int vkey = k0 + 8 * g;
+          if (vkey > kmax) vkey = kmax & ~7;
 #pragma unroll
-        for (int db = 0; db < DBLOCKS; ++db) {
-          uint4 vf = buf[2 * DSTEPS + db][lane];
-          if (tail) vf = zero_keys_beyond(vf, vkey, last_key);
+          for (int db = 0; db < DBLOCKS; ++db) {
+            const uint4 vf = zero_keys_beyond(buf[2 * DSTEPS + db][lane], vkey, last_key);
 #pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
-                                                               __builtin_bit_cast(bf16x8, pf[rt]),
-                                                               o[rt][db], 0, 0, 0);
+            for (int rt = 0; rt < RT; ++rt)
+              o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
+                                                                 __builtin_bit_cast(bf16x8, pf[rt]),
+                                                                 o[rt][db], 0, 0, 0);
+          }
+        } else {
+#pragma unroll
+          for (int db = 0; db < DBLOCKS; ++db) {
+            const uint4 vf = buf[2 * DSTEPS + db][lane];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
+                                                                 __builtin_bit_cast(bf16x8, pf[rt]),
+                                                                 o[rt][db], 0, 0, 0);
+          }
         }
       }
       asm volatile("" ::: "memory");
@@ -685,12 +717,23 @@ extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const v
   if (static_cast<int64_t>(num_units) * kv_heads > 0x7fffffff) return SE_ERR_SHAPE;
   dim3 grid(num_units * kv_heads);
 #define SE_ATT(DS)                                                                                 \
-  case DS:                                                                                         \
-    paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES><<<grid, 256, 0, stream>>>(          \
+  case DS: {                                                                                       \
+    constexpr size_t shared = TILED_STAGES * 4 * DS * 1024 + TILED_MAX_PAGES * sizeof(int32_t);    \
+    static bool allowed = false; /* more than 64 KB of shared memory has to be asked for, once */  \
+    if (!allowed) {                                                                                \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(                                       \
+                                  &paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES>), \
+                              hipFuncAttributeMaxDynamicSharedMemorySize,                          \
+                              static_cast<int>(shared)) != hipSuccess)                             \
+        return SE_ERR_LAUNCH;                                                                      \
+      allowed = true;                                                                              \
+    }                                                                                              \
+    paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES><<<grid, 256, shared, stream>>>( \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(cache), block_table,  \
         bt_stride, units, static_cast<bf16_t*>(out), out_stride, heads,                           \
         kv_heads, page_size, scale_log2e, window);                                                 \
-    break;
+    break;                                                                                         \
+  }
   switch (head_dim / 32) {
     SE_ATT(1) SE_ATT(2) SE_ATT(3) SE_ATT(4)
     default: return SE_ERR_SHAPE;
