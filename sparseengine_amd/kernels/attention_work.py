@@ -14,11 +14,12 @@ import numpy as np
 
 UNIT_FIELDS = 8      # item, row_tile, key_begin, key_end, partial_slot (-1: none), q_start, q_len, ctx_len
 TASK_FIELDS = 6      # item, row_tile, first_slot, num_splits, q_start, q_len
-# Measured on MI355X (48:8 heads of 128, pages of 64): 8 requests x 2048 keys take 20.5 us with 16
-# ranges of 128 keys each against 23.8 us with 32 of 64; 8 x 8192 keys 48 us against 61; 4 x 131072
-# keys 361 us (5.9 TB/s) against 423; 64 requests x 2048 keys 97 us unsplit against 117 us in 4 ranges.
-TARGET_WAVES = 1024    # wavefronts wanted in flight when keys are split (256 CUs x 4 SIMDs)
-NO_SPLIT_WAVES = 512   # from this many tiles x kv heads on, every tile keeps all its keys
+# Measured on MI355X (48:8 heads of 128, pages of 64): one wavefront per SIMD is the sweet spot.
+# 8 requests x 2048 keys take 20 us in 16 ranges of 128 keys against 24 us in 32 of 64; 64 requests
+# x 2060 keys 102 us in 2 ranges (1024 wavefronts) against 146 us unsplit and 118 us in 4 ranges;
+# 64 x 8192 keys 360 us (6.0 TB/s) against 550 us unsplit; 4 x 131072 keys 361 us (5.9 TB/s).
+TARGET_WAVES = 1024    # wavefronts wanted in flight (256 CUs x 4 SIMDs)
+TILED_MIN_WAVES = 2048 # tiles x kv heads from which prompt portions take the shared-memory kernel
 MIN_SPLIT_KEYS = 128
 MAX_SPLITS = 256      # what the merge kernel's shared memory holds
 TILES_PER_BLOCK = 8   # row tiles of one block of the shared-memory kernel
@@ -41,10 +42,10 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
     q_start = np.concatenate(([0], np.cumsum(q_len)[:-1]))      # items' tokens lie one after the other
     tiles = (q_len * group + 15) // 16
     waves = int(tiles.sum()) * kv_heads
-    want = 1 if waves >= min(NO_SPLIT_WAVES, target_waves) else -(-target_waves // max(waves, 1))
+    want = 1 if waves >= target_waves else -(-target_waves // max(waves, 1))
     # blocks of TILES_PER_BLOCK tiles pay off when items have many rows (prompt portions), not for a
     # large batch of single tokens
-    many_rows = int(tiles.sum()) >= 4 * len(tiles) and waves >= 2 * NO_SPLIT_WAVES
+    many_rows = int(tiles.sum()) >= 4 * len(tiles) and waves >= TILED_MIN_WAVES
     if want == 1 and many_rows and head_dim and head_dim % 32 == 0 and head_dim <= TILED_MAX_HEAD_DIM:
         blocks = []
         pos0 = ctx_len - q_len

@@ -436,8 +436,8 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     (8, 8, 32, 8, 0, [4200], [4200]),
     (48, 8, 128, 64, 0, [2048 + 17], [2048 + 17]),
     (12, 2, 128, 16, 300, [5000, 3000], [4100, 2001]),
-    (16, 8, 64, 24, 0, [1200, 700], [1200, 500]),                # pages that are no multiple of a step of 32 keys
-    (24, 8, 96, 40, 333, [1500, 100, 90], [1100, 100, 1]),
+    (16, 8, 64, 24, 0, [1500, 900], [1500, 700]),                # pages that are no multiple of a step of 32 keys
+    (24, 8, 96, 40, 333, [1500, 100, 90], [1400, 100, 1]),
     (8, 8, 32, 8, 0, [17000], [4100])])                          # more pages than the kernel keeps ids of at once
 def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, page, window, lens, q_lens):
     """Steps with many rows: blocks share each step's keys and values through shared memory."""
