@@ -11,14 +11,14 @@
 
 #define ROUTER_MAX_PER_LANE 16  // experts <= 64 * 16
 
+// One wavefront routes one token.
 template <int PER_LANE>  // experts <= 64 * PER_LANE
-__global__ void router_topk_kernel(const float* __restrict__ logits, int64_t stride,
-                                   const float* __restrict__ bias, int32_t* __restrict__ ids,
-                                   float* __restrict__ weights, int tokens, int experts, int top_k,
-                                   int softmax_scoring, int normalize, float scaling) {
+__device__ __forceinline__ void route_token(const float* __restrict__ logits, int64_t stride,
+                                            const float* __restrict__ bias, int32_t* __restrict__ ids,
+                                            float* __restrict__ weights, int token, int experts,
+                                            int top_k, int softmax_scoring, int normalize,
+                                            float scaling) {
   const int lane = threadIdx.x & (SE_WAVE - 1);
-  const int token = blockIdx.x * (blockDim.x / SE_WAVE) + threadIdx.x / SE_WAVE;
-  if (token >= tokens) return;  // whole waves leave together; no block barrier below
   const float* row = logits + static_cast<int64_t>(token) * stride;
 
   float score[PER_LANE], sel[PER_LANE];
@@ -109,6 +109,17 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
   }
 }
 
+template <int PER_LANE>
+__global__ void router_topk_kernel(const float* __restrict__ logits, int64_t stride,
+                                   const float* __restrict__ bias, int32_t* __restrict__ ids,
+                                   float* __restrict__ weights, int tokens, int experts, int top_k,
+                                   int softmax_scoring, int normalize, float scaling) {
+  const int token = blockIdx.x * (blockDim.x / SE_WAVE) + threadIdx.x / SE_WAVE;
+  if (token >= tokens) return;  // whole waves leave together; there is no block barrier
+  route_token<PER_LANE>(logits, stride, bias, ids, weights, token, experts, top_k, softmax_scoring,
+                        normalize, scaling);
+}
+
 // ---------------------------------------------------------------------------------------- //
 // Router logits of a step with few tokens: logits[t, e] = x[t] . w[e], float accumulate from
 // float weights; the activations are widened as they are read (no float copy of x, no library
@@ -168,10 +179,11 @@ router_logits_kernel(const T* __restrict__ x, int64_t x_stride, const float* __r
 // The order of assignments inside one expert's run is not fixed; every row of a tile is
 // computed independently of its neighbours, so results do not depend on it.
 // ---------------------------------------------------------------------------------------- //
-__global__ void moe_align_kernel(const int32_t* __restrict__ ids, int assignments, int experts,
-                                 int tile_rows, int32_t* __restrict__ sorted,
-                                 int32_t* __restrict__ tile_expert, int32_t* __restrict__ counters) {
-  extern __shared__ int32_t sh[];
+// The work of one block of 64 ... 1024 threads (a multiple of 64); sh holds 3 * experts + 1 ints.
+__device__ __forceinline__ void align_assignments(const int32_t* __restrict__ ids, int assignments,
+                                                  int experts, int tile_rows, int32_t* __restrict__ sorted,
+                                                  int32_t* __restrict__ tile_expert,
+                                                  int32_t* __restrict__ counters, int32_t* sh) {
   int32_t* counts = sh;                 // [experts]
   int32_t* offsets = sh + experts;      // [experts + 1] start of each run in `sorted`
   int32_t* cursor = offsets + experts + 1;  // [experts]
@@ -191,7 +203,7 @@ __global__ void moe_align_kernel(const int32_t* __restrict__ ids, int assignment
     stretch[threadIdx.x] = mine;
     __syncthreads();
     if (threadIdx.x < SE_WAVE) {
-      // 1024 / 64 = 16 consecutive stretch totals per lane
+      // blockDim / 64 consecutive stretch totals per lane
       const int per_lane = blockDim.x / SE_WAVE;
       int32_t lane_total = 0;
       for (int i = 0; i < per_lane; ++i) lane_total += stretch[threadIdx.x * per_lane + i];
@@ -231,6 +243,30 @@ __global__ void moe_align_kernel(const int32_t* __restrict__ ids, int assignment
     const int pos = atomicAdd(&cursor[ids[a]], 1);
     sorted[pos] = a;
   }
+}
+
+__global__ void moe_align_kernel(const int32_t* __restrict__ ids, int assignments, int experts,
+                                 int tile_rows, int32_t* __restrict__ sorted,
+                                 int32_t* __restrict__ tile_expert, int32_t* __restrict__ counters) {
+  extern __shared__ int32_t sh[];
+  align_assignments(ids, assignments, experts, tile_rows, sorted, tile_expert, counters, sh);
+}
+
+// A step with few tokens (at most 16): one block routes them, a wavefront each, and then groups
+// the assignments, which saves a launch where launches are most of the time.
+template <int PER_LANE>
+__global__ void router_topk_align_kernel(const float* __restrict__ logits, int64_t stride,
+                                         const float* __restrict__ bias, int32_t* __restrict__ ids,
+                                         float* __restrict__ weights, int tokens, int experts,
+                                         int top_k, int softmax_scoring, int normalize, float scaling,
+                                         int tile_rows, int32_t* __restrict__ sorted,
+                                         int32_t* __restrict__ tile_expert,
+                                         int32_t* __restrict__ counters) {
+  extern __shared__ int32_t sh[];
+  route_token<PER_LANE>(logits, stride, bias, ids, weights, threadIdx.x / SE_WAVE, experts, top_k,
+                        softmax_scoring, normalize, scaling);
+  __syncthreads();   // the block's own writes of ids are visible to all its threads from here on
+  align_assignments(ids, tokens * top_k, experts, tile_rows, sorted, tile_expert, counters, sh);
 }
 
 // ---------------------------------------------------------------------------------------- //
@@ -378,6 +414,28 @@ int se_router_logits(const void* x, int64_t x_stride, const float* w, float* log
   else
     router_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, w,
                                                            logits, out_stride, tokens, experts, K);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+// router_topk for at most 16 tokens followed by moe_align, in one launch
+int se_router_topk_align(const float* logits, int64_t stride, const float* bias, int32_t* ids,
+                         float* weights, int tokens, int experts, int top_k, int softmax_scoring,
+                         int normalize, float scaling, int tile_rows, int32_t* sorted,
+                         int32_t* tile_expert, int32_t* counters, hipStream_t stream) {
+  if (tokens <= 0) return SE_OK;
+  if (tokens > 16 || experts <= 0 || experts > SE_WAVE * ROUTER_MAX_PER_LANE) return SE_ERR_SHAPE;
+  if (top_k <= 0 || top_k > experts || tile_rows <= 0) return SE_ERR_SHAPE;
+  const size_t shmem = (3 * static_cast<size_t>(experts) + 1) * sizeof(int32_t);
+  if (experts <= SE_WAVE * 4) {
+    router_topk_align_kernel<4><<<1, tokens * SE_WAVE, shmem, stream>>>(
+        logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize, scaling,
+        tile_rows, sorted, tile_expert, counters);
+  } else {
+    router_topk_align_kernel<ROUTER_MAX_PER_LANE><<<1, tokens * SE_WAVE, shmem, stream>>>(
+        logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize, scaling,
+        tile_rows, sorted, tile_expert, counters);
+  }
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -92,6 +92,8 @@ _SIGNATURES = {
                            c_int, c_int, c_float, c_void_p],
         "se_router_logits": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
                              c_void_p],
+        "se_router_topk_align": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                 c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_moe_align": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_grouped_gemm_generic": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
@@ -157,6 +159,7 @@ class MoeWorkspace:
         self.sorted = torch.empty(capacity, dtype=torch.int32, device=device)
         self.tile_expert = torch.empty(max_tiles, dtype=torch.int32, device=device)
         self.counters = torch.zeros(2, dtype=torch.int32, device=device)
+        self.grouped = None      # set by router_topk when its launch has grouped the assignments already
         self.act = torch.empty(assignments, intermediate, dtype=dtype, device=device)
         self.slot_out = torch.empty(assignments, hidden, dtype=dtype, device=device)
 
@@ -339,8 +342,13 @@ class HipKernels:
             return out
         return torch.mm(x.float(), weight.t(), out=out)
 
+    FUSED_ROUTER_TOKENS = 16   # up to this many tokens one launch routes and groups the assignments
+
     def router_topk(self, logits, bias, top_k: int, ids, weights, scoring="sigmoid", normalize=True,
-                    scaling: float = 1.0):
+                    scaling: float = 1.0, workspace=None):
+        """Scores, the chosen experts and their weights.  With a ``workspace`` (the one the expert
+        products of the same step will use) and few tokens, the same launch also groups the
+        assignments by expert in tiles of 16; ``moe_experts`` then skips that step."""
         tokens, experts = logits.shape
         _require(logits.dtype == torch.float32 and logits.stride(1) == 1, "router logits must be float32")
         if bias is not None:
@@ -354,6 +362,18 @@ class HipKernels:
         if experts > 1024:
             raise KernelShapeError(f"router: {experts} experts are above the kernel's limit 1024")
         _require(1 <= top_k <= experts, "1 <= top_k <= experts")
+        if workspace is not None:
+            workspace.grouped = None
+            capacity, max_tiles = moe_tile_bounds(tokens * top_k, experts, 16)
+            if (tokens <= self.FUSED_ROUTER_TOKENS and workspace.sorted.numel() >= capacity
+                    and workspace.tile_expert.numel() >= max_tiles):
+                _check(_fn.get("moe", "se_router_topk_align")(
+                    _ptr(logits), logits.stride(0), _ptr(bias), _ptr(ids), _ptr(weights), tokens, experts,
+                    top_k, int(scoring == "softmax"), int(bool(normalize)), float(scaling), 16,
+                    _ptr(workspace.sorted), _ptr(workspace.tile_expert), _ptr(workspace.counters),
+                    _stream()), "router_topk (with grouping)")
+                workspace.grouped = (ids.data_ptr(), tokens, top_k, experts, 16, max_tiles)
+                return
         _check(_fn.get("moe", "se_router_topk")(
             _ptr(logits), logits.stride(0), _ptr(bias), _ptr(ids), _ptr(weights), tokens, experts,
             top_k, int(scoring == "softmax"), int(bool(normalize)), float(scaling), _stream()),
@@ -370,6 +390,14 @@ class HipKernels:
             _ptr(ids), assignments, experts, tile_rows, _ptr(ws.sorted), _ptr(ws.tile_expert),
             _ptr(ws.counters), _stream()), "moe_align")
         return max_tiles
+
+    def _grouped_tiles(self, ids, experts: int, ws: MoeWorkspace, tile_rows: int) -> int:
+        """Group the assignments by expert, unless the router's launch has done just that."""
+        grouped, ws.grouped = ws.grouped, None
+        tokens, top_k = ids.shape
+        if grouped is not None and grouped[:5] == (ids.data_ptr(), tokens, top_k, experts, tile_rows):
+            return grouped[5]
+        return self.moe_align(ids, experts, ws, tile_rows)
 
     def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, tile_rows=None, wide=None, tall=None):
         """``out[t] = sum_k weights[t,k] * W2_e(silu(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``;
@@ -397,7 +425,7 @@ class HipKernels:
                 tall = share > 16          # many rows per expert: the weights go through LDS and are shared
             if tall:
                 tile_rows = 64
-            max_tiles = self.moe_align(ids, experts, ws, tile_rows)
+            max_tiles = self._grouped_tiles(ids, experts, ws, tile_rows)
             if max_tiles > 65535:
                 raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
             if tall:
@@ -421,7 +449,7 @@ class HipKernels:
                       _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
                       tile_rows, wide, _stream()), "moe down (mfma)")
         else:
-            max_tiles = self.moe_align(ids, experts, ws, 16)
+            max_tiles = self._grouped_tiles(ids, experts, ws, 16)
             if max_tiles > 65535:
                 raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
             gg = _fn.get("moe", "se_grouped_gemm_generic")

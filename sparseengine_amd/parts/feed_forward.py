@@ -63,17 +63,18 @@ class RoutedExperts(Part):
         logits = fb.kernels.router_logits(x, p["router"], fb.buffer("moe.logits", (T, s.num_experts), torch.float32))
         ids = fb.buffer("moe.ids", (T, s.top_k), torch.int32)
         weights = fb.buffer("moe.weights", (T, s.top_k), torch.float32)
+        w13, w2 = p["w13"], p["w2"]
+        ws = self._workspace_for(fb, T, w13.dtype)
         fb.kernels.router_topk(logits, p.get("router_bias"), s.top_k, ids, weights, scoring=s.scoring,
-                               normalize=s.norm_topk_prob, scaling=s.routed_scaling_factor)
+                               normalize=s.norm_topk_prob, scaling=s.routed_scaling_factor, workspace=ws)
         if fb.taps is not None:
             fb.taps.setdefault("router", []).append((ids.clone(), weights.clone()))
-        w13, w2 = p["w13"], p["w2"]
         if w13.dtype == x.dtype:
-            fb.kernels.moe_experts(x, w13, w2, ids, weights, out, self._workspace_for(fb, T, x.dtype))
+            fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws)
         else:   # expert weights kept in float32 under a bfloat16 engine
             x32 = x.float()
             out32 = torch.empty_like(x32)
-            fb.kernels.moe_experts(x32, w13, w2, ids, weights, out32, self._workspace_for(fb, T, x32.dtype))
+            fb.kernels.moe_experts(x32, w13, w2, ids, weights, out32, ws)
             out.copy_(out32)
 
 

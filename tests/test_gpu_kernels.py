@@ -252,6 +252,41 @@ def test_router_matches_library_topk(hip, twin):
         assert torch.equal(ids, ids_t)
 
 
+@pytest.mark.parametrize("tokens,experts,k", [(1, 256, 8), (8, 256, 8), (16, 256, 8), (5, 7, 3), (16, 1000, 16), (3, 1, 1)])
+def test_router_with_grouping_in_one_launch(hip, tokens, experts, k):
+    """Few tokens: routing and grouping in one launch give what the two launches give."""
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    torch.manual_seed(tokens + experts)
+    logits = (torch.randn(tokens, experts) * 3).cuda()
+    bias = (torch.randn(experts) * 0.1).cuda()
+    ids_a = torch.empty(tokens, k, dtype=torch.int32, device="cuda"); w_a = torch.empty(tokens, k, device="cuda")
+    ids_b = torch.empty_like(ids_a); w_b = torch.empty_like(w_a)
+    ws_a = MoeWorkspace(tokens, k, experts, 128, 128, torch.bfloat16, "cuda")
+    ws_b = MoeWorkspace(tokens, k, experts, 128, 128, torch.bfloat16, "cuda")
+    hip.router_topk(logits, bias, k, ids_a, w_a)
+    tiles_a = hip.moe_align(ids_a, experts, ws_a, 16)
+    hip.router_topk(logits, bias, k, ids_b, w_b, workspace=ws_b)
+    assert ws_b.grouped is not None and ws_b.grouped[5] == tiles_a
+    assert torch.equal(ids_a, ids_b) and torch.equal(w_a, w_b)
+    assert torch.equal(ws_a.counters, ws_b.counters)
+    n_tiles, n_sorted = ws_a.counters.tolist()
+    assert torch.equal(ws_a.tile_expert[:n_tiles], ws_b.tile_expert[:n_tiles])
+    # the order inside an expert's run is free: compare the runs as sets
+    sa, sb = ws_a.sorted[:n_sorted].view(n_tiles, 16), ws_b.sorted[:n_sorted].view(n_tiles, 16)
+    assert torch.equal(sa.sort(-1).values, sb.sort(-1).values)
+    # and the expert products consume it: same result as with a grouping of their own
+    hidden, inter = 128, 128
+    x = randn(tokens, hidden, dtype=torch.bfloat16, seed=1)
+    w13 = randn(experts, 2 * inter, hidden, dtype=torch.bfloat16, scale=0.1, seed=2)
+    w2 = randn(experts, hidden, inter, dtype=torch.bfloat16, scale=0.1, seed=3)
+    out_a, out_b = torch.empty_like(x), torch.empty_like(x)
+    hip.moe_experts(x, w13, w2, ids_a, w_a, out_a, ws_a)
+    assert ws_b.grouped is not None
+    hip.moe_experts(x, w13, w2, ids_b, w_b, out_b, ws_b)
+    assert ws_b.grouped is None
+    assert torch.equal(out_a, out_b)
+
+
 def test_router_ties_nonfinite_and_bias(hip, twin):
     # tie order and non-finite rows as in the reference's tests/test_minimax_m2_router.py:68-122
     logits = torch.zeros(4, 256).cuda()

@@ -101,7 +101,8 @@ class TwinKernels:
     def router_logits(self, x, weight, out):
         return torch.mm(x.float(), weight.t(), out=out)
 
-    def router_topk(self, logits, bias, top_k, ids, weights, scoring="sigmoid", normalize=True, scaling=1.0):
+    def router_topk(self, logits, bias, top_k, ids, weights, scoring="sigmoid", normalize=True, scaling=1.0,
+                    workspace=None):
         s = torch.sigmoid(logits) if scoring == "sigmoid" else torch.softmax(logits, -1)
         sel = s + bias if bias is not None else s.clone()
         sel = torch.where(torch.isnan(sel), torch.full_like(sel, float("inf")), sel)
