@@ -374,6 +374,8 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   constexpr int D = 32 * DSTEPS;
   constexpr int DBLOCKS = 2 * DSTEPS;
   constexpr int CHUNKS = 4 * DSTEPS;              // per step: 2 * DSTEPS of keys, then 2 * DSTEPS of values
+  // the destination of a load into shared memory is a 16-bit offset: the stages lie in the first 64 KB
+  static_assert(NS * CHUNKS * 1024 <= 65536, "stages must lie within the first 64 KB of shared memory");
   // dynamic: NS stages of CHUNKS x 64 vectors, then TILED_MAX_PAGES page ids (more than a block's
   // static allowance when NS = 4 and head_dim = 128)
   extern __shared__ __align__(16) uint4 tiled_shared[];
