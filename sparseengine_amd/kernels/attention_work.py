@@ -20,7 +20,7 @@ TASK_FIELDS = 6      # item, row_tile, first_slot, num_splits, q_start, q_len
 # 64 x 8192 keys 360 us (6.0 TB/s) against 550 us unsplit; 4 x 131072 keys 361 us (5.9 TB/s).
 TARGET_WAVES = 1024    # wavefronts wanted in flight (256 CUs x 4 SIMDs)
 TILED_MIN_WAVES = 2048 # tiles x kv heads from which prompt portions take the shared-memory kernel
-MIN_SPLIT_KEYS = 128
+MIN_SPLIT_KEYS = 128   # keys of a range; 64 when ranges of 128 would leave most of the chip idle (one request)
 MAX_SPLITS = 256      # what the merge kernel's shared memory holds
 TILES_PER_BLOCK = 8   # row tiles of one block of the shared-memory kernel
 TILED_MAX_HEAD_DIM = 128
@@ -67,7 +67,10 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
     units, tasks, slot = [], [], 0
     for item, (n_tiles, ctx) in enumerate(zip(tiles.tolist(), ctx_len.tolist())):
         reach = min(ctx, window + int(q_len[item])) if window else ctx     # keys a tile can read
-        splits = max(1, min(want, reach // MIN_SPLIT_KEYS, MAX_SPLITS))
+        min_keys = MIN_SPLIT_KEYS
+        if waves * (reach // min_keys) < target_waves // 2:
+            min_keys //= 2
+        splits = max(1, min(want, reach // min_keys, MAX_SPLITS))
         tile_ids = np.arange(n_tiles, dtype=np.int32)
         if splits == 1:
             block = np.zeros((n_tiles, UNIT_FIELDS), dtype=np.int32)
