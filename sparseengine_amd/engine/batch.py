@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
+from ..kernels.attention_work import DeviceAttentionWork, build_attention_work
 from ..parts.base import StepScratch
 
 
@@ -142,13 +143,12 @@ class BatchBuilder:
             parts += [allocation.slots[group.index], tables[group.index].reshape(-1)]
         works = []
         if self.attention_shapes:
-            from ..kernels.attention_work import build_attention_work
             for group in cache.groups:
                 for ratio, window in sorted(self.attention_shapes.get(group.index, ())):
                     work = build_attention_work(q_len, ctx_len, ratio, group.request.kv_heads, window,
                                                 head_dim=group.request.head_dim)
                     works.append((group.index, (ratio, window), work, len(parts)))
-                    parts += [work.units.reshape(-1), work.tasks.reshape(-1)]
+                    parts += [work.units.reshape(-1), work.tasks.reshape(-1), work.block_units.reshape(-1)]
         # every part starts on a 16-byte boundary: kernels read records of four ints at once
         total = sum(-(-p.size // 4) * 4 for p in parts)
         if self._copied is not None:
@@ -183,7 +183,8 @@ class BatchBuilder:
                 item_ctx_len=ctx_len, item_meta=item_meta, max_ctx_len=int(ctx_len.max()),
                 max_q_len=int(q_len.max()))
         for group_index, key, work, at in works:
-            fb.groups[group_index].work[key] = (view(at, work.units.shape), work.units.shape[0],
-                                                view(at + 1, work.tasks.shape), work.tasks.shape[0],
-                                                work.num_slots, work.tiles_per_block)
+            fb.groups[group_index].work[key] = DeviceAttentionWork(
+                view(at, work.units.shape), work.units.shape[0], view(at + 1, work.tasks.shape),
+                work.tasks.shape[0], work.num_slots, view(at + 2, work.block_units.shape),
+                work.block_units.shape[0], work.tiles_per_block)
         return fb

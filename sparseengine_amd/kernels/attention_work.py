@@ -28,10 +28,33 @@ TILED_MAX_HEAD_DIM = 128
 
 @dataclass
 class AttentionWork:
-    units: np.ndarray        # int32 [num_units, UNIT_FIELDS]
-    tasks: np.ndarray        # int32 [num_tasks, TASK_FIELDS]
+    """Both lists may be non-empty: a step's prompt portions go to the block kernel, its single
+    tokens (whose few rows would leave a block mostly idle over a whole context) to the other."""
+    units: np.ndarray        # int32 [num_units, UNIT_FIELDS]: (tile, key range) for one wavefront each
+    tasks: np.ndarray        # int32 [num_tasks, TASK_FIELDS]: merges of split tiles
+    num_slots: int           # partial results the units write
+    block_units: np.ndarray  # int32 [num_block_units, UNIT_FIELDS]: runs of TILES_PER_BLOCK tiles for a block
+    tiles_per_block: int = TILES_PER_BLOCK
+
+
+@dataclass
+class DeviceAttentionWork:
+    """An ``AttentionWork`` whose lists lie in device memory (int32 tensors)."""
+    units: object
+    num_units: int
+    tasks: object
+    num_tasks: int
     num_slots: int
-    tiles_per_block: int = 0  # 0: units are (tile, key range) for one wavefront each; else runs of tiles for a block
+    block_units: object
+    num_block_units: int
+    tiles_per_block: int
+
+
+def _record(rows: int, item, tile, begin, end, slot, q_start, q_len, ctx) -> np.ndarray:
+    block = np.zeros((rows, UNIT_FIELDS), dtype=np.int32)
+    for column, value in enumerate((item, tile, begin, end, slot, q_start, q_len, ctx)):
+        block[:, column] = value
+    return block
 
 
 def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int = 0,
@@ -41,31 +64,37 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
     q_start = np.concatenate(([0], np.cumsum(q_len)[:-1]))      # items' tokens lie one after the other
     tiles = (q_len * group + 15) // 16
-    waves = int(tiles.sum()) * kv_heads
-    want = 1 if waves >= target_waves else -(-target_waves // max(waves, 1))
-    # blocks of TILES_PER_BLOCK tiles pay off when items have many rows (prompt portions), not for a
-    # large batch of single tokens
-    many_rows = int(tiles.sum()) >= 4 * len(tiles) and waves >= TILED_MIN_WAVES
-    if want == 1 and many_rows and head_dim and head_dim % 32 == 0 and head_dim <= TILED_MAX_HEAD_DIM:
+    empty = np.zeros((0, UNIT_FIELDS), np.int32)
+
+    # blocks of TILES_PER_BLOCK tiles pay off for items with many rows (prompt portions) in a step that
+    # fills the chip; items with few rows keep one wavefront per tile and split their keys
+    in_blocks = np.zeros(len(tiles), dtype=bool)
+    if (head_dim and head_dim % 32 == 0 and head_dim <= TILED_MAX_HEAD_DIM
+            and int(tiles.sum()) * kv_heads >= TILED_MIN_WAVES and int(tiles.sum()) >= 4 * len(tiles)):
+        in_blocks = tiles >= TILES_PER_BLOCK // 2
+    block_units = empty
+    if in_blocks.any():
         blocks = []
-        pos0 = ctx_len - q_len
-        for item, (n_tiles, ctx) in enumerate(zip(tiles.tolist(), ctx_len.tolist())):
-            first = np.arange(0, n_tiles, TILES_PER_BLOCK, dtype=np.int32)
-            block = np.zeros((first.size, UNIT_FIELDS), dtype=np.int32)
-            block[:, 0], block[:, 1], block[:, 2], block[:, 3], block[:, 4] = item, first, 0, ctx, -1
-            block[:, 5], block[:, 6], block[:, 7] = q_start[item], q_len[item], ctx
-            blocks.append(block)
-        units = np.concatenate(blocks) if blocks else np.zeros((0, UNIT_FIELDS), np.int32)
+        for item in np.nonzero(in_blocks)[0].tolist():
+            first = np.arange(0, int(tiles[item]), TILES_PER_BLOCK, dtype=np.int32)
+            blocks.append(_record(first.size, item, first, 0, ctx_len[item], -1, q_start[item], q_len[item],
+                                  ctx_len[item]))
+        block_units = np.concatenate(blocks)
         # longest first: a block's work grows with the position of its rows, and the blocks that are
         # started last decide when the kernel ends
-        reach = pos0[units[:, 0]] + ((units[:, 1].astype(np.int64) + TILES_PER_BLOCK) * 16 - 1) // group
-        keys = np.minimum(reach + 1, ctx_len[units[:, 0]])
+        pos0 = ctx_len - q_len
+        reach = pos0[block_units[:, 0]] + ((block_units[:, 1].astype(np.int64) + TILES_PER_BLOCK) * 16 - 1) // group
+        keys = np.minimum(reach + 1, ctx_len[block_units[:, 0]])
         if window:
             keys = np.minimum(keys, window + TILES_PER_BLOCK * 16 // group + 1)
-        units = units[np.argsort(-keys, kind="stable")]
-        return AttentionWork(units, np.zeros((0, TASK_FIELDS), np.int32), 0, TILES_PER_BLOCK)
+        block_units = block_units[np.argsort(-keys, kind="stable")]
+
+    rest = np.nonzero(~in_blocks)[0].tolist()
+    waves = int(tiles[~in_blocks].sum()) * kv_heads
+    want = 1 if waves >= target_waves else -(-target_waves // max(waves, 1))
     units, tasks, slot = [], [], 0
-    for item, (n_tiles, ctx) in enumerate(zip(tiles.tolist(), ctx_len.tolist())):
+    for item in rest:
+        n_tiles, ctx = int(tiles[item]), int(ctx_len[item])
         reach = min(ctx, window + int(q_len[item])) if window else ctx     # keys a tile can read
         min_keys = MIN_SPLIT_KEYS
         if waves * (reach // min_keys) < target_waves // 2:
@@ -73,10 +102,7 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
         splits = max(1, min(want, reach // min_keys, MAX_SPLITS))
         tile_ids = np.arange(n_tiles, dtype=np.int32)
         if splits == 1:
-            block = np.zeros((n_tiles, UNIT_FIELDS), dtype=np.int32)
-            block[:, 0], block[:, 1], block[:, 2], block[:, 3], block[:, 4] = item, tile_ids, 0, ctx, -1
-            block[:, 5], block[:, 6], block[:, 7] = q_start[item], q_len[item], ctx
-            units.append(block)
+            units.append(_record(n_tiles, item, tile_ids, 0, ctx, -1, q_start[item], q_len[item], ctx))
             continue
         first_key = max(0, ctx - reach) // 32 * 32
         chunk = -(-(-(-(ctx - first_key) // splits)) // 32) * 32
@@ -96,5 +122,6 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
         task[:, 4], task[:, 5] = q_start[item], q_len[item]
         tasks.append(task)
         slot += n_tiles * splits
-    return AttentionWork(np.concatenate(units) if units else np.zeros((0, UNIT_FIELDS), np.int32),
-                         np.concatenate(tasks) if tasks else np.zeros((0, TASK_FIELDS), np.int32), slot)
+    return AttentionWork(np.concatenate(units) if units else empty,
+                         np.concatenate(tasks) if tasks else np.zeros((0, TASK_FIELDS), np.int32), slot,
+                         block_units)

@@ -291,24 +291,26 @@ class HipKernels:
         group = heads // kv_heads
         work = None if getattr(meta, "work", None) is None else meta.work.get((group, window))
         if work is None:                      # not prepared by the batch builder: build it here
-            from .attention_work import build_attention_work
+            from .attention_work import DeviceAttentionWork, build_attention_work
             host = build_attention_work(meta.item_q_len, meta.item_ctx_len, group, kv_heads, window,
                                         head_dim=head_dim)
-            work = (torch.from_numpy(host.units).to(q.device), host.units.shape[0],
-                    torch.from_numpy(host.tasks).to(q.device), host.tasks.shape[0], host.num_slots,
-                    host.tiles_per_block)
+            work = DeviceAttentionWork(
+                torch.from_numpy(host.units).to(q.device), host.units.shape[0],
+                torch.from_numpy(host.tasks).to(q.device), host.tasks.shape[0], host.num_slots,
+                torch.from_numpy(host.block_units).to(q.device), host.block_units.shape[0], host.tiles_per_block)
             if getattr(meta, "work", None) is not None:
                 meta.work[(group, window)] = work
-        units, num_units, tasks, num_tasks, num_slots, tiles_per_block = work
-        if tiles_per_block:                   # prompt portions: keys and values shared by a block
+        if work.num_block_units:              # prompt portions: keys and values shared by a block
             _check(_fn.get("attention_mfma", "se_paged_attention_tiled")(
                 _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
-                _ptr(units), num_units, _ptr(out), out.stride(0), heads, kv_heads, head_dim, page_size,
-                float(scale), window, tiles_per_block, _stream()), "paged_attention (tiled)")
+                _ptr(work.block_units), work.num_block_units, _ptr(out), out.stride(0), heads, kv_heads,
+                head_dim, page_size, float(scale), window, work.tiles_per_block, _stream()),
+                "paged_attention (blocks)")
+        if not work.num_units:
             return
         part_o = part_ml = None
-        if num_slots:
-            need = num_slots * kv_heads * 16
+        if work.num_slots:
+            need = work.num_slots * kv_heads * 16
             if self._attention_partials is None or self._attention_partials[0].numel() < need * head_dim:
                 self._attention_partials = (torch.empty(need * head_dim, dtype=torch.float32, device=q.device),
                                             torch.empty(need * 2, dtype=torch.float32, device=q.device))
@@ -318,9 +320,9 @@ class HipKernels:
                 self._attention_partials = (part_o, part_ml)
         _check(_fn.get("attention_mfma", "se_paged_attention_mfma")(
             _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
-            _ptr(units), num_units, _ptr(tasks) if num_tasks else None, num_tasks, _ptr(out), out.stride(0),
-            _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim, page_size, float(scale), window,
-            _stream()), "paged_attention (mfma)")
+            _ptr(work.units), work.num_units, _ptr(work.tasks) if work.num_tasks else None, work.num_tasks,
+            _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim, page_size,
+            float(scale), window, _stream()), "paged_attention (wavefronts)")
 
     # ------------------------------------------------------------------ mixture of experts
     ROUTER_KERNEL_TOKENS = 16   # up to this many tokens the router's product is one small kernel

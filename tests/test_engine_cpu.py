@@ -201,23 +201,39 @@ def test_attention_work_lists_cover_every_row_and_key_once():
 
 
 def test_block_work_lists_for_many_rows_cover_every_tile_once_longest_first():
-    """Steps with enough rows to fill the chip take blocks of consecutive tiles and no splits."""
+    """Steps with enough rows to fill the chip: items with many rows take blocks of consecutive tiles
+    and no splits, items with few rows (a decoded token beside a prompt portion) keep one wavefront
+    per tile with their keys split."""
     from sparseengine_amd.kernels.attention_work import TILES_PER_BLOCK
     for q_len, ctx, group, kvh, window in [([2048], [2048], 6, 8, 0), ([900, 411, 1], [900, 1300, 301], 6, 8, 0),
-                                            ([1500, 600], [1500, 900], 2, 8, 70)]:
+                                            ([1500, 600], [1500, 900], 2, 8, 70),
+                                            ([1, 2048, 1, 3], [70000, 2048, 9, 500], 6, 8, 0)]:
         work = build_attention_work(q_len, ctx, group, kvh, window, head_dim=128)
-        assert work.tiles_per_block == TILES_PER_BLOCK and work.num_slots == 0 and len(work.tasks) == 0
         reach = []
         for item, (ql, c) in enumerate(zip(q_len, ctx)):
-            mine = work.units[work.units[:, 0] == item]
             tiles = -(-ql * group // 16)
-            assert sorted(mine[:, 1].tolist()) == list(range(0, tiles, TILES_PER_BLOCK))
-            assert (mine[:, 2] == 0).all() and (mine[:, 3] == c).all() and (mine[:, 4] == -1).all()
-        for item, first, *_ in work.units.tolist():
+            mine = work.block_units[work.block_units[:, 0] == item]
+            alone = work.units[work.units[:, 0] == item]
+            if tiles >= TILES_PER_BLOCK // 2:
+                assert len(alone) == 0
+                assert sorted(mine[:, 1].tolist()) == list(range(0, tiles, TILES_PER_BLOCK))
+                assert (mine[:, 2] == 0).all() and (mine[:, 3] == c).all() and (mine[:, 4] == -1).all()
+                assert (mine[:, 5:] == [sum(q_len[:item]), ql, c]).all()
+            else:
+                assert len(mine) == 0 and sorted(set(alone[:, 1].tolist())) == list(range(tiles))
+                for tile in range(tiles):      # the tile's key ranges join up and cover its keys
+                    ranges = sorted((b, e) for _, t, b, e, *_ in alone.tolist() if t == tile)
+                    assert ranges[0][0] == 0 and ranges[-1][1] == c
+                    assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:]))
+        assert len(work.block_units) > 0
+        for item, first, *_ in work.block_units.tolist():
             last_row = min((first + TILES_PER_BLOCK) * 16, q_len[item] * group) - 1
             keys = ctx[item] - q_len[item] + last_row // group + 1
             reach.append(min(keys, window + TILES_PER_BLOCK * 16 // group + 1) if window else keys)
         assert reach == sorted(reach, reverse=True)
+    # the long single token beside the prompt is split over many wavefronts
+    work = build_attention_work([1, 2048], [70000, 2048], 6, 8, 0, head_dim=128)
+    assert (work.units[:, 0] == 0).all() and len(work.units) >= 64 and work.num_slots == len(work.units)
     # a head size the block kernel does not take, and a step with few rows, keep the per-wavefront list
-    assert build_attention_work([2048], [2048], 6, 8, 0, head_dim=160).tiles_per_block == 0
-    assert build_attention_work([8], [300], 6, 8, 0, head_dim=128).tiles_per_block == 0
+    assert len(build_attention_work([2048], [2048], 6, 8, 0, head_dim=160).block_units) == 0
+    assert len(build_attention_work([8], [300], 6, 8, 0, head_dim=128).block_units) == 0
