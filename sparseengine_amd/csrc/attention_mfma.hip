@@ -29,6 +29,9 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // A unit carries what its wavefront needs to start (one 32-byte record, no second look-up):
 #define UNIT_FIELDS 8  // item, row_tile, key_begin, key_end, partial_slot (-1: writes out), q_start, q_len, ctx_len
 #define TASK_FIELDS 6  // item, row_tile, first_slot, num_splits, q_start, q_len
+// a block's record: item, first_tile, key_begin, key_end, partial_slot of its first tile (-1: writes
+// out), q_start, q_len, ctx_len, slots between two of its tiles (= key ranges per tile), 3 unused
+#define BLOCK_UNIT_FIELDS 12
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return static_cast<uint32_t>(float_to_bf16_bits(lo)) |
@@ -269,8 +272,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 // barrier is a bare s_barrier: the usual fence would wait for every load in flight.
 // The request's page ids for the block's keys are copied to shared memory first (at most
 // TILED_MAX_PAGES), so that no load in the loop depends on another.
-// A unit is {item, first_tile, key_begin, key_end, -, q_start, q_len, ctx_len}; it always writes the
-// output itself.
+// A unit covers a run of tiles and a range of keys; with the whole range of its rows it writes the
+// output itself, else partial results for the merge kernel, like the units of the kernel above.
 #define TILED_MAX_PAGES 2048
 #define TILED_ROW_TILES 2   // row tiles per wavefront: 8 per block
 #define TILED_STAGES 4      // steps of keys in shared memory at a time
@@ -369,7 +372,8 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                              const bf16_t* __restrict__ cache,
                              const int32_t* __restrict__ block_table, int bt_stride,
                              const int32_t* __restrict__ units, bf16_t* __restrict__ out,
-                             int64_t out_stride, int heads, int kv_heads, int page_size,
+                             int64_t out_stride, float* __restrict__ part_o,
+                             float* __restrict__ part_ml, int heads, int kv_heads, int page_size,
                              float scale_log2e, int window) {
   constexpr int D = 32 * DSTEPS;
   constexpr int DBLOCKS = 2 * DSTEPS;
@@ -390,8 +394,8 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   const int kvh = blockIdx.x % kv_heads;   // units come longest first: all kv heads of one, then the next
   const int group = heads / kv_heads;
 
-  const int32_t* u = units + static_cast<int64_t>(blockIdx.x / kv_heads) * UNIT_FIELDS;
-  const int item = u[0], first_tile = u[1], key_begin = u[2];
+  const int32_t* u = units + static_cast<int64_t>(blockIdx.x / kv_heads) * BLOCK_UNIT_FIELDS;
+  const int item = u[0], first_tile = u[1], key_begin = u[2], slot = u[4], slot_stride = u[8];
   int key_end = u[3];
   const int q_start = u[5], q_len = u[6], ctx_len = u[7];
   const int rows_total = q_len * group;
@@ -581,6 +585,21 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const float total = quad_sum(run_sum[rt]);   // every lane takes part
+    if (slot >= 0) {
+      // one key range of several: the unnormalised sums, their reference and the sum of weights, for
+      // the merge kernel (padding rows included, tiles past the item's rows not: they have no slot)
+      if ((tile0 + rt) * 16 >= rows_total) continue;
+      const int64_t base =
+          (static_cast<int64_t>(slot + (tile0 + rt - first_tile) * slot_stride) * kv_heads + kvh) * 16 + n;
+      float* po = part_o + base * D + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) *reinterpret_cast<floatx4*>(po + db * 16) = o[rt][db];
+      if (g == 0) {
+        part_ml[base * 2] = run_max[rt];
+        part_ml[base * 2 + 1] = total;
+      }
+      continue;
+    }
     if (!row_valid[rt] || !wave_active) continue;
     const float inv = 1.f / total;
     bf16_t* o_row = out + static_cast<int64_t>(token[rt]) * out_stride +
@@ -674,13 +693,14 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
                                        int num_tasks, void* out, int64_t out_stride, float* part_o,
                                        float* part_ml, int heads, int kv_heads, int head_dim,
                                        int page_size, float scale, int window, hipStream_t stream) {
-  if (num_units <= 0) return SE_OK;
+  if (num_units <= 0 && num_tasks <= 0) return SE_OK;
   if (head_dim % 32 || head_dim <= 0 || head_dim > 256) return SE_ERR_SHAPE;
   if (kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 8) return SE_ERR_SHAPE;
   if (q_stride % 8 || out_stride % 4) return SE_ERR_SHAPE;
   if (num_tasks > 0 && (!part_o || !part_ml || !tasks)) return SE_ERR_SHAPE;  // splits per task <= 256 (host)
   const float scale_log2e = scale * 1.4426950408889634f;
   dim3 grid((num_units + 3) / 4, kv_heads);
+  if (num_units > 0) {
 #define SE_ATT(DS)                                                                                 \
   case DS:                                                                                         \
     paged_attention_mfma_kernel<DS><<<grid, 256, 0, stream>>>(                                     \
@@ -694,7 +714,8 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
   }
 #undef SE_ATT
   SE_CHECK_LAUNCH();
-  if (num_tasks > 0) {
+  }
+  if (num_tasks > 0) {   // also merges what the block kernel has left in the same buffers
     attention_merge_kernel<<<dim3(num_tasks, kv_heads), 256, 0, stream>>>(
         tasks, part_o, part_ml, static_cast<bf16_t*>(out), out_stride, heads,
         kv_heads, head_dim);
@@ -703,14 +724,15 @@ extern "C" int se_paged_attention_mfma(const void* q, int64_t q_stride, const vo
   return SE_OK;
 }
 
-// Prompt portions through shared memory: units are {item, first_tile, key_begin, key_end, -, -},
-// each covering `tiles_per_block` (8) row tiles; head_dim % 32 == 0, head_dim <= 128.
+// Prompt portions through shared memory: units of BLOCK_UNIT_FIELDS ints, each covering
+// `tiles_per_block` (8) row tiles; head_dim % 32 == 0, head_dim <= 128.  Units with a partial slot
+// need part_o / part_ml and a merge afterwards (se_paged_attention_mfma with the tiles' tasks).
 extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const void* cache,
                                         const int32_t* block_table, int bt_stride,
                                         const int32_t* units, int num_units, void* out,
-                                        int64_t out_stride, int heads, int kv_heads, int head_dim,
-                                        int page_size, float scale, int window,
-                                        int tiles_per_block, hipStream_t stream) {
+                                        int64_t out_stride, float* part_o, float* part_ml, int heads,
+                                        int kv_heads, int head_dim, int page_size, float scale,
+                                        int window, int tiles_per_block, hipStream_t stream) {
   if (num_units <= 0) return SE_OK;
   if (head_dim % 32 || head_dim <= 0 || head_dim > 128) return SE_ERR_SHAPE;
   if (kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 8) return SE_ERR_SHAPE;
@@ -732,7 +754,7 @@ extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const v
     }                                                                                              \
     paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES><<<grid, 256, shared, stream>>>( \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(cache), block_table,  \
-        bt_stride, units, static_cast<bf16_t*>(out), out_stride, heads,                           \
+        bt_stride, units, static_cast<bf16_t*>(out), out_stride, part_o, part_ml, heads,          \
         kv_heads, page_size, scale_log2e, window);                                                 \
     break;                                                                                         \
   }

@@ -82,10 +82,11 @@ _SIGNATURES = {
         "se_paged_attention_mfma": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p,
                                     c_int, c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                     c_float, c_int, c_void_p],
-        # q, q_stride, cache, block_table, bt_stride, units, num_units, out, out_stride, heads, kv_heads,
-        # head_dim, page_size, scale, window, tiles_per_block, stream
+        # q, q_stride, cache, block_table, bt_stride, units, num_units, out, out_stride, part_o, part_ml,
+        # heads, kv_heads, head_dim, page_size, scale, window, tiles_per_block, stream
         "se_paged_attention_tiled": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p,
-                                     c_int64, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+                                     c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
+                                     c_int, c_void_p],
     },
     "moe": {
         "se_router_topk": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -300,16 +301,8 @@ class HipKernels:
                 torch.from_numpy(host.block_units).to(q.device), host.block_units.shape[0], host.tiles_per_block)
             if getattr(meta, "work", None) is not None:
                 meta.work[(group, window)] = work
-        if work.num_block_units:              # prompt portions: keys and values shared by a block
-            _check(_fn.get("attention_mfma", "se_paged_attention_tiled")(
-                _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
-                _ptr(work.block_units), work.num_block_units, _ptr(out), out.stride(0), heads, kv_heads,
-                head_dim, page_size, float(scale), window, work.tiles_per_block, _stream()),
-                "paged_attention (blocks)")
-        if not work.num_units:
-            return
         part_o = part_ml = None
-        if work.num_slots:
+        if work.num_slots:                    # key ranges leave partial results for the merge
             need = work.num_slots * kv_heads * 16
             if self._attention_partials is None or self._attention_partials[0].numel() < need * head_dim:
                 self._attention_partials = (torch.empty(need * head_dim, dtype=torch.float32, device=q.device),
@@ -318,11 +311,19 @@ class HipKernels:
             if part_ml.numel() < need * 2:
                 part_ml = torch.empty(need * 2, dtype=torch.float32, device=q.device)
                 self._attention_partials = (part_o, part_ml)
-        _check(_fn.get("attention_mfma", "se_paged_attention_mfma")(
-            _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
-            _ptr(work.units), work.num_units, _ptr(work.tasks) if work.num_tasks else None, work.num_tasks,
-            _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim, page_size,
-            float(scale), window, _stream()), "paged_attention (wavefronts)")
+        if work.num_block_units:              # prompt portions: keys and values shared by a block
+            _check(_fn.get("attention_mfma", "se_paged_attention_tiled")(
+                _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
+                _ptr(work.block_units), work.num_block_units, _ptr(out), out.stride(0), _ptr(part_o),
+                _ptr(part_ml), heads, kv_heads, head_dim, page_size, float(scale), window,
+                work.tiles_per_block, _stream()), "paged_attention (blocks)")
+        if work.num_units or work.num_tasks:  # one wavefront per tile and key range; then all merges
+            _check(_fn.get("attention_mfma", "se_paged_attention_mfma")(
+                _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
+                _ptr(work.units) if work.num_units else None, work.num_units,
+                _ptr(work.tasks) if work.num_tasks else None, work.num_tasks, _ptr(out), out.stride(0),
+                _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim, page_size, float(scale), window,
+                _stream()), "paged_attention (wavefronts)")
 
     # ------------------------------------------------------------------ mixture of experts
     ROUTER_KERNEL_TOKENS = 16   # up to this many tokens the router's product is one small kernel

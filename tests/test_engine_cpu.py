@@ -200,40 +200,71 @@ def test_attention_work_lists_cover_every_row_and_key_once():
             assert (q_start, ql) == (starts[item], q_len[item])
 
 
+def _check_ranges(ranges, ctx, first_allowed=0):
+    """Key ranges of one tile (or run of tiles): joined up, multiples of 32 at the seams, ending at ctx."""
+    ranges = sorted(ranges)
+    assert ranges[0][0] <= first_allowed and ranges[-1][1] == ctx
+    assert all(a[1] == b[0] and a[1] % 32 == 0 for a, b in zip(ranges, ranges[1:]))
+
+
 def test_block_work_lists_for_many_rows_cover_every_tile_once_longest_first():
-    """Steps with enough rows to fill the chip: items with many rows take blocks of consecutive tiles
-    and no splits, items with few rows (a decoded token beside a prompt portion) keep one wavefront
-    per tile with their keys split."""
+    """Items with many rows take blocks of consecutive tiles, items with few rows (a decoded token
+    beside a prompt portion) keep one wavefront per tile; both split their keys when their class
+    alone would not fill the chip, and every tile with split keys has one merge task."""
     from sparseengine_amd.kernels.attention_work import TILES_PER_BLOCK
     for q_len, ctx, group, kvh, window in [([2048], [2048], 6, 8, 0), ([900, 411, 1], [900, 1300, 301], 6, 8, 0),
                                             ([1500, 600], [1500, 900], 2, 8, 70),
-                                            ([1, 2048, 1, 3], [70000, 2048, 9, 500], 6, 8, 0)]:
+                                            ([1, 2048, 1, 3], [70000, 2048, 9, 500], 6, 8, 0),
+                                            ([100], [100000], 6, 8, 0), ([512] + [1] * 32, [8192] + [4096] * 32, 6, 8, 0),
+                                            ([40, 1], [5000, 5000], 6, 1, 256)]:
         work = build_attention_work(q_len, ctx, group, kvh, window, head_dim=128)
-        reach = []
+        slots_seen = []
         for item, (ql, c) in enumerate(zip(q_len, ctx)):
             tiles = -(-ql * group // 16)
+            lowest = max(0, c - ql - window + 1) if window else 0
             mine = work.block_units[work.block_units[:, 0] == item]
             alone = work.units[work.units[:, 0] == item]
+            tasks = [t for t in work.tasks.tolist() if t[0] == item]
             if tiles >= TILES_PER_BLOCK // 2:
                 assert len(alone) == 0
-                assert sorted(mine[:, 1].tolist()) == list(range(0, tiles, TILES_PER_BLOCK))
-                assert (mine[:, 2] == 0).all() and (mine[:, 3] == c).all() and (mine[:, 4] == -1).all()
-                assert (mine[:, 5:] == [sum(q_len[:item]), ql, c]).all()
+                assert sorted(set(mine[:, 1].tolist())) == list(range(0, tiles, TILES_PER_BLOCK))
+                assert (mine[:, 5:9] == [sum(q_len[:item]), ql, c, mine[0, 8]]).all()
+                splits = int(mine[0, 8])
+                for first in range(0, tiles, TILES_PER_BLOCK):
+                    runs = mine[mine[:, 1] == first]
+                    assert len(runs) == splits
+                    _check_ranges([(b, e) for b, e in runs[:, 2:4].tolist()], c, lowest)
+                    if splits == 1:
+                        assert runs[0, 4] == -1
+                    else:       # slot of the run's first tile; the other tiles follow at a stride of `splits`
+                        for t in range(first, min(first + TILES_PER_BLOCK, tiles)):
+                            slots_seen += [int(sl) + (t - first) * splits for sl in runs[:, 4]]
             else:
                 assert len(mine) == 0 and sorted(set(alone[:, 1].tolist())) == list(range(tiles))
-                for tile in range(tiles):      # the tile's key ranges join up and cover its keys
-                    ranges = sorted((b, e) for _, t, b, e, *_ in alone.tolist() if t == tile)
-                    assert ranges[0][0] == 0 and ranges[-1][1] == c
-                    assert all(a[1] == b[0] for a, b in zip(ranges, ranges[1:]))
-        assert len(work.block_units) > 0
-        for item, first, *_ in work.block_units.tolist():
+                assert (alone[:, 5:] == [sum(q_len[:item]), ql, c]).all()
+                splits = len(alone) // tiles
+                for tile in range(tiles):
+                    _check_ranges([(b, e) for _, t, b, e, *_ in alone.tolist() if t == tile], c, lowest)
+                slots_seen += [int(sl) for sl in alone[:, 4] if sl >= 0]
+            if splits > 1:
+                assert sorted(t[1] for t in tasks) == list(range(tiles)) and all(t[3] == splits for t in tasks)
+                assert all(t[2] == tasks[0][2] + (t[1] - tasks[0][1]) * splits for t in tasks)
+                assert all(t[4:] == [sum(q_len[:item]), ql] for t in tasks)
+            else:
+                assert not tasks
+        assert sorted(slots_seen) == list(range(work.num_slots))        # every partial slot written exactly once
+        lengths = []
+        for item, first, begin, end, *_ in work.block_units.tolist():
             last_row = min((first + TILES_PER_BLOCK) * 16, q_len[item] * group) - 1
-            keys = ctx[item] - q_len[item] + last_row // group + 1
-            reach.append(min(keys, window + TILES_PER_BLOCK * 16 // group + 1) if window else keys)
-        assert reach == sorted(reach, reverse=True)
-    # the long single token beside the prompt is split over many wavefronts
-    work = build_attention_work([1, 2048], [70000, 2048], 6, 8, 0, head_dim=128)
-    assert (work.units[:, 0] == 0).all() and len(work.units) >= 64 and work.num_slots == len(work.units)
-    # a head size the block kernel does not take, and a step with few rows, keep the per-wavefront list
+            stop = min(ctx[item] - q_len[item] + last_row // group + 1, end)
+            start = begin
+            if window:
+                start = max(begin, ctx[item] - q_len[item] + first * 16 // group - window + 1)
+            lengths.append(max(stop - start, 0))
+        assert lengths == sorted(lengths, reverse=True)
+    # a long single token beside a prompt gets many more ranges than its short neighbours
+    work = build_attention_work([1, 2048, 1], [70000, 2048, 2048], 6, 8, 0, head_dim=128)
+    assert (work.units[:, 0] == 0).sum() >= 20 * (work.units[:, 0] == 2).sum()
+    # a head size the block kernel does not take, and a step of single tokens, keep the per-wavefront list
     assert len(build_attention_work([2048], [2048], 6, 8, 0, head_dim=160).block_units) == 0
-    assert len(build_attention_work([8], [300], 6, 8, 0, head_dim=128).block_units) == 0
+    assert len(build_attention_work([1] * 8, [300] * 8, 6, 8, 0, head_dim=128).block_units) == 0

@@ -474,6 +474,8 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     (16, 8, 64, 24, 0, [1500, 900], [1500, 700]),                # pages that are no multiple of a step of 32 keys
     (24, 8, 96, 40, 333, [1500, 100, 90], [1400, 100, 1]),
     (48, 8, 128, 64, 0, [9000, 2100, 77], [1, 2100, 5]),          # a decoded token with a long context beside a prompt
+    (48, 8, 128, 64, 0, [20000], [100]),                          # few blocks, long context: their keys are split
+    (12, 2, 64, 16, 900, [6000, 5000], [300, 77]),                # the same with a window
     (8, 8, 32, 8, 0, [17000], [4100])])                          # more pages than the kernel keeps ids of at once
 def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, page, window, lens, q_lens):
     """Steps with many rows: blocks share each step's keys and values through shared memory."""
@@ -493,7 +495,8 @@ def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, p
     hip.paged_attention(q, cache, meta, out_h, scale, window)
     work = meta.work[(heads // kv_heads, window)]
     assert work.num_block_units > 0, "expected the shared-memory kernel"
-    assert (work.num_units > 0) == any(n * (heads // kv_heads) < 64 for n in q_lens), "few rows: one wavefront per tile"
+    few_rows = [-(-n * (heads // kv_heads) // 16) < 4 for n in q_lens]
+    assert (work.num_units > 0) == any(few_rows), "few rows: one wavefront per tile"
     twin.paged_attention(q, cache, meta, out_t, scale, window)
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
     for t in sorted({0, 1, 15, 16, q_lens[0] - 1, min(q_lens[0], T - 1), T // 2, T - 1}):
