@@ -54,21 +54,6 @@ class DeviceAttentionWork:
     tiles_per_block: int
 
 
-def _record(rows: int, fields: int, item, tile, begin, end, slot, q_start, q_len, ctx) -> np.ndarray:
-    block = np.zeros((rows, fields), dtype=np.int32)
-    for column, value in enumerate((item, tile, begin, end, slot, q_start, q_len, ctx)):
-        block[:, column] = value
-    return block
-
-
-def _ranges(first_key: int, ctx: int, splits: int):
-    """``splits`` equal key ranges (multiples of 32 keys) over [first_key, ctx): begins, ends."""
-    chunk = -(-(-(-(ctx - first_key) // splits)) // 32) * 32
-    splits = -(-(ctx - first_key) // chunk)
-    begins = first_key + np.arange(splits, dtype=np.int32) * chunk
-    return begins, np.minimum(begins + chunk, ctx)
-
-
 def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int = 0,
                          target_waves: int = TARGET_WAVES, head_dim: int = 0) -> AttentionWork:
     """``head_dim``: 0 keeps every item on the one-wavefront kernel (callers that do not know it).
@@ -96,45 +81,52 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
         share = -(-int((units_per_item * reach).sum()) * kv_heads // wanted)
         return max(least, -(-share // 32) * 32)
 
-    units, tasks, block_units, slot = [], [], [], 0
     nblocks = np.where(in_blocks, -(-tiles // TILES_PER_BLOCK), 0)
     alone = np.where(in_blocks, 0, tiles)
-    block_keys = keys_per_unit(nblocks, TARGET_BLOCKS, MIN_BLOCK_KEYS)
-    wave_keys = keys_per_unit(alone, target_waves, MIN_SPLIT_KEYS)
-    for item in range(len(tiles)):
-        n_tiles, ctx, ql, qs = int(tiles[item]), int(ctx_len[item]), int(q_len[item]), int(q_start[item])
-        keys = block_keys if in_blocks[item] else wave_keys
-        splits = max(1, min(-(-int(reach[item]) // keys), MAX_SPLITS))
-        first_key = max(0, ctx - int(reach[item])) // 32 * 32
-        begins, ends = _ranges(first_key, ctx, splits) if splits > 1 else (np.zeros(1, np.int32), np.full(1, ctx))
-        splits = len(begins)
-        tile_ids = np.arange(n_tiles, dtype=np.int32)
-        if in_blocks[item]:
-            first = np.arange(0, n_tiles, TILES_PER_BLOCK, dtype=np.int32)
-            block = np.zeros((first.size, splits, BLOCK_UNIT_FIELDS), dtype=np.int32)
-            block[:, :, 0], block[:, :, 1] = item, first[:, None]
-            block[:, :, 2], block[:, :, 3] = begins[None, :], ends[None, :]
-            block[:, :, 4] = -1 if splits == 1 else slot + first[:, None] * splits + np.arange(splits)[None, :]
-            block[:, :, 5], block[:, :, 6], block[:, :, 7], block[:, :, 8] = qs, ql, ctx, splits
-            block_units.append(block.reshape(-1, BLOCK_UNIT_FIELDS))
-        elif splits == 1:
-            units.append(_record(n_tiles, UNIT_FIELDS, item, tile_ids, 0, ctx, -1, qs, ql, ctx))
-        else:
-            block = np.zeros((n_tiles, splits, UNIT_FIELDS), dtype=np.int32)
-            block[:, :, 0], block[:, :, 1] = item, tile_ids[:, None]
-            block[:, :, 2], block[:, :, 3] = begins[None, :], ends[None, :]
-            block[:, :, 4] = slot + tile_ids[:, None] * splits + np.arange(splits)[None, :]
-            block[:, :, 5], block[:, :, 6], block[:, :, 7] = qs, ql, ctx
-            units.append(block.reshape(-1, UNIT_FIELDS))
-        if splits > 1:
-            task = np.zeros((n_tiles, TASK_FIELDS), dtype=np.int32)
-            task[:, 0], task[:, 1], task[:, 3] = item, tile_ids, splits
-            task[:, 2] = slot + tile_ids * splits
-            task[:, 4], task[:, 5] = qs, ql
-            tasks.append(task)
-            slot += n_tiles * splits
+    keys = np.where(in_blocks, keys_per_unit(nblocks, TARGET_BLOCKS, MIN_BLOCK_KEYS),
+                    keys_per_unit(alone, target_waves, MIN_SPLIT_KEYS))
+    # equal ranges (multiples of 32 keys) over [first_key, ctx) of every item
+    first_key = np.maximum(0, ctx_len - reach) // 32 * 32
+    span = ctx_len - first_key
+    splits = np.clip(-(-reach // keys), 1, MAX_SPLITS)
+    chunk = -(-(-(-span // splits)) // 32) * 32
+    splits = np.where(splits > 1, -(-span // np.maximum(chunk, 1)), 1)
+    chunk = np.where(splits > 1, chunk, span)
+    # partial slots: tile t, range s of an item -> base + t * splits + s, for items with several ranges
+    slots_of = np.where(splits > 1, tiles * splits, 0)
+    base = np.cumsum(slots_of) - slots_of
+    num_slots = int(slots_of.sum())
 
-    blocks = np.concatenate(block_units) if block_units else np.zeros((0, BLOCK_UNIT_FIELDS), np.int32)
+    def expand(rows_per_item, fields: int, tiles_per_row: int):
+        """One record per (row, range) of every item: rows are tiles or runs of tiles."""
+        if not rows_per_item.any():
+            return np.zeros((0, fields), dtype=np.int32), None
+        count = rows_per_item * splits
+        item = np.repeat(np.arange(len(tiles)), count)
+        j = np.arange(int(count.sum())) - np.repeat(np.cumsum(count) - count, count)
+        row, s = j // splits[item], j % splits[item]
+        out = np.zeros((item.size, fields), dtype=np.int32)
+        out[:, 0], out[:, 1] = item, row * tiles_per_row
+        begin = first_key[item] + s * chunk[item]
+        out[:, 2], out[:, 3] = begin, np.minimum(begin + chunk[item], ctx_len[item])
+        out[:, 4] = np.where(splits[item] > 1, base[item] + row * tiles_per_row * splits[item] + s, -1)
+        out[:, 5], out[:, 6], out[:, 7] = q_start[item], q_len[item], ctx_len[item]
+        return out, item
+
+    units, _ = expand(alone, UNIT_FIELDS, 1)
+    blocks, block_item = expand(nblocks, BLOCK_UNIT_FIELDS, TILES_PER_BLOCK)
+    if block_item is not None:
+        blocks[:, 8] = splits[block_item]
+    tasks = np.zeros((0, TASK_FIELDS), dtype=np.int32)
+    if num_slots:
+        merged = np.nonzero(splits > 1)[0]
+        count = tiles[merged]
+        item = np.repeat(merged, count)
+        tile = np.arange(int(count.sum())) - np.repeat(np.cumsum(count) - count, count)
+        tasks = np.zeros((item.size, TASK_FIELDS), dtype=np.int32)
+        tasks[:, 0], tasks[:, 1], tasks[:, 2] = item, tile, base[item] + tile * splits[item]
+        tasks[:, 3], tasks[:, 4], tasks[:, 5] = splits[item], q_start[item], q_len[item]
+
     if len(blocks):
         # longest first: a block's work grows with the position of its rows, and the blocks that are
         # started last decide when the kernel ends
@@ -145,5 +137,4 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
         if window:
             begin = np.maximum(begin, pos0[blocks[:, 0]] + (blocks[:, 1].astype(np.int64) * 16) // group - window + 1)
         blocks = blocks[np.argsort(-np.maximum(end - begin, 0), kind="stable")]
-    return AttentionWork(np.concatenate(units) if units else np.zeros((0, UNIT_FIELDS), np.int32),
-                         np.concatenate(tasks) if tasks else np.zeros((0, TASK_FIELDS), np.int32), slot, blocks)
+    return AttentionWork(units, tasks, num_slots, blocks)
