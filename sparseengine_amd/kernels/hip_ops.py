@@ -172,7 +172,8 @@ class MoeWorkspace:
 class HipKernels:
     """The kernel interface of the engine, served by the gfx950 libraries."""
 
-    libraries = ("norm", "rope_kv", "attention_generic", "attention_mfma", "moe", "moe_mfma", "sampling")
+    libraries = ("norm", "rope_kv", "attention_generic", "attention_mfma", "moe", "moe_mfma", "sampling",
+                 "host_work")
 
     def __init__(self):
         if not torch.cuda.is_available():

@@ -14,7 +14,7 @@ from .linear import linear
 
 
 class GQAAttention(Part):
-    kernel_libraries = ("rope_kv", "attention_generic", "attention_mfma")
+    kernel_libraries = ("rope_kv", "attention_generic", "attention_mfma", "host_work")
 
     def __init__(self, spec: AttentionSpec, hidden_size: int):
         if spec.num_kv_heads <= 0 or spec.num_heads % spec.num_kv_heads:

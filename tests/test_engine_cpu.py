@@ -268,3 +268,24 @@ def test_block_work_lists_for_many_rows_cover_every_tile_once_longest_first():
     # a head size the block kernel does not take, and a step of single tokens, keep the per-wavefront list
     assert len(build_attention_work([2048], [2048], 6, 8, 0, head_dim=160).block_units) == 0
     assert len(build_attention_work([1] * 8, [300] * 8, 6, 8, 0, head_dim=128).block_units) == 0
+
+
+def test_compiled_work_list_builder_gives_the_same_lists():
+    """csrc/host_work.hip against the numpy builder, list for list, on random steps."""
+    import numpy as np
+    from sparseengine_amd.kernels import attention_work as aw
+    if aw._native_library() is None:
+        pytest.skip("the compiled builder cannot be built here")
+    rng = np.random.default_rng(0)
+    for _ in range(400):
+        items = int(rng.integers(1, 12))
+        q = [int(rng.choice([1, 1, 1, 2, 7, 40, 300, 2048])) for _ in range(items)]
+        c = [n + int(rng.integers(0, 70000)) * int(rng.integers(0, 2)) + int(rng.integers(0, 300)) for n in q]
+        group, kvh = int(rng.choice([1, 2, 6, 16, 20])), int(rng.choice([1, 2, 8]))
+        window, head_dim = int(rng.choice([0, 0, 64, 1000])), int(rng.choice([0, 64, 128, 160]))
+        target = int(rng.choice([1024, 256]))
+        a = aw.build_attention_work(q, c, group, kvh, window, target, head_dim)
+        b = aw.build_attention_work_numpy(q, c, group, kvh, window, target, head_dim)
+        assert a.num_slots == b.num_slots
+        assert np.array_equal(a.units, b.units) and np.array_equal(a.tasks, b.tasks)
+        assert np.array_equal(a.block_units, b.block_units)
