@@ -261,7 +261,7 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
     expected = {r: plain.logits(t).numpy() for r, t in requests.items()}
     records, peak = traces.mixed(requests, seed=1)
     runner = runner_for(folder, dtype, tokens=peak)
-    assert [(g.request.window, g.positions) for g in runner.cache.groups] == [(None, [0, 3]), (24, [2])]
+    assert [(g.request.window, g.positions) for g in runner.cache.groups] == [(None, [0, 3, 5]), (24, [2])]
     assert list(runner.cache.state_positions) == [1]
     from sparseengine_amd.engine.replay import replay_step
     out = {}

@@ -1,7 +1,8 @@
 """A toy architecture defined wholly in the tests, to show that parts, cache groups, state slots
 and the run order are general: layers differ in mixer (full attention, windowed attention, a
-recurrent mixer with state of its own) and in feed-forward (dense, routed), the schedule runs a
-layer twice and lets one position read another position's cache.  Nothing in ``sparseengine_amd``
+recurrent mixer with state of its own), in feed-forward (dense, routed experts, a feed-forward
+with a routing rule of its own) and in position encoding (rotary, none, a rotation with its own
+table), the schedule runs a layer twice and lets one position read another position's cache.  Nothing in ``sparseengine_amd``
 knows about it: it registers itself through the public registries.  It is no model of anyone's.
 """
 from __future__ import annotations
@@ -14,7 +15,7 @@ import torch
 from sparseengine_amd.config.registry import Architecture, WeightSource, register_architecture
 from sparseengine_amd.config.specs import (AttentionSpec, DenseMLPSpec, LayerSpec, ModelSpec, MoESpec, NoPositionSpec,
                                            NormSpec, RotarySpec, ScheduleEntry)
-from sparseengine_amd.parts import MIXERS, ParamDecl, Part, StateRequest, build_model
+from sparseengine_amd.parts import FEED_FORWARDS, MIXERS, POSITIONS, ParamDecl, Part, StateRequest, build_model
 from tests.plain import minimax_m2 as P
 
 
@@ -59,6 +60,61 @@ class DecayMixer(Part):
 MIXERS.register("toy_decay", lambda spec, hidden_size: DecayMixer(spec, hidden_size))
 
 
+# ------------------------------------------------------------------ a feed-forward with its own routing
+@dataclass(frozen=True)
+class SignRoutedSpec:
+    kind: ClassVar[str] = "toy_sign_routed"
+    intermediate_size: int = 16
+
+
+class SignRoutedFFN(Part):
+    """Two small MLPs; a token goes to the one named by the sign of ``x . probe`` (hard top-1)."""
+
+    def __init__(self, spec: SignRoutedSpec, hidden_size: int):
+        self.spec, self.hidden_size = spec, hidden_size
+
+    def param_decls(self):
+        i, h = self.spec.intermediate_size, self.hidden_size
+        return {"probe": ParamDecl((h,), "float32"), "up": ParamDecl((2, i, h)), "down": ParamDecl((2, h, i))}
+
+    def forward(self, fb, x):
+        p = self.params
+        choice = (x.float() @ p["probe"].float() > 0).long()                   # [T]
+        up, down = p["up"].float()[choice], p["down"].float()[choice]          # [T, i, h], [T, h, i]
+        hidden = torch.nn.functional.silu(torch.einsum("tih,th->ti", up, x.float()))
+        return torch.einsum("thi,ti->th", down, hidden).to(x.dtype)
+
+
+FEED_FORWARDS.register("toy_sign_routed", lambda spec, hidden_size, chunk_tokens=0: SignRoutedFFN(spec, hidden_size))
+
+
+# ------------------------------------------------------------------ a position encoding with its own table
+@dataclass(frozen=True)
+class LinearRotarySpec:
+    kind: ClassVar[str] = "toy_linear_rotary"
+    rotary_dim: int = 8
+    slope: float = 0.05
+    max_position: int = 1024
+
+
+class LinearRotary(Part):
+    """NeoX-paired rotation whose angle of pair d at position p is ``p * slope * (d + 1)``."""
+
+    def __init__(self, spec: LinearRotarySpec, head_dim: int):
+        self.spec, self.rotary_dim, self.table = spec, spec.rotary_dim, None
+
+    def prepare(self, device) -> None:
+        angles = linear_rotary_angles(torch.arange(self.spec.max_position), self.spec.rotary_dim, self.spec.slope)
+        self.table = torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous().to(device)
+
+
+def linear_rotary_angles(positions, rotary_dim: int, slope: float):
+    return positions.float()[:, None] * (slope * torch.arange(1, rotary_dim // 2 + 1, dtype=torch.float32))[None, :]
+
+
+POSITIONS.register("toy_linear_rotary", lambda spec, head_dim: LinearRotary(spec, head_dim))
+
+
 # ------------------------------------------------------------------ the architecture
 def parse(raw: dict) -> dict:
     return raw
@@ -69,13 +125,21 @@ def _layer_spec(cfg, layer) -> LayerSpec:
     if layer["mixer"] == "decay":
         mixer = DecayMixerSpec(state_size=layer["state_size"], decay=layer["decay"])
     else:
-        rotary = (RotarySpec(rotary_dim=layer["rotary_dim"], theta=cfg["rope_theta"],
-                             max_position=cfg["max_position_embeddings"]) if layer["rotary_dim"] else NoPositionSpec())
+        if layer.get("linear_rotary"):
+            rotary = LinearRotarySpec(rotary_dim=layer["rotary_dim"], slope=layer["linear_rotary"],
+                                      max_position=cfg["max_position_embeddings"])
+        elif layer["rotary_dim"]:
+            rotary = RotarySpec(rotary_dim=layer["rotary_dim"], theta=cfg["rope_theta"],
+                                max_position=cfg["max_position_embeddings"])
+        else:
+            rotary = NoPositionSpec()
         mixer = AttentionSpec(num_heads=layer["heads"], num_kv_heads=layer["kv_heads"], head_dim=layer["head_dim"],
                               scale=layer["head_dim"] ** -0.5, qk_norm="flat" if layer.get("qk_norm") else "none",
                               qk_norm_eps=cfg["eps"], window=layer.get("window"), position=rotary)
     if layer["ffn"] == "dense":
         ffn = DenseMLPSpec(intermediate_size=layer["intermediate"])
+    elif layer["ffn"] == "sign":
+        ffn = SignRoutedSpec(intermediate_size=layer["intermediate"])
     else:
         ffn = MoESpec(num_experts=layer["experts"], top_k=layer["top_k"], intermediate_size=layer["intermediate"],
                       scoring=layer.get("scoring", "sigmoid"), selection_bias=layer.get("bias", True),
@@ -102,13 +166,15 @@ def random_tensor(cfg, name, shape, generator, options):
         return 1.0 + 0.2 * noise
     if name.endswith("router_bias"):
         return 0.3 * noise
+    if name.endswith("probe"):
+        return noise
     return noise * float(options.get("std", 0.1))
 
 
 TOY = register_architecture(Architecture(
     name="ToyForCausalLM", model_types=("toy",), parse_config=parse, build_spec=build_spec,
     weight_sources=weight_sources, ignored_tensor=lambda name: False, random_tensor=random_tensor,
-    stored_dtype=lambda name: "float32" if name.endswith(("router", "router_bias")) else "bfloat16",
+    stored_dtype=lambda name: "float32" if name.endswith(("router", "router_bias", "probe")) else "bfloat16",
     config_to_dict=lambda cfg: dict(cfg)))
 
 TOY_CONFIG = dict(
@@ -121,9 +187,11 @@ TOY_CONFIG = dict(
         dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, ffn="moe", experts=4, top_k=3,
              intermediate=24),
         dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, ffn="dense", intermediate=48),
+        dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=8, linear_rotary=0.05, ffn="sign",
+             intermediate=20),
     ],
-    # layer 0 runs twice (two caches); the last position reads the cache of position 0 (same geometry)
-    schedule=[dict(layer=0), dict(layer=1), dict(layer=2), dict(layer=0), dict(layer=3, cache_from=0)])
+    # layer 0 runs twice (two caches); position 4 reads the cache of position 0 (same geometry)
+    schedule=[dict(layer=0), dict(layer=1), dict(layer=2), dict(layer=0), dict(layer=3, cache_from=0), dict(layer=4)])
 
 
 # ------------------------------------------------------------------ its plain implementation
@@ -162,7 +230,10 @@ class PlainToy:
                     q = P.flat_qk_norm(q, w[p + "mixer.q_norm"], cfg["eps"])
                     k = P.flat_qk_norm(k, w[p + "mixer.k_norm"], cfg["eps"])
                 q, k, v = q.reshape(T, H, D), k.reshape(T, Hkv, D), v.reshape(T, Hkv, D)
-                if R:
+                if layer.get("linear_rotary"):
+                    angles = linear_rotary_angles(pos, R, layer["linear_rotary"])
+                    q, k = P.partial_rope(q, angles.cos(), angles.sin(), R), P.partial_rope(k, angles.cos(), angles.sin(), R)
+                elif R:
                     cos, sin = P.rope_angles(pos, R, cfg["rope_theta"])
                     q, k = P.partial_rope(q, cos, sin, R), P.partial_rope(k, cos, sin, R)
                 if entry.get("cache_from") is not None:
@@ -175,6 +246,10 @@ class PlainToy:
             if layer["ffn"] == "dense":
                 gu = m @ w[p + "ffn.gate_up"].T
                 x = (torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]) @ w[p + "ffn.down"].T
+            elif layer["ffn"] == "sign":
+                x = torch.stack([
+                    w[p + "ffn.down"][int(t @ w[p + "ffn.probe"] > 0)]
+                    @ torch.nn.functional.silu(w[p + "ffn.up"][int(t @ w[p + "ffn.probe"] > 0)] @ t) for t in m])
             else:
                 logits = m @ w[p + "ffn.router"].T
                 scores = torch.softmax(logits, -1) if layer.get("scoring") == "softmax" else torch.sigmoid(logits)
