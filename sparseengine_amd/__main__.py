@@ -17,17 +17,22 @@ import sys
 import typing
 
 
-def _add_dataclass_options(parser, cls, skip=()):
+def _add_dataclass_options(parser, cls, skip=(), prefix_if_taken: str = ""):
+    """One option per field.  A name another dataclass has taken already gets ``prefix_if_taken``
+    (``eos_token_ids`` is a field of ``Config`` and of ``SamplingParams``: the request-level one is
+    ``--sampling-eos-token-ids``)."""
     hints = typing.get_type_hints(cls)
+    taken = {action.dest for action in parser._actions}
     for f in dataclasses.fields(cls):
         if not f.init or f.name in skip:
             continue
-        flag = "--" + f.name.replace("_", "-")
+        dest = f.name if f.name not in taken else prefix_if_taken + f.name
+        flag = "--" + dest.replace("_", "-")
         kind = hints.get(f.name, str)
         if kind is bool:
-            parser.add_argument(flag, dest=f.name, action=argparse.BooleanOptionalAction, default=None)
+            parser.add_argument(flag, dest=dest, action=argparse.BooleanOptionalAction, default=None)
         else:
-            parser.add_argument(flag, dest=f.name, default=None, help=f"({kind})")
+            parser.add_argument(flag, dest=dest, default=None, help=f"({kind})")
 
 
 def _coerce(value: str):
@@ -37,18 +42,18 @@ def _coerce(value: str):
         return value
 
 
-def _collect(args, cls, skip=()):
+def _collect(args, cls, skip=(), prefix: str = ""):
     out = {}
     for f in dataclasses.fields(cls):
         if not f.init or f.name in skip:
             continue
-        value = getattr(args, f.name, None)
+        value = getattr(args, prefix + f.name, None) if hasattr(args, prefix + f.name) else getattr(args, f.name, None)
         if value is not None:
             out[f.name] = _coerce(value) if isinstance(value, str) else value
     return out
 
 
-def main(argv=None) -> int:
+def build_parser() -> argparse.ArgumentParser:
     from .config.runtime import Config
     from .sampling.params import SamplingParams
     parser = argparse.ArgumentParser(prog="python -m sparseengine_amd", description=__doc__,
@@ -61,7 +66,7 @@ def main(argv=None) -> int:
     gen.add_argument("--prompt-ids", action="append", default=[],
                      help="prompt as JSON list of token ids, or a file with one JSON list per line; repeatable")
     _add_dataclass_options(gen, Config, skip=("model",))
-    _add_dataclass_options(gen, SamplingParams)
+    _add_dataclass_options(gen, SamplingParams, prefix_if_taken="sampling_")
 
     rnd = sub.add_parser("random", help="write a random-weights model folder")
     rnd.add_argument("--config", required=True, help="config.json file (or JSON text) of the architecture")
@@ -73,11 +78,18 @@ def main(argv=None) -> int:
 
     rep = sub.add_parser("replay", help="trace replay (see bin/trace_run)", add_help=False)
     rep.add_argument("rest", nargs=argparse.REMAINDER)
+    return parser
 
+
+def main(argv=None) -> int:
+    from .config.runtime import Config
+    from .sampling.params import SamplingParams
+    argv = sys.argv[1:] if argv is None else list(argv)
+    if argv and argv[0] == "replay":       # its options are its own (they begin with dashes, which the
+        from .engine.replay import main as replay_main      # sub-command parser would claim)
+        return replay_main(argv[1:])
+    parser = build_parser()
     args = parser.parse_args(argv)
-    if args.command == "replay":
-        from .engine.replay import main as replay_main
-        return replay_main(args.rest)
     if args.command == "random":
         import os
         from .weights.random_weights import write_model_folder
@@ -99,7 +111,7 @@ def main(argv=None) -> int:
     if not prompts:
         parser.error("give at least one --prompt or --prompt-ids")
     llm = LLM(args.model, **_collect(args, Config, skip=("model",)))
-    params = SamplingParams(**_collect(args, SamplingParams))
+    params = SamplingParams(**_collect(args, SamplingParams, prefix="sampling_"))
     for prompt, out in zip(prompts, llm.generate(prompts, params, use_tqdm=False)):
         print(json.dumps({"prompt": prompt, **out}))
     return 0

@@ -45,7 +45,11 @@ def write_model_folder(folder: str, raw_config: dict, seed: int, options: dict |
     decls = build_model(arch.build_spec(cfg)).all_param_decls()
     os.makedirs(folder, exist_ok=True)
     tensors = {src.name: value.contiguous() for src, value in checkpoint_tensors(arch, cfg, decls, seed, options)}
-    save_file(tensors, os.path.join(folder, "model.safetensors"))
+    weights_file = os.path.join(folder, "model.safetensors")
+    save_file(tensors, weights_file)
+    umask = os.umask(0)       # the writer leaves the file readable by its owner only: give it the usual mode
+    os.umask(umask)
+    os.chmod(weights_file, 0o666 & ~umask)
     with open(os.path.join(folder, "config.json"), "w") as fh:
         json.dump(arch.config_to_dict(cfg), fh, indent=1)
     return folder

@@ -226,3 +226,29 @@ def test_rope_scaling_tables():
                                                            "original_max_position_embeddings": 4096})
     assert factor == pytest.approx(0.1 * torch.log(torch.tensor(4.0)).item() + 1.0)
     assert torch.equal(inv[:8], base[:8]) and torch.allclose(inv[-4:], base[-4:] / 4)         # fast dims kept, slow dims scaled
+
+
+def test_command_line_options_and_random_folder(tmp_path):
+    """Every field of Config and SamplingParams is an option; the one name both have is told apart;
+    ``random`` writes a folder that loads."""
+    from sparseengine_amd.__main__ import _collect, build_parser, main
+    from sparseengine_amd.sampling.params import SamplingParams
+    parser = build_parser()
+    args = parser.parse_args(["generate", "--model", "/x", "--prompt-ids", "[1, 2]", "--max-tokens", "6",
+                              "--temperature", "0.8", "--top-k", "5", "--seed", "7", "--dtype", "float32",
+                              "--eos-token-ids", "[3]", "--sampling-eos-token-ids", "[4, 5]", "--kv-page-size", "16",
+                              "--no-ignore-eos", "--max-num-batched-tokens", "auto"])
+    assert _collect(args, Config, skip=("model",)) == {"eos_token_ids": [3], "dtype": "float32", "kv_page_size": 16,
+                                                       "max_num_batched_tokens": "auto"}
+    assert _collect(args, SamplingParams, prefix="sampling_") == {
+        "temperature": 0.8, "top_k": 5, "max_tokens": 6, "ignore_eos": False, "eos_token_ids": [4, 5], "seed": 7}
+    SamplingParams(**_collect(args, SamplingParams, prefix="sampling_"))
+    with pytest.raises(SystemExit):
+        parser.parse_args(["generate", "--model", "/x", "--no-such-option", "1"])
+    config_file = tmp_path / "config.json"
+    config_file.write_text(json.dumps(TINY_A))
+    out = tmp_path / "model"
+    assert main(["random", "--config", str(config_file), "--out", str(out), "--seed", "3"]) == 0
+    assert json.load(open(out / "config.json"))["hidden_size"] == TINY_A["hidden_size"]
+    params, _ = load(str(out))            # the written folder loads, tensor for tensor
+    assert params["embed.weight"].shape == (TINY_A["vocab_size"], TINY_A["hidden_size"])

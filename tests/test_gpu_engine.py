@@ -116,6 +116,27 @@ def test_greedy_generation_through_the_entry_point(tmp_path):
     assert alone == mixed
 
 
+def test_command_line_generates_what_the_entry_point_generates(tmp_path, capsys):
+    import json
+    from sparseengine_amd import LLM, SamplingParams
+    from sparseengine_amd.__main__ import main
+    folder = make_folder(tmp_path, "B_loud")
+    prompts = [random_tokens(n, 1000, 40 + n) for n in (7, 23)]
+    llm = LLM(folder, dtype="float32", num_kvcache_slots=512, kv_page_size=16)
+    expected = llm.generate(prompts, SamplingParams(temperature=0.7, top_k=20, max_tokens=9, ignore_eos=True, seed=5),
+                            use_tqdm=False)
+    del llm
+    ids_file = tmp_path / "prompts.jsonl"
+    ids_file.write_text(json.dumps(prompts[1]) + "\n")
+    capsys.readouterr()
+    assert main(["generate", "--model", folder, "--prompt-ids", json.dumps(prompts[0]), "--prompt-ids", str(ids_file),
+                 "--dtype", "float32", "--num-kvcache-slots", "512", "--kv-page-size", "16", "--temperature", "0.7",
+                 "--top-k", "20", "--max-tokens", "9", "--ignore-eos", "--seed", "5"]) == 0
+    lines = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    assert [line["prompt"] for line in lines] == prompts
+    assert [line["token_ids"] for line in lines] == [e["token_ids"] for e in expected]
+
+
 def test_weights_stored_in_32_bit_stay_so_under_bfloat16(tmp_path):
     folder = make_folder(tmp_path, "A_loud")
     path = os.path.join(folder, "model.safetensors")

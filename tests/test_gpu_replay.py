@@ -151,3 +151,12 @@ def test_trace_run_program(model, dtype, tmp_path):
     for step, arr in inproc.items():
         assert np.array_equal(arr, logits[step]), f"step {step}: the program and the in-process replay differ"
     compare(dtype, traces.gather(records, logits), model, routing)
+    if dtype == "float32":      # the same program as a sub-command of the package
+        other = tmp_path / "out_module"
+        proc = subprocess.run(
+            [sys.executable, "-m", "sparseengine_amd", "replay", "--model", folder, "--dtype", dtype, "--out", str(other),
+             "--max-tokens", str(peak), "--page-size", "16"], cwd=ROOT,
+            input="".join(json.dumps(r) + "\n" for r in records[:6]), capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        for r in records[:6]:
+            assert np.array_equal(np.fromfile(other / f"{r['step']}.f32", dtype="<f4").reshape(-1, vocab), logits[r["step"]])
