@@ -2,6 +2,7 @@
 CPU: the kernel twins stand in for the HIP kernels, everything else is the product's own code.
 The kernels themselves are tested on the GPU."""
 import json
+import os
 
 import numpy as np
 import pytest
@@ -289,3 +290,24 @@ def test_compiled_work_list_builder_gives_the_same_lists():
         assert a.num_slots == b.num_slots
         assert np.array_equal(a.units, b.units) and np.array_equal(a.tasks, b.tasks)
         assert np.array_equal(a.block_units, b.block_units)
+
+
+def test_text_prompts_go_through_the_folders_tokenizer(model, tmp_path):
+    """A tokenizer.json in the model folder: strings in, text out, same tokens as the ids would give."""
+    import shutil
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+    folder, _, _, plain = model
+    copy = str(tmp_path / "with_tokenizer")
+    shutil.copytree(folder, copy)
+    vocab = {f"w{i}": i for i in range(plain.cfg.vocab_size)}
+    tok = Tokenizer(WordLevel(vocab, unk_token="w0"))
+    tok.pre_tokenizer = Whitespace()
+    tok.save(os.path.join(copy, "tokenizer.json"))
+    engine = llm(copy)
+    ids = [7, 300, 41, 41, 9]
+    text = " ".join(f"w{i}" for i in ids)
+    out, = engine.generate([text], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True), use_tqdm=False)
+    assert out["token_ids"] == plain.greedy(ids, 6)
+    assert out["text"].split() == [f"w{i}" for i in out["token_ids"]]
