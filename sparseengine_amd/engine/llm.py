@@ -64,6 +64,66 @@ class CacheOracle(MemoryOracle):
         self.cache.free(seq_id)
 
 
+class StepTimes:
+    """Wall time of the sections of ``LLM.step`` (``enable_profiler``): the device is waited for at each
+    section's end, so that a section is charged with the work it started.  The reference's profiler
+    (utils/profiler.py:14-105) keeps named sections and prints their totals; so does ``report``."""
+
+    def __init__(self, enabled: bool, device):
+        self.enabled, self.device = enabled, device
+        self.seconds: dict[str, float] = {}
+        self.calls: dict[str, int] = {}
+        self._mark = 0.0
+
+    def start(self) -> None:
+        if self.enabled:
+            self._mark = time.perf_counter()
+
+    def section(self, name: str) -> None:
+        """Close the section that began at the last ``start`` or ``section`` call."""
+        if not self.enabled:
+            return
+        if getattr(self.device, "type", str(self.device)) == "cuda":
+            torch.cuda.synchronize()
+        now = time.perf_counter()
+        self.seconds[name] = self.seconds.get(name, 0.0) + now - self._mark
+        self.calls[name] = self.calls.get(name, 0) + 1
+        self._mark = now
+
+    def report(self) -> str:
+        total = sum(self.seconds.values()) or 1.0
+        return "\n".join(f"{name:10s} {1e3 * sec:10.1f} ms {100 * sec / total:5.1f} %  {self.calls[name]} calls"
+                         for name, sec in sorted(self.seconds.items(), key=lambda kv: -kv[1]))
+
+
+class ThroughputLog:
+    """A line on stderr every ``interval`` seconds with the tokens per second since the last one
+    (``throughput_log_interval_s``; 0 switches it off).  The reference logs from a thread of its own
+    (engine/llm_engine.py:90-230); here the step that crosses the interval writes the line."""
+
+    def __init__(self, interval: float, stream=None):
+        self.interval, self.stream = float(interval), stream
+        self.prefill = self.decode = self.steps = 0
+        self.since = time.perf_counter()
+
+    def record(self, signed_tokens: int, running: int, waiting: int) -> None:
+        if self.interval <= 0:
+            return
+        if signed_tokens > 0:
+            self.prefill += signed_tokens
+        else:
+            self.decode -= signed_tokens
+        self.steps += 1
+        now = time.perf_counter()
+        if now - self.since < self.interval:
+            return
+        dt = now - self.since
+        print(f"[throughput] prefill {self.prefill / dt:.0f} tok/s, decode {self.decode / dt:.0f} tok/s, "
+              f"{self.steps} steps, {running} running, {waiting} waiting", file=self.stream or sys.stderr, flush=True)
+        self.prefill = self.decode = self.steps = 0
+        self.since = now
+
+
 class LLM:
     def __init__(self, model: str, **kwargs):
         kernels = kwargs.pop("_kernels", None)           # test seam: the kernel twins on the CPU
@@ -92,6 +152,8 @@ class LLM:
         self.tokenizer = self._load_tokenizer(model)
         self.vocab_size = self.runner.spec.vocab_size
         self.last_step_seconds = 0.0
+        self.step_times = StepTimes(config.enable_profiler, self.runner.device)
+        self.throughput_log = ThroughputLog(config.throughput_log_interval_s)
 
     @staticmethod
     def _load_tokenizer(folder: str):
@@ -139,13 +201,17 @@ class LLM:
         """Schedule, run, sample, account.  Returns (finished, signed token count) where finished is
         a list of (seq_id, completion token ids, token logprobs, top logprobs)."""
         started = time.perf_counter()
+        times = self.step_times
+        times.start()
         schedule = self.scheduler.schedule()
+        times.section("schedule")
         if not schedule.items:
             return [], 0
         entries = [StepEntry(i.seq.seq_id, i.seq.next_tokens(i.num_tokens), [i.num_tokens - 1] if i.wants_logits else [])
                    for i in schedule.items]
         try:
             logits = self.runner.step(entries)
+            times.section("model")
             wanting = [i.seq for i in schedule.items if i.wants_logits]
             sampled, logprobs = {}, {}
             if wanting:
@@ -157,6 +223,7 @@ class LLM:
                     sampled[s.seq_id] = t
                     logprobs[s.seq_id] = (c, top)
             self.method.after_step(None)
+            times.section("sample")
         except Exception:
             self.scheduler.fail_step(schedule)
             raise
@@ -164,9 +231,12 @@ class LLM:
         finished = self.scheduler.postprocess(schedule, sampled, logprobs)
         if self.config.validate_runtime_invariants:
             self.runner.cache.check_invariants()
+        times.section("account")
         self.last_step_seconds = time.perf_counter() - started
         outputs = [(s.seq_id, s.completion_token_ids, s.token_logprobs, s.top_logprobs) for s in finished]
-        return outputs, (prefill if prefill else -decode)
+        signed = prefill if prefill else -decode
+        self.throughput_log.record(signed, len(self.scheduler.running), len(self.scheduler.waiting))
+        return outputs, signed
 
     # ------------------------------------------------------------------ the blocking call
     def generate(self, prompts, sampling_params, use_tqdm: bool = True) -> list[dict]:

@@ -311,3 +311,21 @@ def test_text_prompts_go_through_the_folders_tokenizer(model, tmp_path):
     out, = engine.generate([text], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True), use_tqdm=False)
     assert out["token_ids"] == plain.greedy(ids, 6)
     assert out["text"].split() == [f"w{i}" for i in out["token_ids"]]
+
+
+def test_step_times_and_throughput_lines(model):
+    """``enable_profiler`` and ``throughput_log_interval_s`` do what their names say."""
+    import io
+    folder, requests, _, _ = model
+    engine = llm(folder, enable_profiler=True, throughput_log_interval_s=1e-9)
+    engine.throughput_log.stream = lines = io.StringIO()
+    prompts = [t[:9] for t in list(requests.values())[:2]]
+    engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True), use_tqdm=False)
+    assert set(engine.step_times.seconds) == {"schedule", "model", "sample", "account"}
+    assert engine.step_times.calls["model"] == engine.step_times.calls["sample"] >= 4
+    assert "model" in engine.step_times.report()
+    logged = [l for l in lines.getvalue().splitlines() if l.startswith("[throughput]")]
+    assert len(logged) == engine.step_times.calls["model"] and "decode" in logged[-1]
+    quiet = llm(folder)
+    quiet.generate(prompts[:1], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True), use_tqdm=False)
+    assert not quiet.step_times.seconds
