@@ -278,16 +278,6 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 #define TILED_ROW_TILES 2   // row tiles per wavefront: 8 per block
 #define TILED_STAGES 4      // steps of keys in shared memory at a time
 
-// m0 (the destination's base) is set and used inside one statement; naming it as clobbered draws a
-// warning about reserved registers that does not apply here.
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void load16_to_lds(const void* src, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-               :
-               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)   // the base is the same in all lanes
-               : "memory", "m0");
-}
-
 // Maximum / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 that share a row: two register swaps
 // between halves and between rows of 16 lanes instead of trips through the shared-memory crossbar.
 // The library's fmaxf quiets signalling NaNs first, one more instruction per operand; scores are

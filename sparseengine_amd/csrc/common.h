@@ -212,3 +212,18 @@ __device__ __forceinline__ void stage_row(const T* src, float* dst, int n) {
     }
   }
 }
+
+// 16 bytes per lane from global memory straight into shared memory, no register in between: lane l's
+// bytes land at (wave-uniform) lds_addr + 16 l.  The compiler does not see the write: the caller
+// waits for it by hand (s_waitcnt vmcnt) before a barrier, and reads the data only after that barrier.
+// (m0, the destination's base, is set and used inside one statement; naming it as clobbered draws a
+// warning about reserved registers that does not apply here)
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void load16_to_lds(const void* src, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)   // the base is the same in all lanes
+               : "memory", "m0");
+}
+
+

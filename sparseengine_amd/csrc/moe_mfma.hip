@@ -412,6 +412,189 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
   return SE_OK;
 }
 
+// ---------------------------------------------------------------------------------------- //
+// Wide tiles (an expert has hundreds of rows: steps of many thousand tokens).  The 64 x 128 tile
+// above does 43 flop for each byte it takes from the L2, and that is where it stops (about 455
+// TFLOP/s measured).  Here a block computes 128 rows x 256 weight rows (87 flop per byte): four
+// wavefronts, each 64 rows x 128 weight rows (MODE 0: 64 gate rows and the matching 64 up rows, so
+// that the SwiGLU product stays inside a lane).  A step of 64 along K is 48 chunks of 1 KB that go
+// from memory straight into shared memory in operand order (lane l's 16 bytes of a chunk are what
+// lane l feeds the matrix core), three stages deep; twelve chunks per wavefront and step.
+//   MODE 0: out[a, n0 + 64 wc + 16 cb + ...] from gate rows n0 + 64 wc ..., up rows N + n0 + 64 wc ...
+//   MODE 1: out[a, n0 + 128 wc + 16 cb + ...] * route_weight[a]
+// Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1); tiles of 128 sorted rows.
+// ---------------------------------------------------------------------------------------- //
+#define WIDE_STAGES 3
+#define WIDE_CHUNKS 48      // per stage: 32 of weights (16 row blocks x 2 halves of the step), 16 of activations
+
+template <int MODE>
+__global__ void __launch_bounds__(256)
+grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                         bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                         const int32_t* __restrict__ tile_expert,
+                         const int32_t* __restrict__ counters,
+                         const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                         int K) {
+  constexpr int BM = 128;
+  constexpr int OUT_COLS = MODE == 0 ? 128 : 256;
+  int tile, column_block;
+  if (!xcd_work_item(N / OUT_COLS, counters[0], tile, column_block)) return;  // uniform
+  extern __shared__ __align__(16) uint4 wide_shared[];     // WIDE_STAGES x WIDE_CHUNKS x 64 vectors, then the rows
+  int32_t* rows = reinterpret_cast<int32_t*>(wide_shared + WIDE_STAGES * WIDE_CHUNKS * 64);
+  static_assert(WIDE_STAGES * WIDE_CHUNKS * 1024 <= 160 * 1024 - 1024, "stages must fit shared memory");
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (SE_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SE_WAVE);
+  const int col = lane & 15, kgroup = lane >> 4;
+  const int wr = wave >> 1, wc = wave & 1;       // the wave's 64 rows and 128 weight rows of the tile
+  const int expert = tile_expert[tile];
+  const int n0 = column_block * OUT_COLS;
+  if (tid < BM) rows[tid] = sorted[tile * BM + tid];
+  __syncthreads();
+
+  const int64_t w_rows = MODE == 0 ? 2 * static_cast<int64_t>(N) : N;
+  const bf16_t* we = w + static_cast<int64_t>(expert) * w_rows * K;
+
+  // Row block rb (16 rows) of the tile's 256 weight rows: blocks 8 wc' ... 8 wc' + 7 belong to the
+  // wave column wc'; in MODE 0 its first four are gate rows, its last four the matching up rows.
+  auto weight_row = [&](int rb, int r) -> int64_t {
+    const int wcol = rb >> 3, cb = rb & 7;
+    if (MODE == 0) return (cb < 4 ? 0 : static_cast<int64_t>(N)) + n0 + 64 * wcol + 16 * (cb & 3) + r;
+    return n0 + 128 * wcol + 16 * cb + r;
+  };
+  // The wave brings six "row block pairs" of a step: pair p < 16 is weight row block p, pair p >= 16
+  // is activation row block p - 16; both halves of the step (chunks 2 p and 2 p + 1).
+  const bf16_t* src[6];
+#pragma unroll
+  for (int j = 0; j < 6; ++j) {
+    const int p = wave * 6 + j;
+    if (p < 16) {
+      src[j] = we + weight_row(p, col) * K + kgroup * 8;
+    } else {
+      const int a = rows[(p - 16) * 16 + col];
+      const int64_t token = a < assignments ? static_cast<int64_t>(MODE == 0 ? a / top_k : a) : 0;  // padding reads row 0
+      src[j] = in + token * K + kgroup * 8;
+    }
+  }
+  const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wide_shared));
+  auto issue = [&](int step) {
+    const uint32_t dst = stage_base + static_cast<uint32_t>((step % WIDE_STAGES) * WIDE_CHUNKS + wave * 12) * 1024u;
+    const int k0 = step * 64;
+#pragma unroll
+    for (int j = 0; j < 6; ++j) {
+      load16_to_lds(src[j] + k0, dst + static_cast<uint32_t>(2 * j) * 1024u);
+      load16_to_lds(src[j] + k0 + 32, dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
+    }
+  };
+
+  floatx4 acc[8][4];      // [weight row block of the wave][row block of the wave]
+#pragma unroll
+  for (int cb = 0; cb < 8; ++cb)
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) acc[cb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int steps = K / 64;
+#pragma unroll
+  for (int j = 0; j < WIDE_STAGES - 1; ++j)
+    if (j < steps) issue(j);
+  for (int step = 0; step < steps; ++step) {
+    // this step's data: all but the loads of the steps after it must have come back
+    if (step + WIDE_STAGES - 2 < steps) {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((WIDE_STAGES - 2) * 12));    // vmcnt((stages - 2) * 12)
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);                               // vmcnt(0)
+    }
+    __builtin_amdgcn_s_barrier();   // everyone's part of the step is in; everyone has left step - 1
+    asm volatile("" ::: "memory");
+    if (step + WIDE_STAGES - 1 < steps) issue(step + WIDE_STAGES - 1);   // into the buffer step - 1 used
+    const uint4(*chunk)[64] = reinterpret_cast<const uint4(*)[64]>(wide_shared) + (step % WIDE_STAGES) * WIDE_CHUNKS;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      uint4 bfrag[4];
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) bfrag[mb] = chunk[2 * (16 + 4 * wr + mb) + sub][lane];
+#pragma unroll
+      for (int cb = 0; cb < 8; ++cb) {
+        const uint4 afrag = chunk[2 * (8 * wc + cb) + sub][lane];
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+          acc[cb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, afrag),
+                                                               __builtin_bit_cast(bf16x8, bfrag[mb]),
+                                                               acc[cb][mb], 0, 0, 0);
+      }
+    }
+    asm volatile("" ::: "memory");
+  }
+
+  // lane (kgroup, col): acc[cb][mb][i] belongs to weight row 4 * kgroup + i of block cb, tile row 64 wr + 16 mb + col
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    const int a = rows[64 * wr + 16 * mb + col];
+    if (a >= assignments) continue;
+    bf16_t* o_row = out + static_cast<int64_t>(a) * N + n0 + 4 * kgroup;
+    if (MODE == 0) {
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) {
+        uint16_t y[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float gate = round_to<bf16_t>(acc[cb][mb][i]);
+          const float up = round_to<bf16_t>(acc[cb + 4][mb][i]);
+          const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
+          y[i] = float_to_bf16_bits(act * up);
+        }
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(y[0]) | (static_cast<uint32_t>(y[1]) << 16);
+        packed.y = static_cast<uint32_t>(y[2]) | (static_cast<uint32_t>(y[3]) << 16);
+        *reinterpret_cast<uint2*>(o_row + 64 * wc + 16 * cb) = packed;
+      }
+    } else {
+      const float rw = route_weight[a];
+#pragma unroll
+      for (int cb = 0; cb < 8; ++cb) {
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][0] * rw)) |
+                   (static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][1] * rw)) << 16);
+        packed.y = static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][2] * rw)) |
+                   (static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][3] * rw)) << 16);
+        *reinterpret_cast<uint2*>(o_row + 128 * wc + 16 * cb) = packed;
+      }
+    }
+  }
+}
+
+// tile_rows: 128.  MODE 0 needs N % 128 == 0, MODE 1 N % 256 == 0; K % 64 == 0.
+extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, const int32_t* sorted,
+                                    const int32_t* tile_expert, const int32_t* counters,
+                                    const float* route_weight, int assignments, int top_k, int N,
+                                    int K, int max_tiles, int mode, int tile_rows, hipStream_t stream) {
+  if (assignments <= 0) return SE_OK;
+  if (K <= 0 || K % 64 || N <= 0 || N % (mode == 0 ? 128 : 256) || tile_rows != 128) return SE_ERR_SHAPE;
+  if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
+  const int64_t items = static_cast<int64_t>(N / (mode == 0 ? 128 : 256)) * max_tiles;
+  const int grid = static_cast<int>((items + 7) / 8 * 8);
+  constexpr size_t shared = WIDE_STAGES * WIDE_CHUNKS * 1024 + 128 * sizeof(int32_t);
+  static bool allowed[2] = {false, false};   // more than 64 KB of shared memory has to be asked for, once
+#define SE_WIDE(MODE)                                                                              \
+  {                                                                                                \
+    if (!allowed[MODE]) {                                                                          \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_wide_kernel<MODE>),     \
+                              hipFuncAttributeMaxDynamicSharedMemorySize,                          \
+                              static_cast<int>(shared)) != hipSuccess)                             \
+        return SE_ERR_LAUNCH;                                                                      \
+      allowed[MODE] = true;                                                                        \
+    }                                                                                              \
+    grouped_gemm_wide_kernel<MODE><<<grid, 256, shared, stream>>>(                                 \
+        static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
+        tile_expert, counters, route_weight, assignments, top_k, N, K);                            \
+  }
+  if (mode == 0) SE_WIDE(0) else SE_WIDE(1)
+#undef SE_WIDE
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
 // Dense product of a few rows: out[rows, N] = x[rows, K] . w[N, K]^T (bfloat16, float accumulate).
 // A projection has only N / 16 blocks, far fewer than an expert layer: K is split over as many
 // wavefronts per block (up to 16) as it takes to put a few thousand of them in flight.

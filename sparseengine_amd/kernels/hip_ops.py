@@ -108,6 +108,8 @@ _SIGNATURES = {
         "se_skinny_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_tall": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "se_grouped_gemm_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "sampling": {
         "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -423,17 +425,21 @@ class HipKernels:
             # matrix-core path: tiles as tall as an expert's usual share of the step, blocks as wide
             # as still leaves enough workgroups for the whole chip
             share = assignments / min(experts, assignments)
+            asked_rows = tile_rows
             if tile_rows is None:
                 tile_rows = 16 if share <= 16 else 64
             if tall is None:
                 tall = share > 16          # many rows per expert: the weights go through LDS and are shared
             if tall:
-                tile_rows = 64
+                # hundreds of rows per expert: the 128 x 256 tile, which takes half as many bytes from
+                # the L2 per flop as the 64 x 128 one (it needs rows to fill its tiles)
+                wide_tile = ((share >= 192 and asked_rows is None) or asked_rows == 128) and inter % 128 == 0 and hidden % 256 == 0
+                tile_rows = 128 if wide_tile else 64
             max_tiles = self._grouped_tiles(ids, experts, ws, tile_rows)
             if max_tiles > 65535:
                 raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
             if tall:
-                gt = _fn.get("moe_mfma", "se_grouped_gemm_tall")
+                gt = _fn.get("moe_mfma", "se_grouped_gemm_wide" if tile_rows == 128 else "se_grouped_gemm_tall")
                 _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
                           _stream()), "moe gate-up (tall)")

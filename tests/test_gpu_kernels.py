@@ -357,7 +357,9 @@ def test_moe_align_groups_every_assignment_once(hip):
     (1, 64, 32, 8, 2), (45, 96, 48, 16, 4), (130, 200, 72, 5, 5), (9, 256, 128, 1, 1), (64, 384, 160, 32, 8),
     # sizes the matrix-core kernels take (hidden and width multiples of 128), tiles of 16, 32 and 64 rows
     (1, 256, 128, 8, 2), (3, 384, 256, 16, 4), (70, 256, 128, 4, 2), (200, 512, 384, 6, 3), (33, 3072, 1536, 16, 8),
-    (2048, 256, 128, 64, 8)])
+    (2048, 256, 128, 64, 8),
+    # hundreds of rows per expert: tiles of 128 rows x 256 weight rows
+    (2048, 256, 128, 8, 8), (1000, 512, 384, 6, 3), (777, 768, 256, 3, 1)])
 def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     x = randn(tokens, hidden, dtype=dtype, seed=11)
@@ -371,6 +373,11 @@ def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
     hip.moe_experts(x, w13, w2, ids, weights, out_h, ws)
     twin.moe_experts(x, w13, w2, ids, weights, out_t)
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
+    if dtype == torch.bfloat16 and hidden % 256 == 0 and inter % 128 == 0 and tokens <= 200:
+        # the wide tile on a step that would not choose it: mostly padding, same result
+        out_w = torch.empty_like(x)
+        hip.moe_experts(x, w13, w2, ids, weights, out_w, ws, tile_rows=128, tall=True)
+        torch.testing.assert_close(out_w, out_t, **tol(dtype))
     if experts == 1:   # one expert, k = 1: a plain SwiGLU feed-forward
         xf = x.float()
         ref = (torch.nn.functional.silu(xf @ w13[0, :inter].float().T) * (xf @ w13[0, inter:].float().T)) @ w2[0].float().T
