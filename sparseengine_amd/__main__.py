@@ -4,6 +4,8 @@
              every ``SamplingParams`` field too)
   random     write a model folder (config.json, model.safetensors) from a configuration and a seed
   replay     the trace replay tool (same as bin/trace_run)
+  bench      throughput of the whole engine for given prompt lengths and batch sizes (the reference's
+             benchmark/microbench.py options: --model_path --lengths --batch_sizes --output_len ...)
 
 The reference has no generation command line (its console scripts are the server's,
 pyproject.toml:66-69); option names here are the names of its ``Config`` and ``SamplingParams``.
@@ -78,6 +80,8 @@ def build_parser() -> argparse.ArgumentParser:
 
     rep = sub.add_parser("replay", help="trace replay (see bin/trace_run)", add_help=False)
     rep.add_argument("rest", nargs=argparse.REMAINDER)
+    ben = sub.add_parser("bench", help="engine throughput by prompt length and batch size", add_help=False)
+    ben.add_argument("rest", nargs=argparse.REMAINDER)
     return parser
 
 
@@ -88,6 +92,9 @@ def main(argv=None) -> int:
     if argv and argv[0] == "replay":       # its options are its own (they begin with dashes, which the
         from .engine.replay import main as replay_main      # sub-command parser would claim)
         return replay_main(argv[1:])
+    if argv and argv[0] == "bench":
+        from .engine.microbench import main as bench_main
+        return bench_main(argv[1:])
     parser = build_parser()
     args = parser.parse_args(argv)
     if args.command == "random":

@@ -43,11 +43,11 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def _check(status: int, what: str):
+def _check(status: int, what: str, takes: str = ""):
     if status == 0:
         return
     if status == -1:
-        raise KernelShapeError(f"{what}: the kernel refuses these sizes")
+        raise KernelShapeError(f"{what}: the kernel refuses these sizes" + (f" (it takes {takes})" if takes else ""))
     raise RuntimeError(f"{what}: kernel launch failed (status {status})")
 
 
@@ -319,14 +319,16 @@ class HipKernels:
                 _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
                 _ptr(work.block_units), work.num_block_units, _ptr(out), out.stride(0), _ptr(part_o),
                 _ptr(part_ml), heads, kv_heads, head_dim, page_size, float(scale), window,
-                work.tiles_per_block, _stream()), "paged_attention (blocks)")
+                work.tiles_per_block, _stream()), "paged_attention (blocks)",
+                "head_dim a multiple of 32 up to 128, page_size a multiple of 8")
         if work.num_units or work.num_tasks:  # one wavefront per tile and key range; then all merges
             _check(_fn.get("attention_mfma", "se_paged_attention_mfma")(
                 _ptr(q), q.stride(0), _ptr(cache), _ptr(meta.block_table), meta.block_table.stride(0),
                 _ptr(work.units) if work.num_units else None, work.num_units,
                 _ptr(work.tasks) if work.num_tasks else None, work.num_tasks, _ptr(out), out.stride(0),
                 _ptr(part_o), _ptr(part_ml), heads, kv_heads, head_dim, page_size, float(scale), window,
-                _stream()), "paged_attention (wavefronts)")
+                _stream()), "paged_attention (wavefronts)",
+                "head_dim a multiple of 32 up to 256, page_size a multiple of 8")
 
     # ------------------------------------------------------------------ mixture of experts
     ROUTER_KERNEL_TOKENS = 16   # up to this many tokens the router's product is one small kernel
@@ -433,7 +435,8 @@ class HipKernels:
             if tall:
                 # hundreds of rows per expert: the 128 x 256 tile, which takes half as many bytes from
                 # the L2 per flop as the 64 x 128 one (it needs rows to fill its tiles)
-                wide_tile = ((share >= 192 and asked_rows is None) or asked_rows == 128) and inter % 128 == 0 and hidden % 256 == 0
+                wide_tile = (((share >= 192 and asked_rows is None) or asked_rows == 128)
+                             and inter % 128 == 0 and hidden % 256 == 0)
                 tile_rows = 128 if wide_tile else 64
             max_tiles = self._grouped_tiles(ids, experts, ws, tile_rows)
             if max_tiles > 65535:
@@ -442,22 +445,21 @@ class HipKernels:
                 gt = _fn.get("moe_mfma", "se_grouped_gemm_wide" if tile_rows == 128 else "se_grouped_gemm_tall")
                 _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                          _stream()), "moe gate-up (tall)")
+                          _stream()), "moe gate-up (tall)", "hidden and intermediate sizes in multiples of 128")
                 _check(gt(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                          tile_rows, _stream()), "moe down (tall)")
-                _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
-                                                    _stream()), "moe_sum")
-                return
-            gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
-            if wide is None:
-                wide = 2 if max_tiles * (inter // 32) >= 2048 else 1
-            _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
-                      _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                      wide, _stream()), "moe gate-up (mfma)")
-            _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
-                      _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                      tile_rows, wide, _stream()), "moe down (mfma)")
+                          tile_rows, _stream()), "moe down (tall)", "hidden and intermediate sizes in multiples of 128")
+            else:
+                gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
+                if wide is None:
+                    wide = 2 if max_tiles * (inter // 32) >= 2048 else 1
+                _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                          _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
+                          wide, _stream()), "moe gate-up (mfma)", "hidden and intermediate sizes in multiples of 128")
+                _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                          _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
+                          tile_rows, wide, _stream()), "moe down (mfma)",
+                       "hidden and intermediate sizes in multiples of 128")
         else:
             max_tiles = self._grouped_tiles(ids, experts, ws, 16)
             if max_tiles > 65535:
@@ -489,7 +491,8 @@ class HipKernels:
                 and out.is_contiguous() and out.dtype == torch.bfloat16):
             _require(weight.shape[1] == k and out.shape == (rows, n), "linear shapes")
             _check(_fn.get("moe_mfma", "se_skinny_gemm_mfma")(_ptr(x), _ptr(weight), _ptr(out), rows, n, k,
-                                                              _stream()), "skinny gemm")
+                                                              _stream()), "skinny gemm",
+                   "K a multiple of 128, N a multiple of 16")
             return out
         return torch.mm(x, weight.t(), out=out)
 

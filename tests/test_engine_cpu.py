@@ -329,3 +329,28 @@ def test_step_times_and_throughput_lines(model):
     quiet = llm(folder)
     quiet.generate(prompts[:1], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True), use_tqdm=False)
     assert not quiet.step_times.seconds
+
+
+def test_engine_bench_counts_every_token_once(model, tmp_path, capsys):
+    """The bench sub-command: each case feeds batch x length prompt tokens; a request decodes
+    output_len - 1 tokens (its first completion token comes from the prompt's last step), of which
+    those that ride in a step beside prompt portions are counted with that step, as prefill."""
+    from sparseengine_amd.engine import microbench
+    folder = model[0]
+    out = tmp_path / "rows.jsonl"
+    rc = microbench.main(["--model_path", str(folder), "--lengths", "9,20", "--batch_sizes", "1,3", "--output_len", "5",
+                          "--hyper_params", json.dumps({"max_num_batched_tokens": 16}), "--output_jsonl", str(out)],
+                         llm_factory=lambda path, **kw: llm(path, **kw))
+    assert rc == 0
+    rows = [json.loads(line) for line in out.read_text().splitlines()]
+    assert [json.loads(line) for line in capsys.readouterr().out.splitlines()] == rows
+    assert [(r["length"], r["batch_size"]) for r in rows] == [(9, 1), (9, 3), (20, 1), (20, 3)]
+    for r in rows:
+        assert r["completed"] == r["batch_size"] and r["output_len"] == 5
+        assert r["prefill_tokens"] == r["batch_size"] * r["length"]
+        assert 0 < r["decode_tokens"] <= r["batch_size"] * 4
+        if r["batch_size"] == 1:
+            assert r["decode_tokens"] == 4 and r["decode_steps"] == 4
+        assert r["decode_tok_s"] > 0 and r["prefill_tok_s"] > 0 and r["total_s"] >= r["prefill_s"] + r["decode_s"] - 1e-3
+    with pytest.raises(SystemExit):
+        microbench.main(["--model_path", str(folder), "--lengths", "0"], llm_factory=lambda path, **kw: llm(path, **kw))

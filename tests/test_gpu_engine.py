@@ -137,6 +137,21 @@ def test_command_line_generates_what_the_entry_point_generates(tmp_path, capsys)
     assert [line["token_ids"] for line in lines] == [e["token_ids"] for e in expected]
 
 
+def test_command_line_bench_runs_every_case_on_the_gpu(tmp_path, capsys):
+    import json
+    from sparseengine_amd.__main__ import main
+    folder = make_folder(tmp_path, "A_loud")
+    capsys.readouterr()
+    assert main(["bench", "--model_path", folder, "--lengths", "40,130", "--batch_sizes", "1,4", "--output_len", "6",
+                 "--hyper_params", json.dumps({"kv_page_size": 16, "num_kvcache_slots": 2048,
+                                               "max_num_batched_tokens": 96})]) == 0
+    rows = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
+    assert [(r["length"], r["batch_size"]) for r in rows] == [(40, 1), (40, 4), (130, 1), (130, 4)]
+    for r in rows:
+        assert r["completed"] == r["batch_size"] and r["prefill_tokens"] == r["batch_size"] * r["length"]
+        assert r["decode_tok_s"] > 0 and r["prefill_tok_s"] > 0
+
+
 def test_weights_stored_in_32_bit_stay_so_under_bfloat16(tmp_path):
     folder = make_folder(tmp_path, "A_loud")
     path = os.path.join(folder, "model.safetensors")
