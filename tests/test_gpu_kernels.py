@@ -522,3 +522,81 @@ def test_skinny_linear(hip, rows, n, k):
     hip.linear(x, w, out)
     ref = x.float() @ w.float().T
     torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1.6e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_cache_pages_beyond_four_gigabytes(hip, twin, dtype):
+    """A layer's cache tensor larger than 2^32 bytes and 2^31 elements: the write and both
+    attention kernels must address its last pages with 64-bit offsets (a 32-bit offset would wrap
+    into the first pages, which stay zero here)."""
+    heads, kv_heads, head_dim, page, rotary = 48, 8, 128, 64, 64
+    pages = 17000
+    assert pages * 2 * kv_heads * page * head_dim > 2 ** 31
+    cache = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device="cuda")
+    lens, q_lens = [700, 130], [200, 1]
+    need = [-(-n // page) for n in lens]
+    ids = [list(range(16990, 16990 - need[0], -1)), list(range(16900, 16900 + need[1]))]
+    table = torch.full((2, max(need) + 1), -1, dtype=torch.int32)
+    for r, row in enumerate(ids):
+        table[r, :len(row)] = torch.tensor(row, dtype=torch.int32)
+    table = table.cuda()
+    T = sum(lens)
+    width = (heads + 2 * kv_heads) * head_dim
+    qkv = randn(T, width, dtype=dtype, seed=11)
+    positions = torch.cat([torch.arange(n) for n in lens]).to(torch.int32).cuda()
+    slots = torch.cat([torch.tensor([ids[r][p // page] * page + p % page for p in range(n)]) for r, n in enumerate(lens)])
+    used = sorted(set(sum(ids, [])))
+    remap = {p: i for i, p in enumerate(used)}
+    small_slots = torch.tensor([remap[int(s) // page] * page + int(s) % page for s in slots], dtype=torch.int32).cuda()
+    slots = slots.to(torch.int32).cuda()
+    cos_sin = rope_table(2048, rotary, 5e6)
+    qw = (1 + 0.1 * torch.randn(heads * head_dim)).to(dtype).cuda()
+    kw = (1 + 0.1 * torch.randn(kv_heads * head_dim)).to(dtype).cuda()
+    small = torch.zeros(len(used), 2, kv_heads, page, head_dim, dtype=dtype, device="cuda")
+    a, b = qkv.clone(), qkv.clone()
+    hip.qk_norm_rope_store(a, positions, cos_sin, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache, slots, page)
+    twin.qk_norm_rope_store(b, positions, cos_sin, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, small, small_slots, page)
+    torch.testing.assert_close(cache[torch.tensor(used).cuda()], small, **tol(dtype))
+    assert float(cache[:16384].abs().max()) == 0.0                 # nothing wrapped into the low pages
+    # attention over these pages: a prompt portion (blocks of tiles in bfloat16) and a decoded token
+    rows = torch.cat([torch.arange(lens[0] - q_lens[0], lens[0]), torch.tensor([T - 1])]).cuda()
+    q = a[rows, :heads * head_dim].reshape(-1, heads, head_dim).contiguous()
+    meta = make_meta(table, lens, q_lens)
+    out = torch.empty(q.shape[0], heads * head_dim, dtype=dtype, device="cuda")
+    hip.paged_attention(q, cache, meta, out, head_dim ** -0.5, 0)
+    for t in (0, 77, 199, 200):
+        row, pos = int(meta.token_row[t]), int(meta.positions[t])
+        ref = dense_attention(q[t], cache, table, row, pos, head_dim ** -0.5, 0, page)
+        torch.testing.assert_close(out[t].float(), ref, rtol=1.6e-2, atol=1.6e-2)
+    del cache
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("tokens", [3, 40, 600])
+def test_expert_weights_beyond_two_to_the_31_elements(hip, twin, tokens):
+    """MiniMax-M2's expert tables hold 2.4e9 and 1.2e9 elements; the last experts lie beyond a
+    32-bit element offset (and, in bytes, beyond 2^32).  Only those are chosen here, in the
+    streaming, the tall and the wide kernel."""
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    dtype, experts, hidden, inter, k = torch.bfloat16, 256, 3072, 1536, 2
+    assert (experts - 3) * 2 * inter * hidden > 2 ** 31
+    w13 = torch.zeros(experts, 2 * inter, hidden, dtype=dtype, device="cuda")
+    w2 = torch.zeros(experts, hidden, inter, dtype=dtype, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(5)
+    for e in (experts - 3, experts - 2, experts - 1):
+        w13[e] = (torch.randn(2 * inter, hidden, generator=g, device="cuda") * hidden ** -0.5).to(dtype)
+        w2[e] = (torch.randn(hidden, inter, generator=g, device="cuda") * inter ** -0.5).to(dtype)
+    x = randn(tokens, hidden, dtype=dtype, seed=21)
+    ids = torch.stack([experts - 3 + torch.randperm(3)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
+    weights = torch.rand(tokens, k).cuda()
+    weights = weights / weights.sum(-1, keepdim=True)
+    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+    out_h = torch.empty_like(x)
+    hip.moe_experts(x, w13, w2, ids, weights, out_h, ws)
+    # the twin on the three used experts alone
+    out_t = torch.empty_like(x)
+    twin.moe_experts(x, w13[experts - 3:].clone(), w2[experts - 3:].clone(), ids - (experts - 3), weights, out_t)
+    assert float(out_t.abs().max()) > 0.1
+    torch.testing.assert_close(out_h, out_t, **tol(dtype))
+    del w13, w2
+    torch.cuda.empty_cache()
