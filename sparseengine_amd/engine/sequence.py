@@ -53,9 +53,15 @@ class Sequence:
         return self.status is SequenceStatus.RUNNING and self.num_remaining_tokens == 1 and self.num_completion_tokens > 0
 
     def next_tokens(self, n: int) -> list[int]:
-        start = self.num_computed_tokens
-        known = self.prompt_token_ids + self.completion_token_ids
-        return known[start:start + n]
+        """The next ``n`` known tokens that are not in the cache yet (no copy of the whole history:
+        a decode step of a long request asks for one token)."""
+        start, stop = self.num_computed_tokens, self.num_computed_tokens + n
+        prompt = len(self.prompt_token_ids)
+        if stop <= prompt:
+            return self.prompt_token_ids[start:stop]
+        if start >= prompt:
+            return self.completion_token_ids[start - prompt:stop - prompt]
+        return self.prompt_token_ids[start:] + self.completion_token_ids[:stop - prompt]
 
     def append_token(self, token: int, logprob=None, top=None) -> None:
         self.completion_token_ids.append(int(token))
