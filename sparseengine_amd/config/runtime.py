@@ -1,7 +1,7 @@
 """The typed runtime configuration.  Its fields are exactly the keyword arguments of
 ``LLM(model, **kwargs)``; an unknown keyword is an error.  Names and meanings are the reference's
 where it has them (configs/runtime.py:51-105, configs/groups.py, configs/scheduling.py:15-186);
-``dtype``, ``kv_page_size`` and ``sampler_seed`` are this engine's own.
+``dtype``, ``kv_page_size``, ``sampler_seed`` and ``tiny_random_on_device`` are this engine's own.
 """
 from __future__ import annotations
 
@@ -37,6 +37,7 @@ class Config:
     tiny_random: bool = False                     # random weights for the folder's config.json
     tiny_random_config: str | None = None         # JSON (text or file) of config.json overrides
     tiny_random_seed: int = 0
+    tiny_random_on_device: bool | None = None     # draw with the device's generator; None: above 2^30 parameters
     eos: int = -1
     eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
     enable_profiler: bool = False

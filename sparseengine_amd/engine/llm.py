@@ -136,6 +136,7 @@ class LLM:
                       mlp_chunk_size=config.mlp_chunk_size, kernels=kernels)
         if config.tiny_random:
             self.runner = ModelRunner.from_random(config.raw_model_config, seed=config.tiny_random_seed,
+                                                  on_device=config.tiny_random_on_device,
                                                   num_kvcache_tokens=cache_tokens,
                                                   gpu_memory_utilization=config.gpu_memory_utilization, **common)
         else:

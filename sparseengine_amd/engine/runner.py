@@ -115,14 +115,19 @@ class ModelRunner:
 
     @classmethod
     def from_random(cls, raw_config: dict, seed: int = 0, options: dict | None = None,
-                    on_device: bool = False, **kwargs) -> "ModelRunner":
+                    on_device: bool | None = False, **kwargs) -> "ModelRunner":
+        """``on_device``: draw the weights with the device's generator (other values than the
+        host's, which a written folder holds); None decides by size: above 2^30 parameters the host
+        would take minutes."""
         arch = resolve_architecture(raw_config)
         cfg = arch.parse_config(raw_config)
 
         def factory(decls, dtype, device):
             dtypes = random_weights.random_parameter_dtypes(arch, cfg, decls, dtype)
             params = weight_loader.allocate_parameters(decls, dtypes, device)
-            random_weights.fill_random(params, arch, cfg, decls, seed, options, on_device=on_device)
+            large = sum(p.numel() for p in params.values()) > 2 ** 30
+            draw_there = (large if on_device is None else bool(on_device)) and torch.device(device).type == "cuda"
+            random_weights.fill_random(params, arch, cfg, decls, seed, options, on_device=draw_there)
             return params
         return cls(arch, cfg, factory, **kwargs)
 

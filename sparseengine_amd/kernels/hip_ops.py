@@ -424,14 +424,21 @@ class HipKernels:
         assignments = tokens * top_k
         code = _code(x.dtype)
         if x.dtype == torch.bfloat16 and hidden % 128 == 0 and inter % 128 == 0:
-            # matrix-core path: tiles as tall as an expert's usual share of the step, blocks as wide
-            # as still leaves enough workgroups for the whole chip
+            # matrix-core path.  The streaming kernel reads an expert's weights once per tile of 16
+            # rows, the tall one once per 64 rows and shares them among the tiles of an expert that
+            # run side by side.  Which experts a step uses is known on the device only: the choice
+            # goes by the average share and has to hold for even and for lumpy routing alike.
+            # Measured at MiniMax-M2 sizes (256 experts, top 8): with even routing the streaming
+            # kernel wins by 3 to 5 % up to 128 tokens and loses by 11 % at 512; when the tokens of
+            # a step agree on a few dozen experts (deep layers of a prompt) the tall kernel wins
+            # from 48 tokens on, by a factor of two at 512.  So: tall from three rows per expert on
+            # (a decode batch of 64 keeps the streaming kernel, a prompt portion of 96 does not).
             share = assignments / min(experts, assignments)
             asked_rows = tile_rows
-            if tile_rows is None:
-                tile_rows = 16 if share <= 16 else 64
             if tall is None:
-                tall = share > 16          # many rows per expert: the weights go through LDS and are shared
+                tall = share >= 3 if tile_rows is None else tile_rows >= 64
+            if tile_rows is None:
+                tile_rows = 64 if tall else 16
             if tall:
                 # hundreds of rows per expert: the 128 x 256 tile, which takes half as many bytes from
                 # the L2 per flop as the 64 x 128 one (it needs rows to fill its tiles)

@@ -12,6 +12,8 @@ from __future__ import annotations
 import hashlib
 import json
 import os
+import sys
+import time
 
 import torch
 from safetensors.torch import save_file
@@ -78,6 +80,13 @@ def fill_random(params: dict[str, torch.Tensor], arch: Architecture, cfg, decls,
     values than the host's; for sizes where host generation would take minutes)."""
     options = options or {}
     device = next(iter(params.values())).device if on_device else None
+    total = sum(p.numel() for p in params.values())
+    done, last = 0, time.monotonic()
     for src, value in checkpoint_tensors(arch, cfg, decls, seed, options, device=device):
         target = params[src.param]
         (target[src.index] if src.index else target).copy_(value)
+        done += value.numel()
+        if time.monotonic() - last > 20:      # a large model takes minutes on the host: say that it moves
+            last = time.monotonic()
+            print(f"[sparseengine_amd] random weights: {100 * done / total:.0f} % of {total / 1e9:.1f} G values drawn",
+                  file=sys.stderr, flush=True)
