@@ -64,6 +64,9 @@ class CacheManager:
         (an int for all groups or {group index: pages})."""
         if page_size <= 0 or max_rows <= 0 or max_model_len <= 0:
             raise ValueError("page_size, max_rows and max_model_len must be positive")
+        if page_size % 8:
+            raise ValueError(f"page_size must be a multiple of 8 (a page keeps its elements in groups of "
+                             f"eight, cache/layout.py), got {page_size}")
         self.page_size = int(page_size)
         self.max_rows = int(max_rows)
         self.max_model_len = int(max_model_len)

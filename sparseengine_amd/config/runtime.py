@@ -70,8 +70,8 @@ class Config:
         self.prefill_schedule_policy = resolve_prefill_schedule_policy(self.sparse_method, self.prefill_schedule_policy)
         if self.dtype not in ("bfloat16", "float32"):
             raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
-        if self.kv_page_size <= 0:
-            raise ValueError("kv_page_size must be positive")
+        if self.kv_page_size <= 0 or self.kv_page_size % 8:
+            raise ValueError(f"kv_page_size must be a positive multiple of 8, got {self.kv_page_size}")
         if not 0.0 < self.gpu_memory_utilization <= 1.0:
             raise ValueError("gpu_memory_utilization must be in (0, 1]")
         if self.max_num_seqs_in_batch <= 0:

@@ -1,11 +1,11 @@
 // Paged causal GQA attention, general form, for gfx950: one wavefront per (token, query head).
 //
 // Works for every head size that is a multiple of 8 up to 512, any number of heads and groups,
-// any page size, float and bfloat16 storage, with an optional sliding window.  It is the
+// page sizes in steps of 8, float and bfloat16 storage, with an optional sliding window.  It is the
 // float path of the engine and the fallback for shapes the matrix-core kernels refuse.
 //
-// Cache layer layout: [pages, 2, kv_heads, page_size * head_dim]; keys [page_size][head_dim],
-// values transposed [head_dim][page_size].
+// Cache layer layout: [pages, 2, kv_heads, page_size * head_dim]; inside a page a head's keys and
+// values lie in groups of eight elements (key_place / value_place in common.h); page_size % 8 == 0.
 //
 // For the query at position p of a request the keys n in [max(0, p - window + 1), p] are read
 // from the request's pages through its block-table row: this step's own keys were written
@@ -58,12 +58,11 @@ __global__ void paged_attention_generic_kernel(
     if (valid) {
       const int page = table[n / page_size];
       slot = page * page_size + (n % page_size);
-      const T* kr = cache + (static_cast<int64_t>(page) * 2) * plane + head_off +
-                    static_cast<int64_t>(n % page_size) * head_dim;
+      const T* kr = cache + (static_cast<int64_t>(page) * 2) * plane + head_off;
       float dot = 0.f;
       for (int d = 0; d < head_dim; d += VN) {
         Vec16<T> kv;
-        kv.v = *reinterpret_cast<const decltype(kv.v)*>(kr + d);
+        kv.v = *reinterpret_cast<const decltype(kv.v)*>(kr + key_place(page_size, n % page_size, d));
 #pragma unroll
         for (int i = 0; i < VN; ++i) dot += qs[d + i] * kv.get(i);
       }
@@ -81,12 +80,12 @@ __global__ void paged_attention_generic_kernel(
     for (int j = 0; j < count; ++j) {
       const float pj = __shfl(p_store, j, SE_WAVE);
       const int sj = __shfl(slot, j, SE_WAVE);
-      const T* vr = cache + (static_cast<int64_t>(sj / page_size) * 2 + 1) * plane + head_off +
-                    (sj % page_size);
+      const T* vr = cache + (static_cast<int64_t>(sj / page_size) * 2 + 1) * plane + head_off;
+      const int off_j = sj % page_size;
 #pragma unroll
       for (int i = 0; i < ATT_MAX_D_PER_LANE; ++i) {
         const int d = lane + i * SE_WAVE;
-        if (d < head_dim) acc[i] += pj * to_float(vr[static_cast<int64_t>(d) * page_size]);
+        if (d < head_dim) acc[i] += pj * to_float(vr[value_place(head_dim, off_j, d)]);
       }
     }
   }
@@ -107,7 +106,7 @@ extern "C" int se_paged_attention_generic(const void* q, int64_t q_stride, const
                                           int window, int dtype, hipStream_t stream) {
   if (tokens <= 0) return SE_OK;
   if (head_dim <= 0 || head_dim % 8 || head_dim > SE_WAVE * ATT_MAX_D_PER_LANE) return SE_ERR_SHAPE;
-  if (kv_heads <= 0 || heads % kv_heads || page_size <= 0) return SE_ERR_SHAPE;
+  if (kv_heads <= 0 || heads % kv_heads || page_size <= 0 || page_size % 8) return SE_ERR_SHAPE;
   if (q_stride % 8 || (dtype != SE_F32 && dtype != SE_BF16)) return SE_ERR_SHAPE;
   const int waves = 4;
   const int64_t work = static_cast<int64_t>(tokens) * heads;

@@ -10,8 +10,8 @@
 //   S^T = K Q^T   v_mfma_f32_16x16x32_bf16, A = 16 keys x 32 dims, B = 32 dims x 16 rows.  The key of
 //                 A-row m in block b is k0 + 8 * (m / 4) + m % 4 + 4 * b, so that a lane ends up with
 //                 the scores of eight consecutive keys for its row: exactly the B operand of
-//   O^T += V^T P^T  A = 16 value dims x 32 keys (values lie transposed in a page, eight consecutive
-//                 keys of one dim are one 16-byte load), B = 32 keys x 16 rows.
+//   O^T += V^T P^T  A = 16 value dims x 32 keys (eight consecutive keys of one dim lie side by side
+//                 in a page and are one 16-byte load), B = 32 keys x 16 rows.
 //
 // Softmax is online, in float, in base 2 (scale * log2(e) folded into the scores); probabilities
 // are rounded to bfloat16 for the value product, the running sum uses them unrounded.
@@ -19,8 +19,10 @@
 // writes its unnormalised O, running maximum and sum; the merge kernel combines a tile's splits
 // in the order of the key ranges.
 //
-// Cache layer: [pages, 2, kv_heads, page_size * head_dim]; keys [page_size][head_dim], values
-// [head_dim][page_size].  Requires head_dim % 32 == 0, head_dim <= 256, page_size % 8 == 0.
+// Cache layer: [pages, 2, kv_heads, page_size * head_dim]; inside a page a head's keys lie
+// [head_dim / 8][page_size][8] and its values [page_size / 8][head_dim][8] (common.h: key_place,
+// value_place): the sixteen lanes that hold neighbouring rows of an operand read one contiguous
+// stretch.  Requires head_dim % 32 == 0, head_dim <= 256, page_size % 8 == 0.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -133,17 +135,19 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     _Pragma("unroll") for (int b = 0; b < 2; ++b) {                                               \
       int key = (K0) + 8 * (n >> 2) + (n & 3) + 4 * b;                                            \
       if (key > last_key) key = last_key; /* reads stay inside the request's pages */            \
+      /* dims 32 ds + 8 g ... of the key: group 4 ds + g of the page's [head_dim / 8][page_size][8] */ \
       const bf16_t* k_row = cache + (static_cast<int64_t>(PK) * 2) * plane + kvh * head_span +    \
-                            static_cast<int64_t>(key % page_size) * D + g * 8;                    \
+                            (static_cast<int64_t>(g) * page_size + key % page_size) * 8;          \
       _Pragma("unroll") for (int ds = 0; ds < DSTEPS; ++ds)                                       \
-          KF[b][ds] = *reinterpret_cast<const uint4*>(k_row + ds * 32);                           \
+          KF[b][ds] = *reinterpret_cast<const uint4*>(k_row + static_cast<int64_t>(ds) * 32 * page_size); \
     }                                                                                             \
     int vkey = (K0) + 8 * g;                                                                      \
     if (vkey > last_key) vkey = last_key & ~7;                                                    \
+    /* eight keys of dim 16 db + n: the page's [page_size / 8][head_dim][8] */                     \
     const bf16_t* v_col = cache + (static_cast<int64_t>(PV) * 2 + 1) * plane + kvh * head_span +  \
-                          static_cast<int64_t>(n) * page_size + (vkey % page_size);               \
+                          static_cast<int64_t>(vkey % page_size) * D + n * 8;                     \
     _Pragma("unroll") for (int db = 0; db < DBLOCKS; ++db)                                        \
-        VF[db] = *reinterpret_cast<const uint4*>(v_col + static_cast<int64_t>(db) * 16 * page_size); \
+        VF[db] = *reinterpret_cast<const uint4*>(v_col + db * 128);                               \
   }
 
 #define ATT_COMPUTE(KF, VF, K0)                                                                   \
@@ -468,10 +472,12 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   const int clamp_page = clamp_key / page_size, clamp_off = clamp_key % page_size;
   int next_key = k_first + lane_key;                     // the lane's key of the next step to be issued
   int next_page = next_key / page_size, next_off = next_key % page_size;
-  const int64_t lane_base = loads_keys ? g * 8
-                                       : plane + static_cast<int64_t>((wave - 2) * DSTEPS * 16 + n) * page_size;
-  const int off_scale = loads_keys ? D : 1;
-  const int64_t load_stride = loads_keys ? 32 : static_cast<int64_t>(16) * page_size;
+  // keys lie [head_dim / 8][page_size][8], values [page_size / 8][head_dim][8]: sixteen lanes of a
+  // chunk (keys: runs of four; values: all sixteen) read one contiguous stretch
+  const int64_t lane_base = loads_keys ? static_cast<int64_t>(g) * page_size * 8
+                                       : plane + static_cast<int64_t>((wave - 2) * DSTEPS * 16 + n) * 8;
+  const int off_scale = loads_keys ? 8 : D;
+  const int64_t load_stride = loads_keys ? static_cast<int64_t>(32) * page_size : 128;
   auto issue = [&](int step) {
     const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS + wave * DSTEPS) * 1024u;
     const bool over = next_key > kmax;

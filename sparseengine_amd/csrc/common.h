@@ -213,6 +213,22 @@ __device__ __forceinline__ void stage_row(const T* src, float* dst, int n) {
   }
 }
 
+// Where an element of a kv head lies inside its page (page_size * head_dim elements), for keys
+// and for values.  Loads of 16 bytes per lane reach the caches fastest when neighbouring lanes
+// read neighbouring addresses; a matrix-core operand puts neighbouring *rows* into neighbouring
+// lanes, eight elements each.  So the cache keeps eight-element groups of neighbouring rows side
+// by side:
+//   keys:   [head_dim / 8][page_size][8]   lanes = keys, a lane's eight elements = eight dims
+//   values: [page_size / 8][head_dim][8]   lanes = dims, a lane's eight elements = eight keys
+// (measured on MI355X: 16 lanes x 16 bytes from 16 different rows arrive at 16 bytes a clock and
+// CU, from one contiguous stretch at three times that).  page_size % 8 == 0, head_dim % 8 == 0.
+__host__ __device__ __forceinline__ int64_t key_place(int page_size, int off, int d) {
+  return (static_cast<int64_t>(d >> 3) * page_size + off) * 8 + (d & 7);
+}
+__host__ __device__ __forceinline__ int64_t value_place(int head_dim, int off, int d) {
+  return (static_cast<int64_t>(off >> 3) * head_dim + d) * 8 + (off & 7);
+}
+
 // 16 bytes per lane from global memory straight into shared memory, no register in between: lane l's
 // bytes land at (wave-uniform) lds_addr + 16 l.  The compiler does not see the write: the caller
 // waits for it by hand (s_waitcnt vmcnt) before a barrier, and reads the data only after that barrier.

@@ -8,9 +8,10 @@
 // two-step tensor expression would; in float storage both roundings are the identity.
 //
 // Cache layer layout: [num_pages, 2 (k, v), kv_heads, page_size * head_dim]; inside a page a kv
-// head's keys lie [page_size][head_dim] and its values transposed, [head_dim][page_size] (the
-// matrix-core attention reads eight consecutive keys of one value dim as one operand).  A
-// token's slot is page * page_size + offset; negative slots are skipped.
+// head's keys and values lie in groups of eight elements (key_place / value_place in common.h),
+// so that what one matrix-core operand load of sixteen lanes takes is one contiguous stretch.  A
+// token's slot is page * page_size + offset; negative slots are skipped.  page_size % 8 == 0 and
+// head_dim % 8 == 0.
 #include "common.h"
 
 // the storage value whose widening to float is `v`, bit for bit (NaN payloads included)
@@ -68,12 +69,14 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
   const int half = rotary_dim / 2;
   const float* cs = cos_sin + static_cast<int64_t>(position) * rotary_dim;
   int64_t k_dst = -1, v_dst = -1;
+  int page_off = 0;
   if (slot >= 0) {
     const int64_t page = slot / page_size;
     const int64_t off = slot % page_size;
     const int64_t plane = static_cast<int64_t>(kv_heads) * page_size * head_dim;
-    k_dst = (page * 2) * plane + off * head_dim;   // + head * page_size * head_dim + d
-    v_dst = (page * 2 + 1) * plane + off;          // + head * page_size * head_dim + d * page_size
+    k_dst = (page * 2) * plane;       // + head * page_size * head_dim + key_place(page_size, off, d)
+    v_dst = (page * 2 + 1) * plane;   // + head * page_size * head_dim + value_place(head_dim, off, d)
+    page_off = static_cast<int>(off);
   }
 
   // one thread per element of q and k: normed value, then the rotation with its partner
@@ -101,7 +104,7 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
     src[c] = stored;
     if (!is_q && k_dst >= 0) {
       const int head = local / head_dim;
-      cache[k_dst + static_cast<int64_t>(head) * page_size * head_dim + d] = stored;
+      cache[k_dst + static_cast<int64_t>(head) * page_size * head_dim + key_place(page_size, page_off, d)] = stored;
     }
   }
   if (v_dst >= 0) {
@@ -109,7 +112,7 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
     const float* v = row + q_width + k_width;
     for (int c = threadIdx.x; c < k_width; c += blockDim.x) {
       const int head = c / head_dim, d = c % head_dim;
-      cache[v_dst + static_cast<int64_t>(head) * page_size * head_dim + static_cast<int64_t>(d) * page_size] =
+      cache[v_dst + static_cast<int64_t>(head) * page_size * head_dim + value_place(head_dim, page_off, d)] =
           narrow_exact<T>(v[c]);
     }
   }
@@ -220,12 +223,14 @@ qk_norm_rope_store_vec_kernel(T* qkv, int64_t row_stride, const int32_t* __restr
   }
 
   int64_t k_dst = -1, v_dst = -1;
+  int page_off = 0;
   if (slot >= 0) {
     const int64_t page = slot / page_size;
     const int64_t off = slot % page_size;
     const int64_t plane = static_cast<int64_t>(kv_heads) * page_size * head_dim;
-    k_dst = (page * 2) * plane + off * head_dim;   // + head * page_size * head_dim + d
-    v_dst = (page * 2 + 1) * plane + off;          // + head * page_size * head_dim + d * page_size
+    k_dst = (page * 2) * plane;       // + head * page_size * head_dim + key_place(page_size, off, d)
+    v_dst = (page * 2 + 1) * plane;   // + head * page_size * head_dim + value_place(head_dim, off, d)
+    page_off = static_cast<int>(off);
   }
 
 #pragma unroll
@@ -263,15 +268,16 @@ qk_norm_rope_store_vec_kernel(T* qkv, int64_t row_stride, const int32_t* __restr
     *reinterpret_cast<raw_t*>(src + c0) = outv.v;
     if (!is_q && k_dst >= 0) {
       const int head = local0 / head_dim;
-      *reinterpret_cast<raw_t*>(cache + k_dst + static_cast<int64_t>(head) * page_size * head_dim + d0) = outv.v;
+      *reinterpret_cast<raw_t*>(cache + k_dst + static_cast<int64_t>(head) * page_size * head_dim +
+                                key_place(page_size, page_off, d0)) = outv.v;
     }
   }
 #undef QK_FETCH_TABLES
-  if (v_dst >= 0) {   // values: a copy, bit for bit, to their transposed place
+  if (v_dst >= 0) {   // values: a copy, bit for bit, to their place among the page's groups of eight keys
     const T* v = reinterpret_cast<const T*>(row_bytes) + q_width + k_width;
     for (int c = threadIdx.x; c < k_width; c += threads) {
       const int head = c / head_dim, d = c % head_dim;
-      cache[v_dst + static_cast<int64_t>(head) * page_size * head_dim + static_cast<int64_t>(d) * page_size] = v[c];
+      cache[v_dst + static_cast<int64_t>(head) * page_size * head_dim + value_place(head_dim, page_off, d)] = v[c];
     }
   }
 }

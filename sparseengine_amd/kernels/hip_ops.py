@@ -227,7 +227,8 @@ class HipKernels:
                            head_dim, rotary_dim, cache=None, slots=None, page_size=0):
         """In place on ``qkv [T, (heads + 2 kv_heads) * head_dim]``: flat QK norm (if weights are
         given), partial rotation by ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half), and
-        the write of k and v to ``cache [pages, 2, kv_heads, page_size, head_dim]`` at ``slots``."""
+        the write of k and v to ``cache [pages, 2, kv_heads, page_size, head_dim]`` at ``slots`` (the
+        last two sizes are a page's geometry; the order of its elements is cache/layout.py's)."""
         tokens = qkv.shape[0]
         width = (heads + 2 * kv_heads) * head_dim
         _require(qkv.dim() == 2 and qkv.shape[1] == width and qkv.stride(1) == 1, "qkv shape")
@@ -246,6 +247,8 @@ class HipKernels:
             _require(slots.numel() == tokens, "slots length")
             _require(cache.dtype == qkv.dtype and cache.is_contiguous() and cache.dim() == 5
                      and tuple(cache.shape[1:]) == (2, kv_heads, page_size, head_dim), "cache layout")
+            if page_size % 8 or head_dim % 8:
+                raise KernelShapeError(f"cache pages take page_size {page_size} and head_dim {head_dim} in steps of 8")
         wd = _code(q_weight.dtype) if q_weight is not None else _code(qkv.dtype)
         _check(_fn.get("rope_kv", "se_qk_norm_rope_store")(
             _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(cos_sin) if rotary_dim else None,
@@ -276,8 +279,10 @@ class HipKernels:
         _require(meta.token_row.numel() == tokens and meta.positions.numel() == tokens, "meta length")
         if heads % kv_heads:
             raise KernelShapeError(f"attention: {heads} heads do not divide into {kv_heads} kv heads")
+        if page_size % 8:
+            raise KernelShapeError(f"attention: page_size {page_size} must be a multiple of 8")
         window = int(window or 0)
-        if (q.dtype == torch.bfloat16 and head_dim % 32 == 0 and head_dim <= 256 and page_size % 8 == 0
+        if (q.dtype == torch.bfloat16 and head_dim % 32 == 0 and head_dim <= 256
                 and getattr(meta, "item_q_len", None) is not None):      # the step's items are known
             return self._paged_attention_mfma(q, cache, meta, out, scale, window)
         if head_dim % 8 or head_dim > 512:

@@ -4,6 +4,7 @@ from types import SimpleNamespace
 import pytest
 import torch
 
+from sparseengine_amd.cache import layout
 from tests.twin_kernels import TwinKernels
 
 pytestmark = pytest.mark.gpu
@@ -116,7 +117,9 @@ def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary,
     for t in range(tokens):
         s = int(slots[t])
         if s >= 0:
-            assert torch.equal(cache_h[s // page, 0, :, s % page], kq[t])
+            at = (torch.tensor([s // page]).cuda(), torch.tensor([s % page]).cuda())
+            assert torch.equal(layout.read_keys(cache_h, *at)[0], kq[t])
+            assert torch.equal(layout.read_values(cache_h, *at)[0], a[t, (heads + kv_heads) * head_dim:].view(kv_heads, head_dim))
 
 
 def make_paged(dtype, kv_heads, head_dim, page, lens, seed=0, extra_pages=3):
@@ -152,8 +155,8 @@ def dense_attention(q, cache, table, row, pos, scale, window, page):
     first = max(0, pos - window + 1) if window else 0
     n = torch.arange(first, pos + 1, device="cuda")
     pages = table[row, n // page].long()
-    k = cache[pages, 0, :, n % page, :].float().transpose(0, 1)   # [Hkv, n, D]
-    v = cache[:, 1].view(cache.shape[0], cache.shape[2], cache.shape[4], page)[pages, :, :, n % page].float().transpose(0, 1)
+    k = layout.read_keys(cache, pages, n % page).float().transpose(0, 1)   # [Hkv, n, D]
+    v = layout.read_values(cache, pages, n % page).float().transpose(0, 1)
     H, D = q.shape
     group = H // k.shape[0]
     k = k.repeat_interleave(group, 0)
@@ -206,14 +209,14 @@ def test_paged_attention_finds_one_far_key(hip, dtype):
         # key of the target = 40 * direction of the first query head of each group
         for kvh in range(kv_heads):
             qh = q[0, kvh * (heads // kv_heads)].float()
-            c[pg, 0, kvh, off] = (qh / qh.norm() * 60).to(dtype)
+            layout.keys_view(c)[pg, kvh, off] = (qh / qh.norm() * 60).to(dtype).view(-1, 8)
         meta = make_meta(table, [n], [1])
         out = torch.empty(1, heads * head_dim, dtype=dtype, device="cuda")
         hip.paged_attention(q, c, meta, out, 1.0, 0)
         for kvh in range(kv_heads):
             head = kvh * (heads // kv_heads)
             got = out[0, head * head_dim:(head + 1) * head_dim].float()
-            value = c[pg, 1, kvh].view(head_dim, page)[:, off].float()     # values lie transposed in a page
+            value = layout.values_view(c)[pg, kvh, off // 8, off % 8].float()
             torch.testing.assert_close(got, value, rtol=2e-2, atol=2e-2)
 
 
@@ -491,8 +494,9 @@ def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, p
     # a page's slots past a request's end may hold anything an earlier owner left, even NaN
     last_page = int(table[0, (lens[0] - 1) // page])
     if lens[0] % page:
-        cache[last_page, 0, :, lens[0] % page:, :] = float("nan")
-        cache[last_page, 1].view(kv_heads, head_dim, page)[:, :, lens[0] % page:] = float("nan")
+        beyond = torch.arange(lens[0] % page, page, device="cuda")
+        layout.keys_view(cache)[last_page, :, beyond] = float("nan")
+        layout.values_view(cache)[last_page, :, beyond // 8, beyond % 8] = float("nan")
     meta = make_meta(table, lens, q_lens)
     T = sum(q_lens)
     q = randn(T, heads, head_dim, dtype=dtype, seed=3)

@@ -10,6 +10,8 @@ from __future__ import annotations
 import numpy as np
 import torch
 
+from sparseengine_amd.cache import layout
+
 
 def _r(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return x.to(dtype).float()
@@ -72,10 +74,8 @@ class TwinKernels:
             keep = slots >= 0
             s = slots[keep].long()
             page, off = s // page_size, s % page_size
-            # keys [page_size][head_dim]; values transposed inside the page, [head_dim][page_size]
-            cache[page, 0, :, off, :] = qkv[keep, qw:qw + kw].view(-1, kv_heads, head_dim)
-            values_t = cache[:, 1].view(cache.shape[0], kv_heads, head_dim, page_size)
-            values_t[page, :, :, off] = v[keep].reshape(-1, kv_heads, head_dim)
+            layout.write_keys(cache, page, off, qkv[keep, qw:qw + kw].view(-1, kv_heads, head_dim))
+            layout.write_values(cache, page, off, v[keep].reshape(-1, kv_heads, head_dim))
 
     def paged_attention(self, q, cache, meta, out, scale, window=0):
         T, H, D = q.shape
@@ -88,8 +88,8 @@ class TwinKernels:
             first = max(0, pos - window + 1) if window else 0
             n = torch.arange(first, pos + 1, device=q.device)
             pages = meta.block_table[row, (n // ps)].long()
-            keys = cache[pages, 0, :, n % ps, :].float()      # [n, Hkv, D]
-            vals = cache[:, 1].view(cache.shape[0], Hkv, D, ps)[pages, :, :, n % ps].float()
+            keys = layout.read_keys(cache, pages, n % ps).float()      # [n, Hkv, D]
+            vals = layout.read_values(cache, pages, n % ps).float()
             qt = q[t].float().view(Hkv, group, D)
             scores = torch.einsum("hgd,nhd->hgn", qt, keys) * scale
             m = scores.max(-1, keepdim=True).values
