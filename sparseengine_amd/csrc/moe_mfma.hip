@@ -53,6 +53,8 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   int tile, column_block;
   if (!xcd_work_item(N / BN, MODE == 2 ? max_tiles : counters[0], tile, column_block)) return;  // uniform
 
+  constexpr bool TILED = MODE != 2;
+  constexpr int KSCALE = TILED ? 16 : 1;       // a step of 32 along k is 512 elements further in a tiled table
   constexpr int P = NB * MB;                   // output blocks of 16 x 16 (gate/up pairs in MODE 0)
   constexpr int PARTS = MODE == 0 ? 2 : 1;
   // block p is finished by wave p % KW; the other waves leave their partial sums here
@@ -76,7 +78,10 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
   for (int nb = 0; nb < NBT; ++nb) {
     const int block_row = (MODE == 0 && nb >= NB) ? N + n0 + (nb - NB) * 16 : n0 + nb * 16;
-    a_ptr[nb] = we + static_cast<int64_t>(block_row + col) * K + kgroup * 8;
+    // expert tables lie in tiles of 16 rows x 32 k, each 1 KB in the order of the lanes that hold it
+    // as an operand (tile_expert_weights in kernels/hip_ops.py); dense tables lie in rows
+    a_ptr[nb] = TILED ? we + static_cast<int64_t>(block_row / 16) * (K / 32) * 512 + lane * 8
+                      : we + static_cast<int64_t>(block_row + col) * K + kgroup * 8;
   }
   const bf16_t* b_ptr[MB];
 #pragma unroll
@@ -103,7 +108,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     for (int k = k_begin; k < k_end; k += 32) {
       uint4 af[NBT], bf[MB];
 #pragma unroll
-      for (int nb = 0; nb < NBT; ++nb) af[nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + k);
+      for (int nb = 0; nb < NBT; ++nb) af[nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + static_cast<int64_t>(k) * KSCALE);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) bf[mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k);
 #pragma unroll
@@ -121,7 +126,8 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
     for (int u = 0; u < UU; ++u) {
 #pragma unroll
-      for (int nb = 0; nb < NBT; ++nb) af[u][nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + k + 32 * u);
+      for (int nb = 0; nb < NBT; ++nb)
+        af[u][nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + static_cast<int64_t>(k + 32 * u) * KSCALE);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) bf[u][mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k + 32 * u);
     }
@@ -263,7 +269,9 @@ grouped_gemm_tall_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   constexpr int WROWS = 128;
   int tile, column_block;
   if (!xcd_work_item(N / (MODE == 0 ? 64 : 128), counters[0], tile, column_block)) return;  // uniform
-  __shared__ __attribute__((aligned(16))) uint16_t ws[2][WROWS][TALL_LD];
+  // the weights of a step: 8 row blocks x 2 halves of k, each a tile of 64 16-byte vectors in the
+  // order of the lanes that hold it as an operand, as it lies in memory
+  __shared__ __attribute__((aligned(16))) uint4 ws[2][WROWS / 16 * 2][SE_WAVE];
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][BM][TALL_LD];
   __shared__ int32_t rows[BM];
 
@@ -285,15 +293,21 @@ grouped_gemm_tall_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   // loads stay in registers while they are in flight.
   static_assert(MB == 4, "the staging below moves exactly two activation chunks per thread");
   const int r0 = tid >> 3, kc = (tid & 7) * 8;
-  const bf16_t* wp0 = we + static_cast<int64_t>(n0 + r0) * K + kc;                  // tile rows r0, r0 + 32
-  const bf16_t* wp1 = wp0 + static_cast<int64_t>(32) * K;
-  const bf16_t* wp2 = MODE == 0 ? we + (static_cast<int64_t>(N) + n0 + r0) * K + kc  // tile rows 64 + r0, 96 + r0
-                                : wp0 + static_cast<int64_t>(64) * K;
-  const bf16_t* wp3 = wp2 + static_cast<int64_t>(32) * K;
+  // weights: wave w brings row blocks 2 w and 2 w + 1 of the step's 8 (MODE 0: blocks 0-3 are gate
+  // rows n0 + 16 b, blocks 4-7 the matching up rows; MODE 1: rows n0 + 16 b), both halves of k;
+  // a lane brings its own 16 bytes of each tile
+  auto block_row = [&](int rb) -> int64_t {
+    return MODE == 0 ? (rb < 4 ? 0 : static_cast<int64_t>(N)) + n0 + 16 * (rb & 3) : n0 + 16 * rb;
+  };
+  const int64_t tiles_per_row_block = K / 32;
+  const bf16_t* wp0 = we + (block_row(2 * wave) / 16) * tiles_per_row_block * 512 + lane * 8;   // + 512 for the second half
+  const bf16_t* wp2 = we + (block_row(2 * wave + 1) / 16) * tiles_per_row_block * 512 + lane * 8;
+  const bf16_t* wp1 = wp0 + 512;
+  const bf16_t* wp3 = wp2 + 512;
   const int a0 = rows[r0], a1 = rows[r0 + 32];
   const bf16_t* xp0 = in + (a0 < assignments ? static_cast<int64_t>(MODE == 0 ? a0 / top_k : a0) : 0) * K + kc;
   const bf16_t* xp1 = in + (a1 < assignments ? static_cast<int64_t>(MODE == 0 ? a1 / top_k : a1) : 0) * K + kc;
-  const int lds0 = r0 * TALL_LD + kc;               // element offset of the thread's first chunk
+  const int lds0 = r0 * TALL_LD + kc;               // element offset of the thread's first activation chunk
   constexpr int LDS32 = 32 * TALL_LD;
 
   floatx4 acc[2][MB];
@@ -302,29 +316,29 @@ grouped_gemm_tall_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // rows of the weight tile this wave multiplies: block 0 and block 1
-  const int a_row0 = MODE == 0 ? 16 * wave + col : 32 * wave + col;
-  const int a_row1 = MODE == 0 ? 64 + 16 * wave + col : 32 * wave + 16 + col;
+  // row blocks of the step's weights this wave multiplies
+  const int a_block0 = MODE == 0 ? wave : 2 * wave;
+  const int a_block1 = MODE == 0 ? 4 + wave : 2 * wave + 1;
 
 #define TALL_FETCH(S, K0)                                        \
-  S##w0 = *reinterpret_cast<const uint4*>(wp0 + (K0));           \
-  S##w1 = *reinterpret_cast<const uint4*>(wp1 + (K0));           \
-  S##w2 = *reinterpret_cast<const uint4*>(wp2 + (K0));           \
-  S##w3 = *reinterpret_cast<const uint4*>(wp3 + (K0));           \
+  S##w0 = *reinterpret_cast<const uint4*>(wp0 + static_cast<int64_t>(K0) * 16); /* 32 k = one tile = 512 elements */ \
+  S##w1 = *reinterpret_cast<const uint4*>(wp1 + static_cast<int64_t>(K0) * 16); \
+  S##w2 = *reinterpret_cast<const uint4*>(wp2 + static_cast<int64_t>(K0) * 16); \
+  S##w3 = *reinterpret_cast<const uint4*>(wp3 + static_cast<int64_t>(K0) * 16); \
   S##x0 = *reinterpret_cast<const uint4*>(xp0 + (K0));           \
   S##x1 = *reinterpret_cast<const uint4*>(xp1 + (K0));
 #define TALL_STASH(S, BUF)                                                          \
-  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0) = S##w0;                         \
-  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0 + LDS32) = S##w1;                 \
-  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0 + 2 * LDS32) = S##w2;             \
-  *reinterpret_cast<uint4*>(&ws[BUF][0][0] + lds0 + 3 * LDS32) = S##w3;             \
+  ws[BUF][4 * wave][lane] = S##w0;                                                  \
+  ws[BUF][4 * wave + 1][lane] = S##w1;                                              \
+  ws[BUF][4 * wave + 2][lane] = S##w2;                                              \
+  ws[BUF][4 * wave + 3][lane] = S##w3;                                              \
   *reinterpret_cast<uint4*>(&xs[BUF][0][0] + lds0) = S##x0;                         \
   *reinterpret_cast<uint4*>(&xs[BUF][0][0] + lds0 + LDS32) = S##x1;
 #define TALL_COMPUTE(BUF)                                                                              \
   _Pragma("unroll") for (int sub = 0; sub < TALL_BK / 32; ++sub) {                                     \
     const int ko = sub * 32 + kgroup * 8;                                                              \
-    const uint4 af0 = *reinterpret_cast<const uint4*>(&ws[BUF][a_row0][ko]);                           \
-    const uint4 af1 = *reinterpret_cast<const uint4*>(&ws[BUF][a_row1][ko]);                           \
+    const uint4 af0 = ws[BUF][2 * a_block0 + sub][lane];                                               \
+    const uint4 af1 = ws[BUF][2 * a_block1 + sub][lane];                                               \
     _Pragma("unroll") for (int mb = 0; mb < MB; ++mb) {                                                \
       const uint4 bf = *reinterpret_cast<const uint4*>(&xs[BUF][mb * 16 + col][ko]);                   \
       acc[0][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af0),            \
@@ -469,8 +483,8 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
   for (int j = 0; j < 6; ++j) {
     const int p = wave * 6 + j;
-    if (p < 16) {
-      src[j] = we + weight_row(p, col) * K + kgroup * 8;
+    if (p < 16) {     // a tile of 16 rows x 32 k is 512 elements in the order of the lanes; the next 32 k follow it
+      src[j] = we + (weight_row(p, 0) / 16) * (K / 32) * 512 + lane * 8;
     } else {
       const int a = rows[(p - 16) * 16 + col];
       const int64_t token = a < assignments ? static_cast<int64_t>(MODE == 0 ? a / top_k : a) : 0;  // padding reads row 0
@@ -483,8 +497,10 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     const int k0 = step * 64;
 #pragma unroll
     for (int j = 0; j < 6; ++j) {
-      load16_to_lds(src[j] + k0, dst + static_cast<uint32_t>(2 * j) * 1024u);
-      load16_to_lds(src[j] + k0 + 32, dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
+      const bool weights = wave * 6 + j < 16;      // the same for all lanes
+      const bf16_t* first = weights ? src[j] + static_cast<int64_t>(k0) * 16 : src[j] + k0;
+      load16_to_lds(first, dst + static_cast<uint32_t>(2 * j) * 1024u);
+      load16_to_lds(first + (weights ? 512 : 32), dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
     }
   };
 

@@ -64,6 +64,7 @@ class ModelRunner:
         decls = self.model.all_param_decls()
         self.params = params_factory(decls, self.dtype, self.device)
         self.model.bind_all(self.params)
+        self.model.finalize_all(kernels)
 
         self.max_model_len = int(max_model_len or self.spec.max_position)
         if self.max_model_len > self.spec.max_position:

@@ -52,6 +52,10 @@ class Part:
     def bind(self, params: dict[str, torch.Tensor]) -> None:
         self.params = params
 
+    def finalize(self, kernels) -> None:
+        """Once, after ``bind``: whatever the part does to its tensors for the kernels that will
+        run it (a layout, a table).  The checkpoint's values are not there to be read back afterwards."""
+
     def children(self) -> dict[str, "Part"]:
         return {}
 
@@ -66,6 +70,11 @@ class Part:
         self.bind({name: tensors[prefix + name] for name in self.param_decls()})
         for child_name, child in self.children().items():
             child.bind_all(tensors, f"{prefix}{child_name}.")
+
+    def finalize_all(self, kernels) -> None:
+        self.finalize(kernels)
+        for child in self.children().values():
+            child.finalize_all(kernels)
 
     def all_kernel_libraries(self) -> set[str]:
         libs = set(self.kernel_libraries)

@@ -29,6 +29,7 @@ class RoutedExperts(Part):
         self.hidden_size = int(hidden_size)
         self.chunk_tokens = int(chunk_tokens)
         self._workspace = None
+        self._tiled = False
 
     def param_decls(self):
         s = self.spec
@@ -38,6 +39,13 @@ class RoutedExperts(Part):
         if s.selection_bias:
             decls["router_bias"] = ParamDecl((s.num_experts,), "float32")
         return decls
+
+    def finalize(self, kernels) -> None:
+        """The matrix-core expert kernels read the tables in tiles laid out for their operand loads;
+        kernels that have such a layout put the tables into it here, once."""
+        arrange = getattr(kernels, "arrange_expert_weights", None)
+        if arrange is not None:
+            self._tiled = bool(arrange(self.params["w13"], self.params["w2"]))
 
     def _workspace_for(self, fb, tokens: int, dtype):
         s = self.spec
@@ -70,7 +78,10 @@ class RoutedExperts(Part):
         if fb.taps is not None:
             fb.taps.setdefault("router", []).append((ids.clone(), weights.clone()))
         if w13.dtype == x.dtype:
-            fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws)
+            if self._tiled:
+                fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws, tiled=True)
+            else:
+                fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws)
         else:   # expert weights kept in float32 under a bfloat16 engine
             x32 = x.float()
             out32 = torch.empty_like(x32)

@@ -604,3 +604,33 @@ def test_expert_weights_beyond_two_to_the_31_elements(hip, twin, tokens):
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
     del w13, w2
     torch.cuda.empty_cache()
+
+
+def test_expert_tables_arranged_in_place_are_the_tiled_copy(hip, twin):
+    """What the model does once (``arrange_expert_weights``, in place) and what a call with row-major
+    tables does on the fly (``tile_expert_weights``) are the same layout, element for element; a call
+    on arranged tables gives the twin's result."""
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    dtype, tokens, hidden, inter, experts, k = torch.bfloat16, 37, 256, 128, 19, 3
+    w13 = randn(experts, 2 * inter, hidden, dtype=dtype, scale=hidden ** -0.5, seed=1)
+    w2 = randn(experts, hidden, inter, dtype=dtype, scale=inter ** -0.5, seed=2)
+    # the layout, spelled out: element (n, k) of an expert lies at tile (n // 16, k // 32), place [(k % 32) // 8][n % 16][k % 8]
+    tiled = hip.tile_expert_weights(w13)
+    e, n, kk = 5, 37 + 16 * 3, 100
+    tile = (n // 16) * (hidden // 32) + kk // 32
+    place = tile * 512 + ((kk % 32) // 8 * 16 + n % 16) * 8 + kk % 8
+    assert tiled[e].reshape(-1)[place] == w13[e, n, kk]
+    a13, a2 = w13.clone(), w2.clone()
+    assert hip.arrange_expert_weights(a13, a2) is True
+    assert torch.equal(a13, tiled) and torch.equal(a2, hip.tile_expert_weights(w2))
+    assert hip.arrange_expert_weights(w13.float(), w2.float()) is False          # float tables stay in rows
+    odd = randn(2, 2 * 72, 200, dtype=dtype, seed=3)
+    assert hip.arrange_expert_weights(odd, randn(2, 200, 72, dtype=dtype, seed=4)) is False   # sizes of the general kernel
+    x = randn(tokens, hidden, dtype=dtype, seed=11)
+    ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
+    weights = torch.rand(tokens, k).cuda()
+    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+    out_h, out_t = torch.empty_like(x), torch.empty_like(x)
+    hip.moe_experts(x, a13, a2, ids, weights, out_h, ws, tiled=True)
+    twin.moe_experts(x, w13, w2, ids, weights, out_t)
+    torch.testing.assert_close(out_h, out_t, **tol(dtype))
