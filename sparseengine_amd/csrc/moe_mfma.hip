@@ -15,6 +15,12 @@
 //   MODE 2 (dense, few rows): out[t, n] = x[t] . w[n] for one weight matrix [N, K]; tile t holds rows
 //       16 * MB * t ...; the same streaming loop serves the skinny projections of decode steps.
 //
+// Expert tables (MODE 0 and 1, in all three kernels of this file) lie in tiles: tile
+// (n / 16, k / 32) of an expert is 512 consecutive elements in the order [(k % 32) / 8][n % 16][k % 8],
+// which is the order of the lanes that hold the tile as an A operand, so a wavefront's load of a
+// tile is one contiguous kilobyte (kernels/hip_ops.py: tile_expert_weights puts a table into this
+// order).  Dense tables (MODE 2) lie in rows: the BLAS library reads them too.
+//
 // Every output element is one dot product in a fixed order of K, so a row's result does not
 // depend on its place in the tile or on what else is in the batch.
 // Requires K % 128 == 0 and N % BN == 0; other sizes take the general kernel in moe.hip.
@@ -250,12 +256,13 @@ static void launch(const void* in, const void* w, void* out, const int32_t* sort
 // tile are used by many rows, so they are staged through LDS and shared by the block's four
 // waves.  A block computes BM = 16 * MB rows x 128 weight rows (MODE 0: 64 gate + 64 up rows ->
 // 64 outputs; MODE 1: 128 outputs) in steps of 64 along K, double-buffered: the loads of the next
-// step are in flight while the matrix cores work on the current one.  Wave w owns 32 of the
+// step are in flight while the matrix cores work on the current one.  The weights stay in the
+// order of their tiles in LDS, the activation rows lie in padded rows.  Wave w owns 32 of the
 // weight rows (MODE 0: gate rows 16 w .. and the matching up rows) and all rows of the tile.
 // Each output is one dot product in the order of K, as in the streaming kernel.
 // ---------------------------------------------------------------------------------------- //
 #define TALL_BK 64
-#define TALL_LD 72          // row stride in LDS (elements): 64 + 8 keeps 16-byte reads off the same banks
+#define TALL_LD 72          // stride of an activation row in LDS (elements): 64 + 8 keeps 16-byte reads off the same banks
 
 template <int MODE, int MB>
 __global__ void __launch_bounds__(256)
