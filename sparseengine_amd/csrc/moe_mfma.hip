@@ -435,21 +435,27 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 
 // ---------------------------------------------------------------------------------------- //
 // Wide tiles (an expert has hundreds of rows: steps of many thousand tokens).  The 64 x 128 tile
-// above does 43 flop for each byte it takes from the L2, and that is where it stops (about 455
-// TFLOP/s measured).  Here a block computes 128 rows x 256 weight rows (87 flop per byte): four
-// wavefronts, each 64 rows x 128 weight rows (MODE 0: 64 gate rows and the matching 64 up rows, so
-// that the SwiGLU product stays inside a lane).  A step of 64 along K is 48 chunks of 1 KB that go
-// from memory straight into shared memory in operand order (lane l's 16 bytes of a chunk are what
-// lane l feeds the matrix core), three stages deep; twelve chunks per wavefront and step.
-//   MODE 0: out[a, n0 + 64 wc + 16 cb + ...] from gate rows n0 + 64 wc ..., up rows N + n0 + 64 wc ...
-//   MODE 1: out[a, n0 + 128 wc + 16 cb + ...] * route_weight[a]
+// above does 43 flop for each byte it brings in, and that is where it stops (about 455 TFLOP/s
+// measured).  Here a block computes 128 rows x 256 weight rows (87 flop per byte) with eight
+// wavefronts, two per SIMD, each 64 rows x 64 weight rows (MODE 0: 32 gate rows and the matching
+// 32 up rows, so that the SwiGLU product stays inside a lane); four wavefronts of 64 x 128 read a
+// quarter less from LDS per flop but, one to a SIMD, cannot issue LDS reads fast enough (measured:
+// 120 bytes a clock and CU with four wavefronts, 220 with eight).  A step of 64 along K is 48
+// chunks of 1 KB that go from memory straight into shared memory in operand order (lane l's 16
+// bytes of a chunk are what lane l feeds the matrix core), three stages deep; six chunks per
+// wavefront and step.  Weight chunks are tiles of the table as it lies in memory.
+//   MODE 0: out[a, n0 + 32 wc + 16 cb + ...] from gate rows n0 + 32 wc ..., up rows N + n0 + 32 wc ...
+//   MODE 1: out[a, n0 + 64 wc + 16 cb + ...] * route_weight[a]
 // Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1); tiles of 128 sorted rows.
 // ---------------------------------------------------------------------------------------- //
 #define WIDE_STAGES 3
+#ifndef WIDE_WAVES
+#define WIDE_WAVES 8     // wavefronts per block
+#endif
 #define WIDE_CHUNKS 48      // per stage: 32 of weights (16 row blocks x 2 halves of the step), 16 of activations
 
-template <int MODE>
-__global__ void __launch_bounds__(256)
+template <int MODE, int WAVES>   // WAVES: 4 (each 64 rows x 128 weight rows) or 8 (each 64 x 64)
+__global__ void __launch_bounds__(64 * WAVES)
 grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
                          bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
                          const int32_t* __restrict__ tile_expert,
@@ -458,6 +464,9 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
                          int K) {
   constexpr int BM = 128;
   constexpr int OUT_COLS = MODE == 0 ? 128 : 256;
+  constexpr int WCOLS = WAVES / 2;               // wave columns: the tile's 256 weight rows in 2 or 4 parts
+  constexpr int CB = 16 / WCOLS;                 // weight row blocks of a wave: 8 or 4
+  constexpr int PAIRS = 24 / WAVES;              // row block pairs a wave brings per step: 6 or 3
   int tile, column_block;
   if (!xcd_work_item(N / OUT_COLS, counters[0], tile, column_block)) return;  // uniform
   extern __shared__ __align__(16) uint4 wide_shared[];     // WIDE_STAGES x WIDE_CHUNKS x 64 vectors, then the rows
@@ -468,7 +477,7 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   const int lane = tid & (SE_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / SE_WAVE);
   const int col = lane & 15, kgroup = lane >> 4;
-  const int wr = wave >> 1, wc = wave & 1;       // the wave's 64 rows and 128 weight rows of the tile
+  const int wr = wave / WCOLS, wc = wave % WCOLS;   // the wave's 64 rows and its part of the weight rows
   const int expert = tile_expert[tile];
   const int n0 = column_block * OUT_COLS;
   if (tid < BM) rows[tid] = sorted[tile * BM + tid];
@@ -477,21 +486,23 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   const int64_t w_rows = MODE == 0 ? 2 * static_cast<int64_t>(N) : N;
   const bf16_t* we = w + static_cast<int64_t>(expert) * w_rows * K;
 
-  // Row block rb (16 rows) of the tile's 256 weight rows: blocks 8 wc' ... 8 wc' + 7 belong to the
-  // wave column wc'; in MODE 0 its first four are gate rows, its last four the matching up rows.
-  auto weight_row = [&](int rb, int r) -> int64_t {
-    const int wcol = rb >> 3, cb = rb & 7;
-    if (MODE == 0) return (cb < 4 ? 0 : static_cast<int64_t>(N)) + n0 + 64 * wcol + 16 * (cb & 3) + r;
-    return n0 + 128 * wcol + 16 * cb + r;
+  // Row block rb (16 rows) of the tile's 256 weight rows: blocks CB wc' ... CB wc' + CB - 1 belong to
+  // the wave column wc'; in MODE 0 the first half of them are gate rows, the second half the matching
+  // up rows.
+  auto weight_row = [&](int rb) -> int64_t {
+    const int wcol = rb / CB, cb = rb % CB;
+    if (MODE == 0)
+      return (cb < CB / 2 ? 0 : static_cast<int64_t>(N)) + n0 + (8 * CB) * wcol + 16 * (cb % (CB / 2));
+    return n0 + (16 * CB) * wcol + 16 * cb;
   };
-  // The wave brings six "row block pairs" of a step: pair p < 16 is weight row block p, pair p >= 16
+  // The wave brings PAIRS "row block pairs" of a step: pair p < 16 is weight row block p, pair p >= 16
   // is activation row block p - 16; both halves of the step (chunks 2 p and 2 p + 1).
-  const bf16_t* src[6];
+  const bf16_t* src[PAIRS];
 #pragma unroll
-  for (int j = 0; j < 6; ++j) {
-    const int p = wave * 6 + j;
+  for (int j = 0; j < PAIRS; ++j) {
+    const int p = wave * PAIRS + j;
     if (p < 16) {     // a tile of 16 rows x 32 k is 512 elements in the order of the lanes; the next 32 k follow it
-      src[j] = we + (weight_row(p, 0) / 16) * (K / 32) * 512 + lane * 8;
+      src[j] = we + (weight_row(p) / 16) * (K / 32) * 512 + lane * 8;
     } else {
       const int a = rows[(p - 16) * 16 + col];
       const int64_t token = a < assignments ? static_cast<int64_t>(MODE == 0 ? a / top_k : a) : 0;  // padding reads row 0
@@ -500,20 +511,21 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   }
   const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wide_shared));
   auto issue = [&](int step) {
-    const uint32_t dst = stage_base + static_cast<uint32_t>((step % WIDE_STAGES) * WIDE_CHUNKS + wave * 12) * 1024u;
+    const uint32_t dst =
+        stage_base + static_cast<uint32_t>((step % WIDE_STAGES) * WIDE_CHUNKS + wave * 2 * PAIRS) * 1024u;
     const int k0 = step * 64;
 #pragma unroll
-    for (int j = 0; j < 6; ++j) {
-      const bool weights = wave * 6 + j < 16;      // the same for all lanes
+    for (int j = 0; j < PAIRS; ++j) {
+      const bool weights = wave * PAIRS + j < 16;      // the same for all lanes
       const bf16_t* first = weights ? src[j] + static_cast<int64_t>(k0) * 16 : src[j] + k0;
       load16_to_lds(first, dst + static_cast<uint32_t>(2 * j) * 1024u);
       load16_to_lds(first + (weights ? 512 : 32), dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
     }
   };
 
-  floatx4 acc[8][4];      // [weight row block of the wave][row block of the wave]
+  floatx4 acc[CB][4];      // [weight row block of the wave][row block of the wave]
 #pragma unroll
-  for (int cb = 0; cb < 8; ++cb)
+  for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) acc[cb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
@@ -524,7 +536,7 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   for (int step = 0; step < steps; ++step) {
     // this step's data: all but the loads of the steps after it must have come back
     if (step + WIDE_STAGES - 2 < steps) {
-      __builtin_amdgcn_s_waitcnt(0x0F70 | ((WIDE_STAGES - 2) * 12));    // vmcnt((stages - 2) * 12)
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((WIDE_STAGES - 2) * 2 * PAIRS));    // vmcnt((stages - 2) * loads per step)
     } else {
       __builtin_amdgcn_s_waitcnt(0x0F70);                               // vmcnt(0)
     }
@@ -538,8 +550,8 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) bfrag[mb] = chunk[2 * (16 + 4 * wr + mb) + sub][lane];
 #pragma unroll
-      for (int cb = 0; cb < 8; ++cb) {
-        const uint4 afrag = chunk[2 * (8 * wc + cb) + sub][lane];
+      for (int cb = 0; cb < CB; ++cb) {
+        const uint4 afrag = chunk[2 * (CB * wc + cb) + sub][lane];
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb)
           acc[cb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, afrag),
@@ -558,30 +570,30 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     bf16_t* o_row = out + static_cast<int64_t>(a) * N + n0 + 4 * kgroup;
     if (MODE == 0) {
 #pragma unroll
-      for (int cb = 0; cb < 4; ++cb) {
+      for (int cb = 0; cb < CB / 2; ++cb) {
         uint16_t y[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float gate = round_to<bf16_t>(acc[cb][mb][i]);
-          const float up = round_to<bf16_t>(acc[cb + 4][mb][i]);
+          const float up = round_to<bf16_t>(acc[cb + CB / 2][mb][i]);
           const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
           y[i] = float_to_bf16_bits(act * up);
         }
         uint2 packed;
         packed.x = static_cast<uint32_t>(y[0]) | (static_cast<uint32_t>(y[1]) << 16);
         packed.y = static_cast<uint32_t>(y[2]) | (static_cast<uint32_t>(y[3]) << 16);
-        *reinterpret_cast<uint2*>(o_row + 64 * wc + 16 * cb) = packed;
+        *reinterpret_cast<uint2*>(o_row + (8 * CB) * wc + 16 * cb) = packed;
       }
     } else {
       const float rw = route_weight[a];
 #pragma unroll
-      for (int cb = 0; cb < 8; ++cb) {
+      for (int cb = 0; cb < CB; ++cb) {
         uint2 packed;
         packed.x = static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][0] * rw)) |
                    (static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][1] * rw)) << 16);
         packed.y = static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][2] * rw)) |
                    (static_cast<uint32_t>(float_to_bf16_bits(acc[cb][mb][3] * rw)) << 16);
-        *reinterpret_cast<uint2*>(o_row + 128 * wc + 16 * cb) = packed;
+        *reinterpret_cast<uint2*>(o_row + (16 * CB) * wc + 16 * cb) = packed;
       }
     }
   }
@@ -602,13 +614,13 @@ extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, co
 #define SE_WIDE(MODE)                                                                              \
   {                                                                                                \
     if (!allowed[MODE]) {                                                                          \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_wide_kernel<MODE>),     \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_wide_kernel<MODE, WIDE_WAVES>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize,                          \
                               static_cast<int>(shared)) != hipSuccess)                             \
         return SE_ERR_LAUNCH;                                                                      \
       allowed[MODE] = true;                                                                        \
     }                                                                                              \
-    grouped_gemm_wide_kernel<MODE><<<grid, 256, shared, stream>>>(                                 \
+    grouped_gemm_wide_kernel<MODE, WIDE_WAVES><<<grid, 64 * WIDE_WAVES, shared, stream>>>(         \
         static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
         tile_expert, counters, route_weight, assignments, top_k, N, K);                            \
   }
