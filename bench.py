@@ -175,7 +175,7 @@ def main() -> int:
 
     achieved = decode_bytes(args.batch, distinct, context) / step_s
     line = {
-        "metric": "decode tok/s @ batch 8 (MiniMax-M2 sizes, 16 layers, 1 GPU)", "value": round(args.batch / step_s, 1),
+        "metric": f"decode tok/s @ batch {args.batch} (MiniMax-M2 sizes, {L} layers, 1 GPU)", "value": round(args.batch / step_s, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random token ids, random weights",
