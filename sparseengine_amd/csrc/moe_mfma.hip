@@ -434,16 +434,19 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 }
 
 // ---------------------------------------------------------------------------------------- //
-// Wide tiles (an expert has hundreds of rows: steps of many thousand tokens).  The 64 x 128 tile
-// above does 43 flop for each byte it brings in, and that is where it stops (about 455 TFLOP/s
-// measured).  Here a block computes 128 rows x 256 weight rows (87 flop per byte) with eight
-// wavefronts, two per SIMD, each 64 rows x 64 weight rows (MODE 0: 32 gate rows and the matching
-// 32 up rows, so that the SwiGLU product stays inside a lane); four wavefronts of 64 x 128 read a
-// quarter less from LDS per flop but, one to a SIMD, cannot issue LDS reads fast enough (measured:
-// 120 bytes a clock and CU with four wavefronts, 220 with eight).  A step of 64 along K is 48
-// chunks of 1 KB that go from memory straight into shared memory in operand order (lane l's 16
-// bytes of a chunk are what lane l feeds the matrix core), three stages deep; six chunks per
-// wavefront and step.  Weight chunks are tiles of the table as it lies in memory.
+// Wide tiles (an expert has sixteen rows or more: prompt portions from 512 tokens on).  The 64 x 128
+// kernel above brings its operands through registers, and registers are fed at about 16 bytes a
+// clock and CU whatever the addresses; loads that go straight into LDS are fed at three times that
+// when the lanes of a load read one contiguous stretch, which the tiled expert tables provide.
+// Here a block computes 128 rows x 256 weight rows (87 flop per byte) with eight wavefronts, each
+// 64 rows x 64 weight rows (MODE 0: 32 gate rows and the matching 32 up rows, so that the SwiGLU
+// product stays inside a lane).  A step of 32 along K is 24 chunks of 1 KB that go from memory
+// straight into shared memory in operand order (lane l's 16 bytes of a chunk are what lane l feeds
+// the matrix core), three stages deep, three chunks per wavefront and step; 72 KB of LDS, so that
+// two blocks share a CU and one computes while the other waits at its barrier.  Measured at 16384
+// tokens (gate-up + down): four wavefronts of 64 x 128 and steps of 64, one block per CU: 6.2 ms;
+// eight wavefronts: 5.9 (LDS reads issue at 220 instead of 120 bytes a clock); steps of 32 and two
+// blocks per CU: 5.1.
 //   MODE 0: out[a, n0 + 32 wc + 16 cb + ...] from gate rows n0 + 32 wc ..., up rows N + n0 + 32 wc ...
 //   MODE 1: out[a, n0 + 64 wc + 16 cb + ...] * route_weight[a]
 // Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1); tiles of 128 sorted rows.
@@ -452,10 +455,12 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 #ifndef WIDE_WAVES
 #define WIDE_WAVES 8     // wavefronts per block
 #endif
-#define WIDE_CHUNKS 48      // per stage: 32 of weights (16 row blocks x 2 halves of the step), 16 of activations
+#ifndef WIDE_KSTEP
+#define WIDE_KSTEP 32    // k per stage
+#endif
 
-template <int MODE, int WAVES>   // WAVES: 4 (each 64 rows x 128 weight rows) or 8 (each 64 x 64)
-__global__ void __launch_bounds__(64 * WAVES)
+template <int MODE, int WAVES, int KSTEP>   // WAVES: 4 (each 64 rows x 128 weight rows) or 8 (each 64 x 64); KSTEP: 32 or 64
+__global__ void __launch_bounds__(64 * WAVES, KSTEP == 32 ? 2 : 1)
 grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
                          bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
                          const int32_t* __restrict__ tile_expert,
@@ -466,12 +471,14 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   constexpr int OUT_COLS = MODE == 0 ? 128 : 256;
   constexpr int WCOLS = WAVES / 2;               // wave columns: the tile's 256 weight rows in 2 or 4 parts
   constexpr int CB = 16 / WCOLS;                 // weight row blocks of a wave: 8 or 4
-  constexpr int PAIRS = 24 / WAVES;              // row block pairs a wave brings per step: 6 or 3
+  constexpr int PAIRS = 24 / WAVES;              // row blocks a wave brings per step: 6 or 3
+  constexpr int HALVES = KSTEP / 32;             // chunks of 32 k per row block and step
+  constexpr int CHUNKS = 24 * HALVES;            // per stage
   int tile, column_block;
   if (!xcd_work_item(N / OUT_COLS, counters[0], tile, column_block)) return;  // uniform
-  extern __shared__ __align__(16) uint4 wide_shared[];     // WIDE_STAGES x WIDE_CHUNKS x 64 vectors, then the rows
-  int32_t* rows = reinterpret_cast<int32_t*>(wide_shared + WIDE_STAGES * WIDE_CHUNKS * 64);
-  static_assert(WIDE_STAGES * WIDE_CHUNKS * 1024 <= 160 * 1024 - 1024, "stages must fit shared memory");
+  extern __shared__ __align__(16) uint4 wide_shared[];     // WIDE_STAGES x CHUNKS x 64 vectors, then the rows
+  int32_t* rows = reinterpret_cast<int32_t*>(wide_shared + WIDE_STAGES * CHUNKS * 64);
+  static_assert(WIDE_STAGES * CHUNKS * 1024 <= 160 * 1024 - 1024, "stages must fit shared memory");
 
   const int tid = threadIdx.x;
   const int lane = tid & (SE_WAVE - 1);
@@ -512,14 +519,14 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wide_shared));
   auto issue = [&](int step) {
     const uint32_t dst =
-        stage_base + static_cast<uint32_t>((step % WIDE_STAGES) * WIDE_CHUNKS + wave * 2 * PAIRS) * 1024u;
-    const int k0 = step * 64;
+        stage_base + static_cast<uint32_t>((step % WIDE_STAGES) * CHUNKS + wave * HALVES * PAIRS) * 1024u;
+    const int k0 = step * KSTEP;
 #pragma unroll
     for (int j = 0; j < PAIRS; ++j) {
       const bool weights = wave * PAIRS + j < 16;      // the same for all lanes
       const bf16_t* first = weights ? src[j] + static_cast<int64_t>(k0) * 16 : src[j] + k0;
-      load16_to_lds(first, dst + static_cast<uint32_t>(2 * j) * 1024u);
-      load16_to_lds(first + (weights ? 512 : 32), dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
+      load16_to_lds(first, dst + static_cast<uint32_t>(HALVES * j) * 1024u);
+      if (HALVES == 2) load16_to_lds(first + (weights ? 512 : 32), dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
     }
   };
 
@@ -529,29 +536,29 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) acc[cb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const int steps = K / 64;
+  const int steps = K / KSTEP;
 #pragma unroll
   for (int j = 0; j < WIDE_STAGES - 1; ++j)
     if (j < steps) issue(j);
   for (int step = 0; step < steps; ++step) {
     // this step's data: all but the loads of the steps after it must have come back
     if (step + WIDE_STAGES - 2 < steps) {
-      __builtin_amdgcn_s_waitcnt(0x0F70 | ((WIDE_STAGES - 2) * 2 * PAIRS));    // vmcnt((stages - 2) * loads per step)
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((WIDE_STAGES - 2) * HALVES * PAIRS));    // vmcnt((stages - 2) * loads per step)
     } else {
       __builtin_amdgcn_s_waitcnt(0x0F70);                               // vmcnt(0)
     }
     __builtin_amdgcn_s_barrier();   // everyone's part of the step is in; everyone has left step - 1
     asm volatile("" ::: "memory");
     if (step + WIDE_STAGES - 1 < steps) issue(step + WIDE_STAGES - 1);   // into the buffer step - 1 used
-    const uint4(*chunk)[64] = reinterpret_cast<const uint4(*)[64]>(wide_shared) + (step % WIDE_STAGES) * WIDE_CHUNKS;
+    const uint4(*chunk)[64] = reinterpret_cast<const uint4(*)[64]>(wide_shared) + (step % WIDE_STAGES) * CHUNKS;
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
+    for (int sub = 0; sub < HALVES; ++sub) {
       uint4 bfrag[4];
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb) bfrag[mb] = chunk[2 * (16 + 4 * wr + mb) + sub][lane];
+      for (int mb = 0; mb < 4; ++mb) bfrag[mb] = chunk[HALVES * (16 + 4 * wr + mb) + sub][lane];
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) {
-        const uint4 afrag = chunk[2 * (CB * wc + cb) + sub][lane];
+        const uint4 afrag = chunk[HALVES * (CB * wc + cb) + sub][lane];
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb)
           acc[cb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, afrag),
@@ -609,18 +616,18 @@ extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, co
   if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
   const int64_t items = static_cast<int64_t>(N / (mode == 0 ? 128 : 256)) * max_tiles;
   const int grid = static_cast<int>((items + 7) / 8 * 8);
-  constexpr size_t shared = WIDE_STAGES * WIDE_CHUNKS * 1024 + 128 * sizeof(int32_t);
+  constexpr size_t shared = WIDE_STAGES * 24 * (WIDE_KSTEP / 32) * 1024 + 128 * sizeof(int32_t);
   static bool allowed[2] = {false, false};   // more than 64 KB of shared memory has to be asked for, once
 #define SE_WIDE(MODE)                                                                              \
   {                                                                                                \
     if (!allowed[MODE]) {                                                                          \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_wide_kernel<MODE, WIDE_WAVES>), \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_wide_kernel<MODE, WIDE_WAVES, WIDE_KSTEP>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize,                          \
                               static_cast<int>(shared)) != hipSuccess)                             \
         return SE_ERR_LAUNCH;                                                                      \
       allowed[MODE] = true;                                                                        \
     }                                                                                              \
-    grouped_gemm_wide_kernel<MODE, WIDE_WAVES><<<grid, 64 * WIDE_WAVES, shared, stream>>>(         \
+    grouped_gemm_wide_kernel<MODE, WIDE_WAVES, WIDE_KSTEP><<<grid, 64 * WIDE_WAVES, shared, stream>>>(         \
         static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
         tile_expert, counters, route_weight, assignments, top_k, N, K);                            \
   }
