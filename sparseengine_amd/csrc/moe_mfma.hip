@@ -452,28 +452,27 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 // Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1); tiles of 128 sorted rows.
 // ---------------------------------------------------------------------------------------- //
 #define WIDE_STAGES 3
-#ifndef WIDE_WAVES
-#define WIDE_WAVES 8     // wavefronts per block
-#endif
 #ifndef WIDE_KSTEP
 #define WIDE_KSTEP 32    // k per stage
 #endif
 
-template <int MODE, int WAVES, int KSTEP>   // WAVES: 4 (each 64 rows x 128 weight rows) or 8 (each 64 x 64); KSTEP: 32 or 64
-__global__ void __launch_bounds__(64 * WAVES, KSTEP == 32 ? 2 : 1)
+template <int MODE, int BM, int KSTEP>   // BM: 64 or 128 rows per tile; KSTEP: 32 or 64 along K per stage
+__global__ void __launch_bounds__(4 * BM, KSTEP == 32 ? 2 : 1)
 grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
                          bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
                          const int32_t* __restrict__ tile_expert,
                          const int32_t* __restrict__ counters,
                          const float* __restrict__ route_weight, int assignments, int top_k, int N,
                          int K) {
-  constexpr int BM = 128;
   constexpr int OUT_COLS = MODE == 0 ? 128 : 256;
-  constexpr int WCOLS = WAVES / 2;               // wave columns: the tile's 256 weight rows in 2 or 4 parts
-  constexpr int CB = 16 / WCOLS;                 // weight row blocks of a wave: 8 or 4
-  constexpr int PAIRS = 24 / WAVES;              // row blocks a wave brings per step: 6 or 3
+  constexpr int WAVES = BM / 16;                 // 4 or 8: each wavefront 64 rows x 64 weight rows
+  constexpr int WCOLS = 4;                       // wave columns: the tile's 256 weight rows in 4 parts
+  constexpr int CB = 16 / WCOLS;                 // weight row blocks of a wave
+  constexpr int ROW_BLOCKS = 16 + BM / 16;       // weight and activation row blocks of a step
+  constexpr int PAIRS = ROW_BLOCKS / WAVES;      // row blocks a wave brings per step: 5 or 3
   constexpr int HALVES = KSTEP / 32;             // chunks of 32 k per row block and step
-  constexpr int CHUNKS = 24 * HALVES;            // per stage
+  constexpr int CHUNKS = ROW_BLOCKS * HALVES;    // per stage
+  static_assert(ROW_BLOCKS % WAVES == 0, "the step's row blocks are shared out evenly");
   int tile, column_block;
   if (!xcd_work_item(N / OUT_COLS, counters[0], tile, column_block)) return;  // uniform
   extern __shared__ __align__(16) uint4 wide_shared[];     // WIDE_STAGES x CHUNKS x 64 vectors, then the rows
@@ -606,33 +605,47 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   }
 }
 
-// tile_rows: 128.  MODE 0 needs N % 128 == 0, MODE 1 N % 256 == 0; K % 64 == 0.
+// tile_rows: 64 or 128.  MODE 0 needs N % 128 == 0, MODE 1 N % 256 == 0; K % 64 == 0.
+template <int MODE, int BM>
+static int launch_wide(const void* in, const void* w, void* out, const int32_t* sorted,
+                       const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
+                       int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
+  const int64_t items = static_cast<int64_t>(N / (MODE == 0 ? 128 : 256)) * max_tiles;
+  const int grid = static_cast<int>((items + 7) / 8 * 8);
+  constexpr size_t shared = WIDE_STAGES * (16 + BM / 16) * (WIDE_KSTEP / 32) * 1024 + BM * sizeof(int32_t);
+  static bool allowed = false;   // more than 64 KB of shared memory has to be asked for, once
+  if (!allowed) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_wide_kernel<MODE, BM, WIDE_KSTEP>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared)) != hipSuccess)
+      return SE_ERR_LAUNCH;
+    allowed = true;
+  }
+  grouped_gemm_wide_kernel<MODE, BM, WIDE_KSTEP><<<grid, 4 * BM, shared, stream>>>(
+      static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
+      tile_expert, counters, route_weight, assignments, top_k, N, K);
+  return SE_OK;
+}
+
 extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, const int32_t* sorted,
                                     const int32_t* tile_expert, const int32_t* counters,
                                     const float* route_weight, int assignments, int top_k, int N,
                                     int K, int max_tiles, int mode, int tile_rows, hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
-  if (K <= 0 || K % 64 || N <= 0 || N % (mode == 0 ? 128 : 256) || tile_rows != 128) return SE_ERR_SHAPE;
+  if (K <= 0 || K % 64 || N <= 0 || N % (mode == 0 ? 128 : 256)) return SE_ERR_SHAPE;
+  if (tile_rows != 64 && tile_rows != 128) return SE_ERR_SHAPE;
   if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
-  const int64_t items = static_cast<int64_t>(N / (mode == 0 ? 128 : 256)) * max_tiles;
-  const int grid = static_cast<int>((items + 7) / 8 * 8);
-  constexpr size_t shared = WIDE_STAGES * 24 * (WIDE_KSTEP / 32) * 1024 + 128 * sizeof(int32_t);
-  static bool allowed[2] = {false, false};   // more than 64 KB of shared memory has to be asked for, once
-#define SE_WIDE(MODE)                                                                              \
-  {                                                                                                \
-    if (!allowed[MODE]) {                                                                          \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_wide_kernel<MODE, WIDE_WAVES, WIDE_KSTEP>), \
-                              hipFuncAttributeMaxDynamicSharedMemorySize,                          \
-                              static_cast<int>(shared)) != hipSuccess)                             \
-        return SE_ERR_LAUNCH;                                                                      \
-      allowed[MODE] = true;                                                                        \
-    }                                                                                              \
-    grouped_gemm_wide_kernel<MODE, WIDE_WAVES, WIDE_KSTEP><<<grid, 64 * WIDE_WAVES, shared, stream>>>(         \
-        static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
-        tile_expert, counters, route_weight, assignments, top_k, N, K);                            \
-  }
-  if (mode == 0) SE_WIDE(0) else SE_WIDE(1)
-#undef SE_WIDE
+  int status;
+  if (mode == 0)
+    status = tile_rows == 128 ? launch_wide<0, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
+                                                    top_k, N, K, max_tiles, stream)
+                              : launch_wide<0, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
+                                                   top_k, N, K, max_tiles, stream);
+  else
+    status = tile_rows == 128 ? launch_wide<1, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
+                                                    top_k, N, K, max_tiles, stream)
+                              : launch_wide<1, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
+                                                   top_k, N, K, max_tiles, stream);
+  if (status != SE_OK) return status;
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -441,12 +441,14 @@ class HipKernels:
                 w[first:first + 8].copy_(self.tile_expert_weights(w[first:first + 8]))
         return True
 
-    def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, tile_rows=None, wide=None, tall=None,
-                    tiled: bool = False):
+    def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, kernel=None, tile_rows=None,
+                    column_blocks=None, tiled: bool = False):
         """``out[t] = sum_k weights[t,k] * W2_e(silu(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``;
         ``w13 [E, 2I, h]`` holds gate rows then up rows, ``w2 [E, h, I]``.  ``tiled``: the tables
         have been through ``arrange_expert_weights``; row-major tables of sizes the matrix-core
-        kernels take are put into tiles here, call by call (tests; the model arranges them once)."""
+        kernels take are put into tiles here, call by call (tests; the model arranges them once).
+        ``kernel`` ("stream", "tall", "direct"), ``tile_rows`` and ``column_blocks`` override the
+        choice of the matrix-core kernel and its tile (tests and measurements)."""
         tokens, hidden = x.shape
         experts, two_i, _ = w13.shape
         inter = two_i // 2
@@ -463,51 +465,58 @@ class HipKernels:
         if self.takes_tiled_expert_weights(x.dtype, hidden, inter):
             if not tiled:
                 w13, w2 = self.tile_expert_weights(w13), self.tile_expert_weights(w2)
-            # matrix-core path.  The streaming kernel reads an expert's weights once per tile of 16
-            # rows, the tall one once per 64 rows and shares them among the tiles of an expert that
-            # run side by side.  Which experts a step uses is known on the device only: the choice
-            # goes by the average share and has to hold for even and for lumpy routing alike.
-            # Measured at MiniMax-M2 sizes (256 experts, top 8): with even routing the streaming
-            # kernel wins by 3 to 5 % up to 128 tokens and loses by 11 % at 512; when the tokens of
-            # a step agree on a few dozen experts (deep layers of a prompt) the tall kernel wins
-            # from 48 tokens on, by a factor of two at 512.  So: tall from three rows per expert on
-            # (a decode batch of 64 keeps the streaming kernel, a prompt portion of 96 does not).
+            # matrix-core path, three kernels:
+            #   "stream"  weights from memory straight into operands, tiles of 16 (32, 64) rows: an
+            #             expert's table is read once per tile;
+            #   "tall"    64 x 128 tiles, operands through registers into LDS, an expert's tiles side by side;
+            #   "direct"  64 or 128 rows x 256 weight rows, operands straight into LDS as contiguous
+            #             kilobytes of the tiled tables, two blocks per CU.
+            # Which experts a step uses is known on the device only: the choice goes by the average
+            # rows per expert and has to hold for even and for lumpy routing alike.  Measured at
+            # MiniMax-M2 sizes (256 experts, top 8): with even routing "stream" wins by 3 to 5 % up to
+            # 128 tokens and loses by 11 % at 512; when the tokens of a step agree on a few dozen
+            # experts (deep layers of a prompt) it loses from 48 tokens on, by a factor of two at
+            # 512.  So: "stream" below three rows per expert (a decode batch of 64 keeps it, a
+            # prompt portion of 96 does not).  "direct" with 128 rows equals "tall" at 384 tokens of
+            # a prompt and is 6 % faster at 512, 15 % at 1024, 23 % at 2048 (registers are fed at a
+            # third of the rate of direct loads); with tiles of 64 rows it equals "tall" from 96 to
+            # 384 tokens, so that one stays for three to sixteen rows per expert.
             share = assignments / min(experts, assignments)
-            asked_rows = tile_rows
-            if tall is None:
-                tall = share >= 3 if tile_rows is None else tile_rows >= 64
+            direct_ok = inter % 128 == 0 and hidden % 256 == 0
+            if kernel is None:
+                if tile_rows is not None:
+                    kernel = "stream" if tile_rows < 64 else ("direct" if tile_rows == 128 and direct_ok else "tall")
+                else:
+                    kernel = "stream" if share < 3 else ("direct" if share >= 16 and direct_ok else "tall")
+            if kernel not in ("stream", "tall", "direct"):
+                raise ValueError(f"expert kernel {kernel!r} is unknown (stream, tall, direct)")
+            if kernel == "direct" and not direct_ok:
+                raise KernelShapeError("the direct expert kernel takes hidden sizes in steps of 256 and "
+                                       "intermediate sizes in steps of 128")
             if tile_rows is None:
-                tile_rows = 64 if tall else 16
-            if tall:
-                # from 16 rows per expert on: the 128 x 256 tile, whose operands go straight into LDS as
-                # contiguous kilobytes (the 64 x 128 kernel brings them through registers, which the
-                # chip feeds at a third of that rate).  Measured on prompt portions at MiniMax-M2
-                # sizes: equal at 384 tokens, 6 % faster at 512, 15 % at 1024, 23 % at 2048.
-                wide_tile = (((share >= 16 and asked_rows is None) or asked_rows == 128)
-                             and inter % 128 == 0 and hidden % 256 == 0)
-                tile_rows = 128 if wide_tile else 64
+                tile_rows = {"stream": 16, "tall": 64, "direct": 128 if share >= 16 else 64}[kernel]
             max_tiles = self._grouped_tiles(ids, experts, ws, tile_rows)
             if max_tiles > 65535:
                 raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
-            if tall:
-                gt = _fn.get("moe_mfma", "se_grouped_gemm_wide" if tile_rows == 128 else "se_grouped_gemm_tall")
-                _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
-                          _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                          _stream()), "moe gate-up (tall)", "hidden and intermediate sizes in multiples of 128")
-                _check(gt(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
-                          _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                          tile_rows, _stream()), "moe down (tall)", "hidden and intermediate sizes in multiples of 128")
-            else:
+            takes = "hidden and intermediate sizes in multiples of 128"
+            if kernel == "stream":
                 gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
-                if wide is None:
-                    wide = 2 if max_tiles * (inter // 32) >= 2048 else 1
+                if column_blocks is None:
+                    column_blocks = 2 if max_tiles * (inter // 32) >= 2048 else 1
                 _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                          wide, _stream()), "moe gate-up (mfma)", "hidden and intermediate sizes in multiples of 128")
+                          column_blocks, _stream()), "moe gate-up (stream)", takes)
                 _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                          tile_rows, wide, _stream()), "moe down (mfma)",
-                       "hidden and intermediate sizes in multiples of 128")
+                          tile_rows, column_blocks, _stream()), "moe down (stream)", takes)
+            else:
+                gt = _fn.get("moe_mfma", "se_grouped_gemm_wide" if kernel == "direct" else "se_grouped_gemm_tall")
+                _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                          _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
+                          _stream()), f"moe gate-up ({kernel})", takes)
+                _check(gt(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                          _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
+                          tile_rows, _stream()), f"moe down ({kernel})", takes)
         else:
             _require(not tiled, "the general expert kernel reads row-major tables")
             max_tiles = self._grouped_tiles(ids, experts, ws, 16)

@@ -377,10 +377,11 @@ def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
     twin.moe_experts(x, w13, w2, ids, weights, out_t)
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
     if dtype == torch.bfloat16 and hidden % 256 == 0 and inter % 128 == 0 and tokens <= 200:
-        # the wide tile on a step that would not choose it: mostly padding, same result
-        out_w = torch.empty_like(x)
-        hip.moe_experts(x, w13, w2, ids, weights, out_w, ws, tile_rows=128, tall=True)
-        torch.testing.assert_close(out_w, out_t, **tol(dtype))
+        # every kernel and tile on a step that would not choose it (mostly padding): same result
+        for kernel, rows in (("direct", 128), ("direct", 64), ("tall", 64), ("stream", 16), ("stream", 32)):
+            out_w = torch.empty_like(x)
+            hip.moe_experts(x, w13, w2, ids, weights, out_w, ws, kernel=kernel, tile_rows=rows)
+            torch.testing.assert_close(out_w, out_t, **tol(dtype))
     if experts == 1:   # one expert, k = 1: a plain SwiGLU feed-forward
         xf = x.float()
         ref = (torch.nn.functional.silu(xf @ w13[0, :inter].float().T) * (xf @ w13[0, inter:].float().T)) @ w2[0].float().T
