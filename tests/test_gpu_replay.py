@@ -16,7 +16,8 @@ from tests.plain.minimax_m2 import PlainMiniMaxM2
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
-LENGTHS = {"A": [5, 17, 31, 100, 64, 129, 250, 1, 48], "B": [1, 9, 40, 100, 200, 333, 65, 16, 500]}
+LENGTHS = {"A": [5, 17, 31, 100, 64, 129, 250, 1, 48], "B": [1, 9, 40, 100, 200, 333, 65, 16, 500],
+           "C": [3, 40, 130, 700, 64, 257, 1, 33, 520]}
 
 
 def bound(dtype, ref):
@@ -27,7 +28,7 @@ def bound(dtype, ref):
     return 2e-5 * max(scale, 1.0) if dtype == "float32" else 0.04 * scale
 
 
-@pytest.fixture(scope="module", params=["A_loud", "B_loud", "A", "B"])
+@pytest.fixture(scope="module", params=["A_loud", "B_loud", "A", "B", "C_loud"])
 def model(request, tmp_path_factory):
     key = request.param
     folder = make_folder(tmp_path_factory.mktemp("models"), key)
@@ -36,6 +37,11 @@ def model(request, tmp_path_factory):
     plain = PlainMiniMaxM2(folder)
     expected = {rid: plain.logits(toks).numpy() for rid, toks in requests.items()}
     return folder, requests, expected, plain
+
+
+def longest(requests) -> int:
+    """Cache tokens that hold the longest request (requests run one at a time)."""
+    return max(-(-len(t) // 64) * 64 for t in requests.values())
 
 
 def run_records(folder, dtype, records, max_tokens, page_size):
@@ -98,7 +104,7 @@ def compare(dtype, got, model, routing):
 def test_whole_requests(model, dtype, page_size):
     folder, requests = model[:2]
     records = traces.whole(requests)
-    logits, routing = run_records(folder, dtype, records, 512, page_size)
+    logits, routing = run_records(folder, dtype, records, longest(requests), page_size)
     compare(dtype, traces.gather(records, logits), model, routing)
 
 
@@ -106,7 +112,7 @@ def test_whole_requests(model, dtype, page_size):
 def test_prefill_then_last_32_one_by_one(model, dtype):
     folder, requests = model[:2]
     records = traces.prefill_then_decode(requests, tail=32)
-    logits, routing = run_records(folder, dtype, records, 512, 16)
+    logits, routing = run_records(folder, dtype, records, longest(requests), 16)
     compare(dtype, traces.gather(records, logits), model, routing)
 
 
@@ -115,7 +121,7 @@ def test_prefill_then_last_32_one_by_one(model, dtype):
 def test_portions_of_changing_size(model, dtype, page_size):
     folder, requests = model[:2]
     records = traces.changing_portions(requests, seed=page_size)
-    logits, routing = run_records(folder, dtype, records, 512, page_size)
+    logits, routing = run_records(folder, dtype, records, longest(requests), page_size)
     compare(dtype, traces.gather(records, logits), model, routing)
 
 
@@ -160,3 +166,26 @@ def test_trace_run_program(model, dtype, tmp_path):
         assert proc.returncode == 0, proc.stderr[-2000:]
         for r in records[:6]:
             assert np.array_equal(np.fromfile(other / f"{r['step']}.f32", dtype="<f4").reshape(-1, vocab), logits[r["step"]])
+
+
+def test_matrix_core_sizes_take_the_matrix_core_kernels(tmp_path):
+    """Configuration C is there to run what the full-size model runs: its expert tables are put into
+    tiles when the model is built in bfloat16 (and stay in rows in float32), and its head size goes
+    to the matrix-core attention kernels."""
+    from safetensors.torch import load_file
+    from sparseengine_amd.engine.runner import ModelRunner
+    from sparseengine_amd.kernels.hip_ops import HipKernels
+    folder = make_folder(tmp_path, "C_loud")
+    stored = load_file(os.path.join(folder, "model.safetensors"))
+    w1 = stored["model.layers.0.block_sparse_moe.experts.3.w1.weight"].cuda()
+    half = ModelRunner.from_folder(folder, dtype="bfloat16", kv_page_size=16, num_kvcache_tokens=256, max_num_seqs=2)
+    ffn = half.model.layers[0].ffn
+    assert ffn._tiled is True
+    inter = w1.shape[0]
+    tiled_expert = HipKernels.tile_expert_weights(torch.cat([w1, stored["model.layers.0.block_sparse_moe.experts.3.w3.weight"].cuda()])[None])
+    assert torch.equal(ffn.params["w13"][3:4], tiled_expert) and not torch.equal(ffn.params["w13"][3, :inter], w1)
+    full = ModelRunner.from_folder(folder, dtype="float32", kv_page_size=16, num_kvcache_tokens=256, max_num_seqs=2)
+    assert full.model.layers[0].ffn._tiled is False
+    assert torch.equal(full.model.layers[0].ffn.params["w13"][3, :inter], w1.float())
+    spec = half.spec.layers[0].mixer
+    assert spec.head_dim % 32 == 0 and spec.head_dim <= 128
