@@ -85,11 +85,12 @@ def test_first_tokens_of_a_sequence(tmp_path, dtype):
             assert np.abs(logits[2 * i:2 * i + 2] - ref[1:3]).max() <= bound(dtype, ref)
 
 
-def test_greedy_generation_through_the_entry_point(tmp_path):
+@pytest.mark.parametrize("key", ["A_loud", "C_loud"])     # the general kernels; the matrix-core kernels in bfloat16
+def test_greedy_generation_through_the_entry_point(tmp_path, key):
     from sparseengine_amd import LLM, SamplingParams
-    folder = make_folder(tmp_path, "A_loud")
+    folder = make_folder(tmp_path, key)
     plain = PlainMiniMaxM2(folder)
-    prompts = [random_tokens(n, 512, 300 + n) for n in (5, 17, 31, 90)]
+    prompts = [random_tokens(n, CONFIGS[key][0]["vocab_size"], 300 + n) for n in (5, 17, 31, 90)]
     params = SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True)
     expected = [plain.greedy(p, 24) for p in prompts]
     llm = LLM(folder, dtype="float32", num_kvcache_slots=1024, kv_page_size=16, max_num_seqs_in_batch=4,
@@ -101,11 +102,32 @@ def test_greedy_generation_through_the_entry_point(tmp_path):
     assert [o["token_ids"] for o in tight.generate(prompts, params, use_tqdm=False)] == expected
     assert tight.scheduler.total_preemptions >= 1
     # bfloat16: every generated token is, for the plain logits of its own context, as good as the best
-    # one up to bfloat16 rounding
+    # one up to bfloat16 rounding.  Rounding may tip a near-tie of the router, which moves logits by
+    # more than rounding does: the plain implementation runs with the experts the engine chose (the
+    # replay tests check that those are top-k choices up to a small slack).
     half = LLM(folder, dtype="bfloat16", num_kvcache_slots=1024, kv_page_size=16, max_num_seqs_in_batch=4)
-    for prompt, out in zip(prompts, half.generate(prompts, params, use_tqdm=False)):
+    run_step, fed = half.runner.step, {}
+
+    def step_and_note_routing(entries, taps=None):
+        taps = {}
+        logits = run_step(entries, taps=taps)
+        cursor = 0
+        for e in entries:
+            n = len(e.tokens)
+            layers = fed.setdefault(e.request_id, [[] for _ in taps["router"]])
+            for layer, (ids, _) in enumerate(taps["router"]):
+                layers[layer].append(ids[cursor:cursor + n].cpu())
+            cursor += n
+        return logits
+    half.runner.step = step_and_note_routing
+    outs = half.generate(prompts, params, use_tqdm=False)
+    by_request = [fed[k] for k in sorted(fed)]              # sequence ids grow in the order of the prompts
+    assert len(by_request) == len(prompts) and half.scheduler.total_preemptions == 0
+    for prompt, out, layers in zip(prompts, outs, by_request):
         ids = out["token_ids"]
-        logits = plain.logits(prompt + ids)[len(prompt) - 1:-1]
+        routing = [torch.cat(chunks).long() for chunks in layers]
+        assert routing[0].shape[0] == len(prompt) + len(ids) - 1     # every token but the last was fed once
+        logits = plain.logits(prompt + ids[:-1], forced_routing=routing)[len(prompt) - 1:]
         chosen = logits.gather(1, torch.tensor(ids)[:, None])[:, 0]
         assert (logits.max(-1).values - chosen).max() <= 2 * 0.04 * float(logits.abs().max())
     # temperature sampling: the same seed gives the same tokens, alone and in a batch
