@@ -7,7 +7,8 @@ top-8 of width 1536, vocabulary 200064) cut to 16 of its 62 layers, random weigh
 A "step" is one decode step of a batch of 8 requests whose prompts were 2048 random token ids
 (sampling greedily, token ids read back each step).  One JSON line is printed: ``value`` is decoded
 tokens per second at batch 8; ``prefill`` is a 2048-token prompt in one step; ``points`` holds
-decode at batch 1 and 64; ``roofline`` prices the batch-8 decode step against 8 TB/s.
+decode at batch 1 and 64 and the prefill of eight 2048-token prompts in one step; ``roofline``
+prices the batch-8 decode step against 8 TB/s.
 """
 from __future__ import annotations
 
@@ -41,8 +42,8 @@ def main() -> int:
     parser.add_argument("--kv-requests", type=int, default=64, help="requests of full context the cache is sized for")
     parser.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiling decode)")
     parser.add_argument("--no-decode", action="store_true", help="skip the decode measurements (for profiling prefill)")
-    parser.add_argument("--prefill-prompts", type=int, default=1,
-                        help="also time this many 2048-token prompts in one step (reported on stderr only)")
+    parser.add_argument("--prefill-prompts", type=int, default=8,
+                        help="also time this many 2048-token prompts in one step (points.prefill_Nx2048); 1: skip")
     parser.add_argument("--fake-context", action="store_true",
                         help="profiling aid, never used for reported numbers: reserve the prompts' cache pages "
                              "without computing them, so that a kernel trace holds decode steps only")
@@ -147,7 +148,8 @@ def main() -> int:
     peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
     print(f"[bench] prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
 
-    if args.prefill_prompts > 1:          # several prompts in one step: hundreds of rows per expert
+    many_prompts = None
+    if args.prefill_prompts > 1 and not args.no_prefill:      # several prompts in one step: hundreds of rows per expert
         n, best = args.prefill_prompts, float("inf")
         for i in range(3):
             ids = [f"m{i}_{j}" for j in range(n)]
@@ -159,6 +161,7 @@ def main() -> int:
             best = min(best, time.perf_counter() - t)
             for r in ids:
                 runner.release(r)
+        many_prompts = (f"prefill_{n}x{T}", round(n * T / best, 1))
         print(f"[bench] prefill {n} x {T} tokens in one step: {best * 1e3:.1f} ms, {n * T / best:.0f} tokens/s",
               file=sys.stderr, flush=True)
 
@@ -173,6 +176,8 @@ def main() -> int:
         points[f"decode_b{b}"] = round(b / s, 1)
         print(f"[bench] decode batch {b}: {s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
 
+    if many_prompts:
+        points[many_prompts[0]] = many_prompts[1]
     achieved = decode_bytes(args.batch, distinct, context) / step_s
     line = {
         "metric": f"decode tok/s @ batch {args.batch} (MiniMax-M2 sizes, {L} layers, 1 GPU)", "value": round(args.batch / step_s, 1),
