@@ -47,7 +47,7 @@ def replay_with_routing(runner, records):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("key", ["B_loud", "A_loud"])
+@pytest.mark.parametrize("key", ["B_loud", "A_loud", "C_loud"])
 def test_long_decoding_token_by_token(tmp_path, key, dtype):
     """A short prompt and then hundreds of single-token steps across many pages."""
     folder = make_folder(tmp_path, key)
