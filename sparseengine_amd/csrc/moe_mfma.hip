@@ -449,7 +449,8 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 // blocks per CU: 5.1.
 //   MODE 0: out[a, n0 + 32 wc + 16 cb + ...] from gate rows n0 + 32 wc ..., up rows N + n0 + 32 wc ...
 //   MODE 1: out[a, n0 + 64 wc + 16 cb + ...] * route_weight[a]
-// Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1); tiles of 128 sorted rows.
+// Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1); tiles of 128 sorted rows (BM = 64:
+// four wavefronts on 64 rows, measured equal to the tall kernel where that one is used).
 // ---------------------------------------------------------------------------------------- //
 #define WIDE_STAGES 3
 #ifndef WIDE_KSTEP
