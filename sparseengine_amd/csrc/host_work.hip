@@ -53,6 +53,7 @@ int se_attention_work_plan(const int64_t* q_len, const int64_t* ctx_len, int ite
   const bool blocks_allowed = head_dim > 0 && head_dim % 32 == 0 && head_dim <= r.tiled_max_head_dim;
   std::vector<int64_t> tiles(items), reach(items), nblocks(items), alone(items);
   for (int i = 0; i < items; ++i) {
+    if (q_len[i] < 1 || q_len[i] > ctx_len[i]) return -2;   // an item's new tokens are part of its context
     tiles[i] = (q_len[i] * group + 15) / 16;
     reach[i] = window ? std::min<int64_t>(ctx_len[i], window + q_len[i]) : ctx_len[i];
     const bool in_blocks = blocks_allowed && tiles[i] >= r.tiles_per_block / 2;

@@ -75,6 +75,9 @@ def _native_library():
     return _native or None
 
 
+_BAD_LENGTHS = "attention work: every item needs at least one new token and no more new tokens than its context holds"
+
+
 def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int = 0,
                          target_waves: int = TARGET_WAVES, head_dim: int = 0) -> AttentionWork:
     """The work lists of one step; see ``build_attention_work_numpy`` for the rules.  The compiled
@@ -90,8 +93,11 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
     counts = np.empty(4, dtype=np.int64)
     i64p, i32p = ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32)
     as64 = lambda a: a.ctypes.data_as(i64p)
-    if lib.se_attention_work_plan(as64(q), as64(c), q.size, group, kv_heads, int(window or 0), int(head_dim or 0),
-                                  as64(rules), as64(plan), as64(counts)) != 0:
+    status = lib.se_attention_work_plan(as64(q), as64(c), q.size, group, kv_heads, int(window or 0), int(head_dim or 0),
+                                        as64(rules), as64(plan), as64(counts))
+    if status == -2:
+        raise ValueError(_BAD_LENGTHS)
+    if status != 0:
         raise ValueError("attention work: bad arguments")
     units = np.empty((int(counts[0]), UNIT_FIELDS), dtype=np.int32)
     tasks = np.empty((int(counts[1]), TASK_FIELDS), dtype=np.int32)
@@ -111,6 +117,8 @@ def build_attention_work_numpy(q_len, ctx_len, group: int, kv_heads: int, window
     context beside short ones does not become the one long-running unit."""
     q_len = np.asarray(q_len, dtype=np.int64)
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
+    if ((q_len < 1) | (q_len > ctx_len)).any():
+        raise ValueError(_BAD_LENGTHS)
     q_start = np.concatenate(([0], np.cumsum(q_len)[:-1]))      # items' tokens lie one after the other
     tiles = (q_len * group + 15) // 16
     reach = np.minimum(ctx_len, window + q_len) if window else ctx_len      # keys an item's tiles can read

@@ -271,6 +271,15 @@ def test_block_work_lists_for_many_rows_cover_every_tile_once_longest_first():
     assert len(build_attention_work([1] * 8, [300] * 8, 6, 8, 0, head_dim=128).block_units) == 0
 
 
+def test_work_lists_refuse_items_with_more_new_tokens_than_context():
+    from sparseengine_amd.kernels.attention_work import build_attention_work_numpy
+    for builder in (build_attention_work, build_attention_work_numpy):
+        for q_len, ctx_len in (([2], [1]), ([1, 0], [5, 5]), ([3, 9], [3, 8])):
+            with pytest.raises(ValueError, match="new token"):
+                builder(q_len, ctx_len, 6, 8, 0, head_dim=128)
+        builder([3, 8], [3, 8], 6, 8, 0, head_dim=128)
+
+
 def test_compiled_work_list_builder_gives_the_same_lists():
     """csrc/host_work.hip against the numpy builder, list for list, on random steps."""
     import numpy as np
