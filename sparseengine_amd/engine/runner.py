@@ -74,7 +74,7 @@ class ModelRunner:
         requests = self.model.cache_requests()
         if num_kvcache_tokens is None or int(num_kvcache_tokens) <= 0:
             num_kvcache_tokens = self.derive_cache_tokens(requests, max_num_seqs, gpu_memory_utilization)
-        num_pages = max(1, int(num_kvcache_tokens) // self.kv_page_size)
+        num_pages = max(1, -(-int(num_kvcache_tokens) // self.kv_page_size))      # a last page may be partly beyond the count
         self.cache = CacheManager(requests, max_rows=max_num_seqs,
                                   max_model_len=self.max_model_len, page_size=self.kv_page_size,
                                   num_pages=num_pages, dtype=self.dtype, device=self.device)
