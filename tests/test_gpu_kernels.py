@@ -635,3 +635,68 @@ def test_expert_tables_arranged_in_place_are_the_tiled_copy(hip, twin):
     hip.moe_experts(x, a13, a2, ids, weights, out_h, ws, tiled=True)
     twin.moe_experts(x, w13, w2, ids, weights, out_t)
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
+
+
+def test_attention_on_random_shapes(hip):
+    """Seeded random shapes (heads and groups, head sizes up to 256, page sizes that do not divide 32,
+    windows, items from one decoded token to a long prompt) through the matrix-core kernels, each
+    checked at a few rows against the library routine on the gathered keys."""
+    import random
+    rng = random.Random(3)
+    dtype = torch.bfloat16
+    for case in range(24):
+        kv_heads = rng.choice([1, 2, 3, 8])
+        heads = kv_heads * rng.choice([1, 2, 4, 6, 7])
+        head_dim = rng.choice([32, 64, 96, 128, 160, 256])
+        page = rng.choice([8, 16, 24, 40, 64])
+        window = rng.choice([0, 0, 0, 17, 100, 333])
+        lens, q_lens = [], []
+        for _ in range(rng.randint(1, 5)):
+            n = rng.choice([1, 2, 31, 32, 33, 64, 100, 255, 256, 500, 1000, 2500])
+            lens.append(n)
+            q_lens.append(max(1, min(n, rng.choice([1, 1, 2, 16, 65, n]))))
+        cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=case)
+        meta = make_meta(table, lens, q_lens)
+        T = sum(q_lens)
+        q = randn(T, heads, head_dim, dtype=dtype, seed=case + 1)
+        out = torch.full((T, heads * head_dim), float("nan"), dtype=dtype, device="cuda")
+        scale = head_dim ** -0.5
+        hip.paged_attention(q, cache, meta, out, scale, window)
+        what = f"case {case}: heads {heads}/{kv_heads}, head_dim {head_dim}, page {page}, window {window}, lens {lens}, new {q_lens}"
+        assert torch.isfinite(out.float()).all(), what
+        for t in sorted({0, T // 3, T // 2, T - 1}):
+            row, pos = int(meta.token_row[t]), int(meta.positions[t])
+            ref = dense_attention(q[t], cache, table, row, pos, scale, window, page)
+            torch.testing.assert_close(out[t].float(), ref, rtol=1.6e-2, atol=1.6e-2, msg=lambda m: f"{what}, token {t}: {m}")
+
+
+def test_experts_on_random_shapes_and_lumpy_routing(hip, twin):
+    """Seeded random sizes and token counts with routing that prefers a few experts, through the
+    kernel the host would choose and through every other one."""
+    import random
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    rng = random.Random(4)
+    dtype = torch.bfloat16
+    for case in range(16):
+        experts = rng.choice([3, 4, 8, 16, 64])
+        k = rng.randint(1, min(8, experts))
+        hidden, inter = rng.choice([256, 512, 768]), rng.choice([128, 256, 384])
+        tokens = rng.choice([1, 2, 7, 16, 17, 33, 64, 100, 255, 256, 257, 500, 1000, 2100])
+        g = torch.Generator().manual_seed(case)
+        x = torch.randn(tokens, hidden, generator=g).to(dtype).cuda()
+        w13 = (torch.randn(experts, 2 * inter, hidden, generator=g) * hidden ** -0.5).to(dtype).cuda()
+        w2 = (torch.randn(experts, hidden, inter, generator=g) * inter ** -0.5).to(dtype).cuda()
+        liking = torch.rand(experts, generator=g) ** 3 + 1e-3
+        ids = torch.stack([torch.multinomial(liking, k, generator=g) for _ in range(tokens)]).to(torch.int32).cuda()
+        weights = torch.rand(tokens, k, generator=g).cuda()
+        weights = weights / weights.sum(-1, keepdim=True)
+        ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+        ref = torch.empty_like(x)
+        twin.moe_experts(x, w13, w2, ids, weights, ref)
+        a13, a2 = w13.clone(), w2.clone()
+        assert hip.arrange_expert_weights(a13, a2)
+        for kernel, rows in ((None, None), ("stream", 16), ("tall", 64), ("direct", 64), ("direct", 128)):
+            out = torch.full_like(x, float("nan"))
+            hip.moe_experts(x, a13, a2, ids, weights, out, ws, kernel=kernel, tile_rows=rows, tiled=True)
+            torch.testing.assert_close(out, ref, **tol(dtype), msg=lambda m: (
+                f"case {case}: {tokens} tokens, {experts} experts, top {k}, hidden {hidden}, width {inter}, kernel {kernel}: {m}"))
