@@ -138,6 +138,39 @@ def test_greedy_generation_through_the_entry_point(tmp_path, key):
     assert alone == mixed
 
 
+def test_random_workloads_through_the_entry_point(tmp_path):
+    """Seeded random workloads (numbers and lengths of requests, completion lengths, page sizes, cache
+    sizes from ample to barely enough, token budgets down to eight) in float32: every request gets
+    exactly the plain implementation's greedy tokens, whatever was cut, batched, deferred or thrown
+    out and computed again on the way."""
+    import random
+    from sparseengine_amd import LLM, SamplingParams
+    rng = random.Random(11)
+    key = "B_loud"
+    folder = make_folder(tmp_path, key)
+    raw = CONFIGS[key][0]
+    plain = PlainMiniMaxM2(folder)
+    known = {}
+    preemptions = 0
+    for scenario in range(5):
+        n = rng.randint(2, 8)
+        prompts = [random_tokens(rng.choice([1, 3, 17, 40, 90, 150]), raw["vocab_size"], rng.randrange(10 ** 6)) for _ in range(n)]
+        params = [SamplingParams(temperature=0.0, max_tokens=rng.choice([1, 5, 20, 40]), ignore_eos=True) for _ in range(n)]
+        page = rng.choice([8, 16, 32])
+        need = max(len(p) + sp.max_tokens for p, sp in zip(prompts, params))
+        slots = max(-(-need // page) * page + page, rng.choice([160, 192, 256, 512]))
+        in_batch = rng.choice([2, 4, 8])
+        llm = LLM(folder, dtype="float32", num_kvcache_slots=slots, kv_page_size=page, max_num_seqs_in_batch=in_batch,
+                  max_num_batched_tokens=max(in_batch, rng.choice([8, 16, 64, 512])),
+                  decode_reservation_tokens=rng.choice([0, 16, 64]), validate_runtime_invariants=True)
+        outs = llm.generate(prompts, params, use_tqdm=False)
+        for p, sp, o in zip(prompts, params, outs):
+            ref = known.setdefault((tuple(p), sp.max_tokens), plain.greedy(p, sp.max_tokens))
+            assert o["token_ids"] == ref, f"scenario {scenario}: prompt of {len(p)}, {sp.max_tokens} new tokens"
+        preemptions += llm.scheduler.total_preemptions
+    assert preemptions >= 1, "no scenario ran out of pages: the seed no longer covers preemption"
+
+
 def test_command_line_generates_what_the_entry_point_generates(tmp_path, capsys):
     import json
     from sparseengine_amd import LLM, SamplingParams
