@@ -17,7 +17,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
                                             const float* __restrict__ bias, int32_t* __restrict__ ids,
                                             float* __restrict__ weights, int token, int experts,
                                             int top_k, int softmax_scoring, int normalize,
-                                            float scaling) {
+                                            float scaling, int32_t* ids_copy = nullptr) {
   const int lane = threadIdx.x & (SE_WAVE - 1);
   const float* row = logits + static_cast<int64_t>(token) * stride;
 
@@ -104,6 +104,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     if (!(taken & (1u << i))) continue;
     const int slot = my_slot[i] >= 0 ? my_slot[i] : greater_before + (-my_slot[i] - 1);
     ids[static_cast<int64_t>(token) * top_k + slot] = i * SE_WAVE + lane;
+    if (ids_copy) ids_copy[token * top_k + slot] = i * SE_WAVE + lane;
     weights[static_cast<int64_t>(token) * top_k + slot] =
         (normalize ? score[i] / total : score[i]) * scaling;
   }
@@ -124,12 +125,10 @@ __global__ void router_topk_kernel(const float* __restrict__ logits, int64_t str
 // Router logits of a step with few tokens: logits[t, e] = x[t] . w[e], float accumulate from
 // float weights; the activations are widened as they are read (no float copy of x, no library
 // call whose launch and set-up cost more than the product).  One wavefront per expert; a lane
-// takes 8 consecutive k out of every 512 and keeps the sums of up to ROUTER_TOKEN_GROUP tokens.
+// takes 8 consecutive k out of every 512 and keeps the sums of up to TG (1, 2, 4, 8) tokens.
 // Requires K % 8 == 0 and 16-byte aligned rows.
 // ---------------------------------------------------------------------------------------- //
-#define ROUTER_TOKEN_GROUP 8
-
-template <typename T>
+template <typename T, int TG>   // TG tokens at a time share the weight loads
 __global__ void __launch_bounds__(256)
 router_logits_kernel(const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
                      float* __restrict__ logits, int64_t out_stride, int tokens, int experts, int K) {
@@ -137,18 +136,21 @@ router_logits_kernel(const T* __restrict__ x, int64_t x_stride, const float* __r
   const int expert = blockIdx.x * 4 + threadIdx.x / SE_WAVE;
   if (expert >= experts) return;   // whole waves leave together; there is no block barrier below
   constexpr int XV = 8 / Vec16<T>::N;            // 16-byte vectors of 8 activations
+  // steps of 512 along K whose loads go out together: with one token the product is a chain of
+  // memory round trips otherwise (measured at 256 x 3072: 5.8 -> 4.7 us)
+  constexpr int UNROLL = TG <= 2 ? 8 : (TG == 4 ? 4 : 2);
   const float* w_row = w + static_cast<int64_t>(expert) * K;
-  for (int t0 = 0; t0 < tokens; t0 += ROUTER_TOKEN_GROUP) {
-    float acc[ROUTER_TOKEN_GROUP];
+  for (int t0 = 0; t0 < tokens; t0 += TG) {
+    float acc[TG];
 #pragma unroll
-    for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g) acc[g] = 0.f;
-#pragma unroll 2
+    for (int g = 0; g < TG; ++g) acc[g] = 0.f;
+#pragma unroll UNROLL
     for (int k = lane * 8; k < K; k += SE_WAVE * 8) {
       const float4 w0 = *reinterpret_cast<const float4*>(w_row + k);
       const float4 w1 = *reinterpret_cast<const float4*>(w_row + k + 4);
-      Vec16<T> xv[ROUTER_TOKEN_GROUP][XV];
+      Vec16<T> xv[TG][XV];
 #pragma unroll
-      for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g) {
+      for (int g = 0; g < TG; ++g) {
         const int t = min(t0 + g, tokens - 1);     // rows past the end repeat the last one
         const T* xr = x + static_cast<int64_t>(t) * x_stride + k;
 #pragma unroll
@@ -157,13 +159,13 @@ router_logits_kernel(const T* __restrict__ x, int64_t x_stride, const float* __r
       }
       const float wk[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
-      for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g)
+      for (int g = 0; g < TG; ++g)
 #pragma unroll
         for (int j = 0; j < 8; ++j)
           acc[g] = fmaf(xv[g][j / Vec16<T>::N].get(j % Vec16<T>::N), wk[j], acc[g]);
     }
 #pragma unroll
-    for (int g = 0; g < ROUTER_TOKEN_GROUP; ++g) {
+    for (int g = 0; g < TG; ++g) {
       const float total = wave_sum(acc[g]);
       if (lane == 0 && t0 + g < tokens) logits[static_cast<int64_t>(t0 + g) * out_stride + expert] = total;
     }
@@ -263,10 +265,13 @@ __global__ void router_topk_align_kernel(const float* __restrict__ logits, int64
                                          int32_t* __restrict__ tile_expert,
                                          int32_t* __restrict__ counters) {
   extern __shared__ int32_t sh[];
+  // the chosen experts also stay in shared memory: grouping them from there saves the round trip
+  // of writing them to memory and reading them back (about 1.5 us of a 9 us launch)
+  int32_t* chosen = sh + 3 * experts + 1;   // [tokens * top_k]
   route_token<PER_LANE>(logits, stride, bias, ids, weights, threadIdx.x / SE_WAVE, experts, top_k,
-                        softmax_scoring, normalize, scaling);
-  __syncthreads();   // the block's own writes of ids are visible to all its threads from here on
-  align_assignments(ids, tokens * top_k, experts, tile_rows, sorted, tile_expert, counters, sh);
+                        softmax_scoring, normalize, scaling, chosen);
+  __syncthreads();
+  align_assignments(chosen, tokens * top_k, experts, tile_rows, sorted, tile_expert, counters, sh);
 }
 
 // ---------------------------------------------------------------------------------------- //
@@ -408,12 +413,17 @@ int se_router_logits(const void* x, int64_t x_stride, const float* w, float* log
   if (tokens <= 0) return SE_OK;
   if (experts <= 0 || K <= 0 || K % 8 || x_stride % 8) return SE_ERR_SHAPE;
   const dim3 grid((experts + 3) / 4);
-  if (dtype == SE_F32)
-    router_logits_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(x), x_stride, w, logits,
-                                                          out_stride, tokens, experts, K);
-  else
-    router_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, w,
-                                                           logits, out_stride, tokens, experts, K);
+#define SE_RL(T, TG)                                                                              \
+  router_logits_kernel<T, TG><<<grid, 256, 0, stream>>>(static_cast<const T*>(x), x_stride, w, logits, \
+                                                        out_stride, tokens, experts, K)
+#define SE_RL_TG(T)                                                                               \
+  if (tokens <= 1) SE_RL(T, 1);                                                                   \
+  else if (tokens <= 2) SE_RL(T, 2);                                                              \
+  else if (tokens <= 4) SE_RL(T, 4);                                                              \
+  else SE_RL(T, 8)
+  if (dtype == SE_F32) { SE_RL_TG(float); } else { SE_RL_TG(bf16_t); }
+#undef SE_RL_TG
+#undef SE_RL
   SE_CHECK_LAUNCH();
   return SE_OK;
 }
@@ -426,7 +436,8 @@ int se_router_topk_align(const float* logits, int64_t stride, const float* bias,
   if (tokens <= 0) return SE_OK;
   if (tokens > 16 || experts <= 0 || experts > SE_WAVE * ROUTER_MAX_PER_LANE) return SE_ERR_SHAPE;
   if (top_k <= 0 || top_k > experts || tile_rows <= 0) return SE_ERR_SHAPE;
-  const size_t shmem = (3 * static_cast<size_t>(experts) + 1) * sizeof(int32_t);
+  const size_t shmem = (3 * static_cast<size_t>(experts) + 1 + static_cast<size_t>(tokens) * top_k) * sizeof(int32_t);
+  if (shmem > 64 * 1024) return SE_ERR_SHAPE;
   if (experts <= SE_WAVE * 4) {
     router_topk_align_kernel<4><<<1, tokens * SE_WAVE, shmem, stream>>>(
         logits, stride, bias, ids, weights, tokens, experts, top_k, softmax_scoring, normalize, scaling,

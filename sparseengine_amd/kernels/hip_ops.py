@@ -392,6 +392,16 @@ class HipKernels:
             top_k, int(scoring == "softmax"), int(bool(normalize)), float(scaling), _stream()),
             "router_topk")
 
+    def route(self, x, weight, bias, top_k: int, logits, ids, weights, scoring="sigmoid", normalize=True,
+              scaling: float = 1.0, workspace=None):
+        """The whole router: ``logits = x @ weight.T`` in float32, then ``router_topk`` on them.
+        Two launches.  (One launch in which the block that finishes its logits last routes was
+        measured and is not faster on this chip: making the logits visible across the chip's eight
+        L2 caches, the count and the barriers cost about 4.5 us, more than a kernel's boundary.)"""
+        self.router_logits(x, weight, logits)
+        self.router_topk(logits, bias, top_k, ids, weights, scoring=scoring, normalize=normalize,
+                         scaling=scaling, workspace=workspace)
+
     def moe_align(self, ids, experts: int, ws: MoeWorkspace, tile_rows: int = 16):
         _i32(ids, "ids")
         assignments = ids.numel()

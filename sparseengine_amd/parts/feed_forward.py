@@ -68,13 +68,13 @@ class RoutedExperts(Part):
 
     def _forward_chunk(self, fb, x, out):
         s, p, T = self.spec, self.params, x.shape[0]
-        logits = fb.kernels.router_logits(x, p["router"], fb.buffer("moe.logits", (T, s.num_experts), torch.float32))
+        logits = fb.buffer("moe.logits", (T, s.num_experts), torch.float32)
         ids = fb.buffer("moe.ids", (T, s.top_k), torch.int32)
         weights = fb.buffer("moe.weights", (T, s.top_k), torch.float32)
         w13, w2 = p["w13"], p["w2"]
         ws = self._workspace_for(fb, T, w13.dtype)
-        fb.kernels.router_topk(logits, p.get("router_bias"), s.top_k, ids, weights, scoring=s.scoring,
-                               normalize=s.norm_topk_prob, scaling=s.routed_scaling_factor, workspace=ws)
+        fb.kernels.route(x, p["router"], p.get("router_bias"), s.top_k, logits, ids, weights, scoring=s.scoring,
+                         normalize=s.norm_topk_prob, scaling=s.routed_scaling_factor, workspace=ws)
         if fb.taps is not None:
             fb.taps.setdefault("router", []).append((ids.clone(), weights.clone()))
         if w13.dtype == x.dtype:

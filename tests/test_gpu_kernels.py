@@ -290,6 +290,37 @@ def test_router_with_grouping_in_one_launch(hip, tokens, experts, k):
     assert torch.equal(out_a, out_b)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,experts,k,hidden", [(1, 256, 8, 3072), (2, 256, 8, 3072), (3, 64, 6, 512), (8, 256, 8, 3072),
+                                                      (16, 256, 8, 1024), (5, 7, 3, 200), (13, 1000, 16, 264), (3, 1, 1, 8)])
+def test_whole_router(hip, dtype, tokens, experts, k, hidden):
+    """``route`` gives what logits, routing and grouping give one by one, call after call on one workspace."""
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    w = randn(experts, hidden, dtype=torch.float32, scale=3 * hidden ** -0.5, seed=40 + tokens)
+    bias = randn(experts, dtype=torch.float32, scale=0.1, seed=41)
+    ws_a = MoeWorkspace(16, k, experts, 128, 128, torch.bfloat16, "cuda")
+    ws_b = MoeWorkspace(16, k, experts, 128, 128, torch.bfloat16, "cuda")
+    for call in range(3):
+        wide = randn(tokens, hidden + 8, dtype=dtype, seed=50 + call)
+        x = wide[:, :hidden] if call == 1 else wide[:, :hidden].contiguous()     # also a view with a row stride
+        logits_a = torch.empty(tokens, experts, dtype=torch.float32, device="cuda")
+        logits_b = torch.full_like(logits_a, float("nan"))
+        ids_a = torch.empty(tokens, k, dtype=torch.int32, device="cuda"); w_a = torch.empty(tokens, k, device="cuda")
+        ids_b = torch.full_like(ids_a, -1); w_b = torch.full_like(w_a, float("nan"))
+        hip.router_logits(x, w, logits_a)
+        hip.router_topk(logits_a, bias, k, ids_a, w_a)
+        tiles_a = hip.moe_align(ids_a, experts, ws_a, 16)
+        hip.route(x, w, bias, k, logits_b, ids_b, w_b, workspace=ws_b)
+        assert ws_b.grouped is not None and ws_b.grouped[5] == tiles_a
+        torch.testing.assert_close(logits_b, (x.double() @ w.double().T).float(), rtol=1e-5, atol=1e-5)
+        assert torch.equal(logits_a, logits_b) and torch.equal(ids_a, ids_b) and torch.equal(w_a, w_b)
+        assert torch.equal(ws_a.counters, ws_b.counters)
+        n_tiles, n_sorted = ws_a.counters.tolist()
+        assert torch.equal(ws_a.tile_expert[:n_tiles], ws_b.tile_expert[:n_tiles])
+        sa, sb = ws_a.sorted[:n_sorted].view(n_tiles, 16), ws_b.sorted[:n_sorted].view(n_tiles, 16)
+        assert torch.equal(sa.sort(-1).values, sb.sort(-1).values)
+
+
 def test_router_ties_nonfinite_and_bias(hip, twin):
     # tie order and non-finite rows as in the reference's tests/test_minimax_m2_router.py:68-122
     logits = torch.zeros(4, 256).cuda()

@@ -122,6 +122,11 @@ class TwinKernels:
         ids.copy_(out_ids.to(torch.int32))
         weights.copy_(w * scaling)
 
+    def route(self, x, weight, bias, top_k, logits, ids, weights, scoring="sigmoid", normalize=True, scaling=1.0,
+              workspace=None):
+        self.router_logits(x, weight, logits)
+        self.router_topk(logits, bias, top_k, ids, weights, scoring=scoring, normalize=normalize, scaling=scaling)
+
     def moe_experts(self, x, w13, w2, ids, weights, out, ws=None):
         dt = x.dtype
         T, h = x.shape
