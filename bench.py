@@ -143,6 +143,14 @@ def main() -> int:
         runner.release(f"p{i}")
     prefill_s = min(times[1:])
     T = PROMPT_LEN
+    prefill_bytes = None
+    if not args.no_prefill:     # untimed: the experts the prompt touches, layer by layer, are what it has to read
+        taps = {}
+        runner.step([StepEntry("p_taps", prompt(), [PROMPT_LEN - 1])], taps=taps)
+        runner.release("p_taps")
+        touched = [int(torch.unique(i).numel()) for i, _ in taps["router"]]
+        prefill_bytes = L * dense_layer + sum(touched) * expert_bytes + V * h * itemsize
+        del taps
     prefill_flops = L * (2 * T * h * (H + 2 * Hkv) * D + 2 * T * H * D * h + 2 * T * h * E + 2 * T * K * 3 * I * h
                          + 4 * H * D * T * (T + 1) / 2) + 2 * V * h
     peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
@@ -190,7 +198,9 @@ def main() -> int:
                    "num_local_experts": E, "num_experts_per_tok": K, "intermediate_size": I, "vocab_size": V,
                    "kv_page_size": 64, "kv_cache_tokens": args.kv_requests * CONTEXT_LEN, "parallelism": "single GPU"},
         "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
-                    "frac": round(prefill_flops / prefill_s / peak, 5)},
+                    "frac": round(prefill_flops / prefill_s / peak, 5),
+                    # a 2048-token step reads every expert it touches for a few dozen rows each: memory bound too
+                    "hbm_frac": None if prefill_bytes is None else round(prefill_bytes / prefill_s / HBM_PEAK, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,

@@ -447,7 +447,8 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 // tokens (gate-up + down): four wavefronts of 64 x 128 and steps of 64, one block per CU: 6.2 ms;
 // eight wavefronts: 5.9 (LDS reads issue at 220 instead of 120 bytes a clock); steps of 32 and two
 // blocks per CU: 5.1.
-//   MODE 0: out[a, n0 + 32 wc + 16 cb + ...] from gate rows n0 + 32 wc ..., up rows N + n0 + 32 wc ...
+//   MODE 0: columns n0 + 32 wc + 16 cb + ... from gate rows n0 + 32 wc ..., up rows N + n0 + 32 wc ...; the result
+//           lies in operand tiles by sorted position (see the epilogue), which MODE 1 reads as its activations
 //   MODE 1: out[a, n0 + 64 wc + 16 cb + ...] * route_weight[a]
 // Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1); tiles of 128 sorted rows (BM = 64:
 // four wavefronts on 64 rows, measured equal to the tall kernel where that one is used).
@@ -510,10 +511,16 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     const int p = wave * PAIRS + j;
     if (p < 16) {     // a tile of 16 rows x 32 k is 512 elements in the order of the lanes; the next 32 k follow it
       src[j] = we + (weight_row(p) / 16) * (K / 32) * 512 + lane * 8;
-    } else {
+    } else if (MODE == 0) {
       const int a = rows[(p - 16) * 16 + col];
-      const int64_t token = a < assignments ? static_cast<int64_t>(MODE == 0 ? a / top_k : a) : 0;  // padding reads row 0
+      const int64_t token = a < assignments ? static_cast<int64_t>(a / top_k) : 0;  // padding reads row 0
       src[j] = in + token * K + kgroup * 8;
+    } else {
+      // the gate-up launch has left its output in tiles by sorted position (below): row block p - 16
+      // of this tile, like a weight row block.  (Gathering the gate-up launch's rows into such tiles
+      // first was measured too: the extra pass costs more than it saves below 8192 tokens, and
+      // saves 2 % from there on.)
+      src[j] = in + (static_cast<int64_t>(tile) * (BM / 16) + (p - 16)) * (K / 32) * 512 + lane * 8;
     }
   }
   const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(wide_shared));
@@ -523,10 +530,10 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     const int k0 = step * KSTEP;
 #pragma unroll
     for (int j = 0; j < PAIRS; ++j) {
-      const bool weights = wave * PAIRS + j < 16;      // the same for all lanes
-      const bf16_t* first = weights ? src[j] + static_cast<int64_t>(k0) * 16 : src[j] + k0;
+      const bool tiles = MODE == 1 || wave * PAIRS + j < 16;      // the same for all lanes
+      const bf16_t* first = tiles ? src[j] + static_cast<int64_t>(k0) * 16 : src[j] + k0;
       load16_to_lds(first, dst + static_cast<uint32_t>(HALVES * j) * 1024u);
-      if (HALVES == 2) load16_to_lds(first + (weights ? 512 : 32), dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
+      if (HALVES == 2) load16_to_lds(first + (tiles ? 512 : 32), dst + static_cast<uint32_t>(2 * j + 1) * 1024u);
     }
   };
 
@@ -568,7 +575,6 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     }
     asm volatile("" ::: "memory");
   }
-
   // lane (kgroup, col): acc[cb][mb][i] belongs to weight row 4 * kgroup + i of block cb, tile row 64 wr + 16 mb + col
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
@@ -576,6 +582,12 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     if (a >= assignments) continue;
     bf16_t* o_row = out + static_cast<int64_t>(a) * N + n0 + 4 * kgroup;
     if (MODE == 0) {
+      // The result is the down launch's activation operand.  It is written in tiles of 16 sorted
+      // rows x 32 columns, each 1 KB in the order of the lanes that will hold it ([column / 8][row]
+      // [column % 8], like the expert tables), tile (sorted row block, column / 32): the down launch
+      // then loads it as contiguous kilobytes instead of 64 bytes from each of 16 rows.  Rows of
+      // padding are not written; what the down launch computes from them is not stored.
+      bf16_t* t_row = out + (static_cast<int64_t>(tile) * (BM / 16) + 4 * wr + mb) * (N / 32) * 512 + col * 8;
 #pragma unroll
       for (int cb = 0; cb < CB / 2; ++cb) {
         uint16_t y[4];
@@ -589,7 +601,8 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
         uint2 packed;
         packed.x = static_cast<uint32_t>(y[0]) | (static_cast<uint32_t>(y[1]) << 16);
         packed.y = static_cast<uint32_t>(y[2]) | (static_cast<uint32_t>(y[3]) << 16);
-        *reinterpret_cast<uint2*>(o_row + (8 * CB) * wc + 16 * cb) = packed;
+        const int n = n0 + (8 * CB) * wc + 16 * cb + 4 * kgroup;    // first of the lane's four columns
+        *reinterpret_cast<uint2*>(t_row + static_cast<int64_t>(n / 32) * 512 + ((n % 32) / 8) * 128 + n % 8) = packed;
       }
     } else {
       const float rw = route_weight[a];

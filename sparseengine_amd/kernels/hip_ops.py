@@ -163,7 +163,8 @@ class MoeWorkspace:
         self.tile_expert = torch.empty(max_tiles, dtype=torch.int32, device=device)
         self.counters = torch.zeros(2, dtype=torch.int32, device=device)
         self.grouped = None      # set by router_topk when its launch has grouped the assignments already
-        self.act = torch.empty(assignments, intermediate, dtype=dtype, device=device)
+        # rows by assignment, or (the direct kernel) by sorted position, padding included
+        self.act = torch.empty(capacity, intermediate, dtype=dtype, device=device)
         self.slot_out = torch.empty(assignments, hidden, dtype=dtype, device=device)
 
     def fits(self, tokens, top_k, experts, hidden, intermediate, dtype) -> bool:
