@@ -138,7 +138,7 @@ router_logits_kernel(const T* __restrict__ x, int64_t x_stride, const float* __r
   constexpr int XV = 8 / Vec16<T>::N;            // 16-byte vectors of 8 activations
   // steps of 512 along K whose loads go out together: with one token the product is a chain of
   // memory round trips otherwise (measured at 256 x 3072: 5.8 -> 4.7 us)
-  constexpr int UNROLL = TG <= 2 ? 8 : (TG == 4 ? 4 : 2);
+  constexpr int UNROLL = TG <= 2 ? 8 : (TG == 4 ? 6 : 3);
   const float* w_row = w + static_cast<int64_t>(expert) * K;
   for (int t0 = 0; t0 < tokens; t0 += TG) {
     float acc[TG];
