@@ -27,12 +27,16 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
 
-// round to nearest even, NaN kept quiet (same rule as the framework's tensor library)
+// Two floats to two bfloat16, round to nearest even (the rule of the framework's tensor library;
+// NaN stays a quiet NaN): the chip's own conversion, one instruction, where doing the same with
+// integer arithmetic takes eight and made the norm and rotation kernels arithmetic-bound.
+typedef __bf16 se_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float se_floatx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t floats_to_bf16x2_bits(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(se_floatx2{lo, hi}, se_bf16x2));
+}
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return static_cast<uint16_t>(floats_to_bf16x2_bits(f, 0.f));
 }
 
 __device__ __forceinline__ float to_float(float v) { return v; }
@@ -55,6 +59,10 @@ __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
 template <typename T>
 __device__ __forceinline__ float round_to(float v) {
   return to_float(from_float<T>(v));
+}
+template <>
+__device__ __forceinline__ float round_to<bf16_t>(float v) {
+  return __uint_as_float(floats_to_bf16x2_bits(0.f, v) & 0xffff0000u);   // the upper half is v's bfloat16
 }
 
 // Exchange steps of a reduction over the 64 lanes of a wavefront, all inside the vector unit:
