@@ -75,6 +75,8 @@ rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* ou
       if (rr) rv[i].v = *reinterpret_cast<const decltype(rv[i].v)*>(rr + idx * VN);
     }
   }
+  // the sums stay in registers (a thread's own vectors are all it needs after the reduction)
+  float val[MAXV][VN];
   float sq = 0.f;
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
@@ -84,7 +86,7 @@ rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* ou
       for (int j = 0; j < VN; ++j) {
         float v = xv[i].get(j);
         if (rr) v += rv[i].get(j);
-        row_cache[idx * VN + j] = v;
+        val[i][j] = v;
         sq += v * v;
       }
     }
@@ -109,7 +111,7 @@ rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* ou
       Vec16<T> ov, sv;
 #pragma unroll
       for (int j = 0; j < VN; ++j) {
-        const float v = row_cache[idx * VN + j];
+        const float v = val[i][j];
         sv.set(j, v);
         ov.set(j, v * inv * wv[i][j / WN].get(j % WN));
       }
