@@ -400,6 +400,37 @@ __global__ void moe_sum_kernel(const T* __restrict__ y, T* __restrict__ out, int
   out[t * hidden + c] = from_float<T>(acc);
 }
 
+// The same with 16-byte vectors (hidden a multiple of the vector length, 16-byte aligned rows): a
+// thread owns one vector of the output row and asks for up to eight slots' vectors at once.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_sum_vec_kernel(const T* __restrict__ y, T* __restrict__ out, int top_k, int hidden) {
+  constexpr int VN = Vec16<T>::N;
+  typedef decltype(Vec16<T>().v) raw_t;
+  const int64_t t = blockIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VN;
+  if (c >= hidden) return;
+  float acc[VN];
+#pragma unroll
+  for (int j = 0; j < VN; ++j) acc[j] = 0.f;
+  for (int k0 = 0; k0 < top_k; k0 += 8) {
+    Vec16<T> v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (k0 + i < top_k) v[i].v = *reinterpret_cast<const raw_t*>(y + (t * top_k + k0 + i) * hidden + c);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (k0 + i < top_k) {   // slot order, as in the scalar kernel
+#pragma unroll
+        for (int j = 0; j < VN; ++j) acc[j] += v[i].get(j);
+      }
+  }
+  Vec16<T> o;
+#pragma unroll
+  for (int j = 0; j < VN; ++j) o.set(j, acc[j]);
+  *reinterpret_cast<raw_t*>(out + t * hidden + c) = o.v;
+}
+
 // out[t, c] = silu(x[t, c]) * x[t, width + c] with the roundings of the fused expert path
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ out, int width) {
@@ -516,6 +547,19 @@ int se_moe_sum(const void* y, void* out, int tokens, int top_k, int hidden, int 
                hipStream_t stream) {
   if (tokens <= 0) return SE_OK;
   if (hidden <= 0) return SE_ERR_SHAPE;
+  const int vn = dtype == SE_F32 ? 4 : 8;
+  const bool aligned = (reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(out)) % 16 == 0;
+  if (hidden % vn == 0 && aligned) {
+    dim3 vgrid(tokens, (hidden / vn + 255) / 256);
+    if (dtype == SE_F32)
+      moe_sum_vec_kernel<float><<<vgrid, 256, 0, stream>>>(static_cast<const float*>(y),
+                                                           static_cast<float*>(out), top_k, hidden);
+    else
+      moe_sum_vec_kernel<bf16_t><<<vgrid, 256, 0, stream>>>(static_cast<const bf16_t*>(y),
+                                                            static_cast<bf16_t*>(out), top_k, hidden);
+    SE_CHECK_LAUNCH();
+    return SE_OK;
+  }
   dim3 grid(tokens, (hidden + 255) / 256);
   if (dtype == SE_F32)
     moe_sum_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(y),
