@@ -248,16 +248,22 @@ __device__ __forceinline__ void align_assignments(const int32_t* __restrict__ id
   }
   __syncthreads();
   for (int e = threadIdx.x; e < experts; e += blockDim.x) cursor[e] = offsets[e];
-  // Padding entries and the tiles' experts: a wavefront per run, its lanes side by side.  (With a
-  // thread per run, one thread writes up to tile_rows - 1 padding entries in a row: 18 us for 64
-  // tokens on tiles of 128.)
-  {
+  // Padding entries and the tiles' experts.  Large tiles, many wavefronts: a wavefront per run, its
+  // lanes side by side (a thread per run would write up to tile_rows - 1 padding entries in a row:
+  // 18 us for 64 tokens on tiles of 128).  Small tiles or a narrow block (the router's own launch
+  // for a few tokens): a thread per run, since most runs are empty and a run has few entries.
+  if (tile_rows > 32 && blockDim.x >= 4 * SE_WAVE) {
     const int lane = threadIdx.x & (SE_WAVE - 1);
     const int waves = blockDim.x / SE_WAVE;
     for (int e = threadIdx.x / SE_WAVE; e < experts; e += waves) {
       const int begin = offsets[e], end = offsets[e + 1];
       for (int p = begin + counts[e] + lane; p < end; p += SE_WAVE) sorted[p] = assignments;
       for (int t = begin / tile_rows + lane; t < end / tile_rows; t += SE_WAVE) tile_expert[t] = e;
+    }
+  } else {
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+      for (int p = offsets[e] + counts[e]; p < offsets[e + 1]; ++p) sorted[p] = assignments;
+      for (int t = offsets[e] / tile_rows; t < offsets[e + 1] / tile_rows; ++t) tile_expert[t] = e;
     }
   }
   __syncthreads();
