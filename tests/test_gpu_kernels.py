@@ -560,6 +560,30 @@ def test_skinny_linear(hip, rows, n, k):
     torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1.6e-2)
 
 
+def test_rounding_to_bfloat16_is_to_nearest_even(hip):
+    """The kernels round float results to bfloat16 with the chip's conversion instruction: it has to
+    give what the tensor library gives, ties (to even), overflow to infinity and infinities included.
+    Products of two bfloat16 numbers are exact in float and have up to 16 significant bits, so a
+    product with one non-zero term shows the rounding of the result alone."""
+    g = torch.Generator().manual_seed(9)
+    rows, n, k = 16, 512, 128
+    a = torch.randn(rows, generator=g).bfloat16()
+    b = torch.randn(n, generator=g).bfloat16()
+    # ties: (1 + 2^-7) * (1 + 2^-1) = 1.5 + 2^-7 + 2^-8 lies halfway between two bfloat16 numbers, and so
+    # do their neighbours; huge products overflow; an infinite factor stays infinite
+    a[:6] = torch.tensor([1 + 2 ** -7, 1 + 3 * 2 ** -7, -(1 + 2 ** -7), 3e38, float("inf"), 2 ** -120]).bfloat16()
+    b[:6] = torch.tensor([1.5, 1.5, 1.5, 3.0, 1.0, 2 ** -20]).bfloat16()
+    x = torch.zeros(rows, k, dtype=torch.bfloat16); x[:, 0] = a
+    w = torch.zeros(n, k, dtype=torch.bfloat16); w[:, 0] = b
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    hip.linear(x.cuda(), w.cuda(), out)
+    ref = (a.float()[:, None] * b.float()[None, :]).bfloat16()
+    finite = torch.isfinite(ref.float())
+    assert torch.equal(out.cpu()[finite].view(torch.int16), ref[finite].view(torch.int16))
+    assert torch.equal(torch.isinf(out.cpu().float()), torch.isinf(ref.float()))
+    assert torch.equal(torch.isnan(out.cpu().float()), torch.isnan(ref.float()))      # inf * 0 terms
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_cache_pages_beyond_four_gigabytes(hip, twin, dtype):
     """A layer's cache tensor larger than 2^32 bytes and 2^31 elements: the write and both
