@@ -6,7 +6,8 @@ Model: the sizes of MiniMax M2 (hidden 3072, 48 query / 8 kv heads of 128, rotar
 top-8 of width 1536, vocabulary 200064) cut to 16 of its 62 layers, random weights, bfloat16.
 A "step" is one decode step of a batch of 8 requests whose prompts were 2048 random token ids
 (sampling greedily, token ids read back each step).  One JSON line is printed: ``value`` is decoded
-tokens per second at batch 8; ``prefill`` is a 2048-token prompt in one step; ``points`` holds
+tokens per second at batch 8; ``prefill`` is a 2048-token prompt in one step (``frac``: its flops
+against the matrix peak, ``hbm_frac``: the bytes it has to read against 8 TB/s); ``points`` holds
 decode at batch 1 and 64 and the prefill of eight 2048-token prompts in one step; ``roofline``
 prices the batch-8 decode step against 8 TB/s.
 """
