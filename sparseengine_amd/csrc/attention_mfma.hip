@@ -93,11 +93,18 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   const int last_row = (row_tile * 16 + 15 < rows_total) ? row_tile * 16 + 15 : rows_total - 1;
   const int pos_max = ctx_len - q_len + last_row / group;
   if (key_end > pos_max + 1) key_end = pos_max + 1;
+  // With a window the first step of 32 keys may begin before the tile's lowest key, in a page that
+  // the request has given back (its table entry is -1).  No page is looked up and nothing is loaded
+  // for a key below `low_key`: such a key takes the place of `low_key` (its score is masked, so
+  // whatever finite values stand in for it count for nothing).
   int k_first = key_begin;
+  int low_key = 0;
   if (window > 0) {
     const int pos_min = ctx_len - q_len + (row_tile * 16) / group;
     const int lowest = pos_min - window + 1;
     if (lowest > k_first) k_first = lowest & ~31;
+    if (lowest > 0) low_key = lowest;
+    if (key_end <= low_key) key_end = k_first;   // the whole range lies before every row's window
   }
 
   const bf16_t* q_row = q + static_cast<int64_t>(token) * q_stride + static_cast<int64_t>(head) * D + g * 8;
@@ -122,11 +129,13 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   auto page_of_keys = [&](int k0) {     // page of the lane's two key rows (both lie in one group of 8)
     int key = k0 + 8 * (n >> 2);
     if (key > last_key) key = last_key;
+    if (key < low_key) key = low_key;
     return table[key / page_size];
   };
   auto page_of_values = [&](int k0) {   // page of the lane's eight consecutive keys
     int key = k0 + 8 * g;
     if (key > last_key) key = last_key & ~7;
+    if (key + 7 < low_key) key = low_key & ~7;
     return table[key / page_size];
   };
 
@@ -135,6 +144,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     _Pragma("unroll") for (int b = 0; b < 2; ++b) {                                               \
       int key = (K0) + 8 * (n >> 2) + (n & 3) + 4 * b;                                            \
       if (key > last_key) key = last_key; /* reads stay inside the request's pages */            \
+      if (key < low_key) key = low_key;                                                           \
       /* dims 32 ds + 8 g ... of the key: group 4 ds + g of the page's [head_dim / 8][page_size][8] */ \
       const bf16_t* k_row = cache + (static_cast<int64_t>(PK) * 2) * plane + kvh * head_span +    \
                             (static_cast<int64_t>(g) * page_size + key % page_size) * 8;          \
@@ -143,6 +153,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     }                                                                                             \
     int vkey = (K0) + 8 * g;                                                                      \
     if (vkey > last_key) vkey = last_key & ~7;                                                    \
+    if (vkey + 7 < low_key) vkey = low_key & ~7;                                                  \
     /* eight keys of dim 16 db + n: the page's [page_size / 8][head_dim][8] */                     \
     const bf16_t* v_col = cache + (static_cast<int64_t>(PV) * 2 + 1) * plane + kvh * head_span +  \
                           static_cast<int64_t>(vkey % page_size) * D + n * 8;                     \
@@ -191,9 +202,10 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     pf.z = pack_bf16x2(p[4], p[5]);                                                               \
     pf.w = pack_bf16x2(p[6], p[7]);                                                               \
     /* values: lane (g, n) holds value dim db * 16 + n at keys K0 + 8 g .. + 7 */                 \
-    int vkey = (K0) + 8 * g;                                                                      \
-    const bool beyond = vkey + 7 > last_key; /* only in the request's last step */                \
+    int vkey = (K0) + 8 * g; /* clamped as in the load */                                         \
     if (vkey > last_key) vkey = last_key & ~7;                                                    \
+    if (vkey + 7 < low_key) vkey = low_key & ~7;                                                  \
+    const bool beyond = vkey + 7 > last_key; /* the request's last group of eight */              \
     _Pragma("unroll") for (int db = 0; db < DBLOCKS; ++db) {                                      \
       uint4 vf = VF[db];                                                                          \
       if (beyond) vf = zero_keys_beyond(vf, vkey, last_key);                                      \
@@ -399,10 +411,15 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   // the block's rows bound the keys that are loaded; the wave's rows bound what it computes
   const int block_last_row = min((first_tile + 4 * RT) * 16, rows_total) - 1;
   key_end = min(key_end, pos0 + block_last_row / group + 1);
+  // as in the kernel above: nothing is looked up or loaded for a key below `low_key`, whose page the
+  // request may have given back; `low_key` stands in for it
   int k_first = key_begin;
+  int low_key = 0;
   if (window > 0) {
     const int lowest = pos0 + (first_tile * 16) / group - window + 1;
     if (lowest > k_first) k_first = lowest & ~31;
+    if (lowest > 0) low_key = lowest;
+    if (key_end <= low_key) key_end = k_first;   // the whole range lies before every row's window
   }
   const int tile0 = first_tile + wave * RT;
   const bool wave_active = tile0 * 16 < rows_total;
@@ -470,6 +487,9 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   const int lane_key = loads_keys ? 8 * (n >> 2) + (n & 3) + 4 * wave : 8 * g;
   const int clamp_key = loads_keys ? kmax : (kmax & ~7);
   const int clamp_page = clamp_key / page_size, clamp_off = clamp_key % page_size;
+  // a lane's key (values: its group of eight) wholly below `low_key` is replaced by that one's
+  const int low_clamp = loads_keys ? low_key : (low_key & ~7);
+  const int low_page = low_clamp / page_size, low_off = low_clamp % page_size;
   int next_key = k_first + lane_key;                     // the lane's key of the next step to be issued
   int next_page = next_key / page_size, next_off = next_key % page_size;
   // keys lie [head_dim / 8][page_size][8], values [page_size / 8][head_dim][8]: sixteen lanes of a
@@ -481,9 +501,12 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   auto issue = [&](int step) {
     const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS + wave * DSTEPS) * 1024u;
     const bool over = next_key > kmax;
-    const int page = page_ids[(over ? clamp_page : next_page) - window_base];
+    const bool under = next_key < low_clamp;     // only in a unit's first step
+    const int use_page = over ? clamp_page : (under ? low_page : next_page);
+    const int use_off = over ? clamp_off : (under ? low_off : next_off);
+    const int page = page_ids[use_page - window_base];
     const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2) * plane + lane_base +
-                        static_cast<int64_t>(over ? clamp_off : next_off) * off_scale;
+                        static_cast<int64_t>(use_off) * off_scale;
 #pragma unroll
     for (int j = 0; j < DSTEPS; ++j) load16_to_lds(src + j * load_stride, dst + static_cast<uint32_t>(j) * 1024u);
     next_key += 32;
@@ -551,8 +574,9 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
         // of the page left there, possibly not finite.  The loader's clamping is repeated here.
         // Two copies of the loop: folded into one, the masking would be paid in every step.
         if (__builtin_expect(k0 + 31 > kmax, 0)) {
-          int vkey = k0 + 8 * g;
+          int vkey = k0 + 8 * g;      // clamped as the loader clamps it
           if (vkey > kmax) vkey = kmax & ~7;
+          if (vkey < (low_key & ~7)) vkey = low_key & ~7;
 #pragma unroll
           for (int db = 0; db < DBLOCKS; ++db) {
             const uint4 vf = zero_keys_beyond(buf[2 * DSTEPS + db][lane], vkey, last_key);

@@ -37,6 +37,20 @@ def require_true_float32() -> None:
     torch.set_float32_matmul_precision("highest")
 
 
+def kernels_from_environment():
+    """Test seam for the programs (``bin/trace_run``, the command line), which build their engine
+    themselves: ``SPARSEENGINE_AMD_KERNELS=module:factory`` names a stand-in for the HIP kernels that
+    works on CPU tensors (the tests' twins, or their host build of the kernel sources).  Unset,
+    as in every product run, the HIP kernels are the only path."""
+    import importlib
+    import os
+    seam = os.environ.get("SPARSEENGINE_AMD_KERNELS")
+    if not seam:
+        return None
+    module, _, factory = seam.partition(":")
+    return getattr(importlib.import_module(module), factory)()
+
+
 @dataclass
 class StepEntry:
     request_id: object
@@ -52,6 +66,10 @@ class ModelRunner:
         self.dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
         require_true_float32()
+        if kernels is None:
+            kernels = kernels_from_environment()
+            if kernels is not None:
+                self.device = torch.device("cpu")
         if kernels is None:
             from ..kernels.hip_ops import HipKernels      # raises if there is no GPU or no library
             kernels = HipKernels()

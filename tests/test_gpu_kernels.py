@@ -5,22 +5,36 @@ import pytest
 import torch
 
 from sparseengine_amd.cache import layout
+from tests import backends
 from tests.twin_kernels import TwinKernels
 
 pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float32, torch.bfloat16]
+DEV = "cuda"      # where the tensors of a test live: the backend's device (set before every test)
 
 
-@pytest.fixture(scope="module")
+@pytest.fixture(autouse=True)
+def _device():
+    global DEV
+    DEV = backends.ACTIVE.device
+
+
+@pytest.fixture
 def hip():
-    from sparseengine_amd.kernels.hip_ops import HipKernels
-    return HipKernels()
+    return backends.ACTIVE.kernels()
 
 
 @pytest.fixture(scope="module")
 def twin():
     return TwinKernels()
+
+
+def emulator_skips(work: float, limit: float = 3e8):
+    """The emulated backend runs a kernel's threads one after the other: cases whose size says
+    nothing new about indexing are left to the GPU."""
+    if backends.ACTIVE.slow and work > limit:
+        pytest.skip("too large for the emulated backend")
 
 
 def tol(dtype):
@@ -29,15 +43,15 @@ def tol(dtype):
 
 def randn(*shape, dtype, scale=1.0, seed=0):
     g = torch.Generator().manual_seed(seed)
-    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,hidden,vocab", [(1, 64, 50), (37, 3072, 1000), (5, 200, 77)])
 def test_embedding(hip, dtype, tokens, hidden, vocab):
     table = randn(vocab, hidden, dtype=dtype)
-    ids = torch.randint(0, vocab, (tokens,), dtype=torch.int32).cuda()
-    out = torch.empty(tokens, hidden, dtype=dtype, device="cuda")
+    ids = torch.randint(0, vocab, (tokens,), dtype=torch.int32).to(DEV)
+    out = torch.empty(tokens, hidden, dtype=dtype, device=DEV)
     hip.embedding(ids, table, out)
     assert torch.equal(out, table[ids.long()])
 
@@ -49,7 +63,7 @@ def test_rms_norm_plain_and_fused(hip, twin, dtype, wdtype, tokens, hidden):
     wdtype = wdtype or dtype
     x = randn(tokens, hidden, dtype=dtype, seed=1)
     res = randn(tokens, hidden, dtype=dtype, seed=2)
-    w = (1 + 0.2 * torch.randn(hidden)).to(wdtype).cuda()
+    w = (1 + 0.2 * torch.randn(hidden)).to(wdtype).to(DEV)
     # plain
     out_h, out_t = torch.empty_like(x), torch.empty_like(x)
     hip.rms_norm(x, w, 1e-5, out_h)
@@ -63,8 +77,8 @@ def test_rms_norm_plain_and_fused(hip, twin, dtype, wdtype, tokens, hidden):
     assert torch.equal(rh, (x.float() + res.float()).to(dtype))
     torch.testing.assert_close(xh, xt, **tol(dtype))
     # row selection leaves the residual alone
-    rows = torch.tensor([tokens - 1, 0], dtype=torch.int32).cuda()
-    oh = torch.empty(2, hidden, dtype=dtype, device="cuda")
+    rows = torch.tensor([tokens - 1, 0], dtype=torch.int32).to(DEV)
+    oh = torch.empty(2, hidden, dtype=dtype, device=DEV)
     ot = torch.empty_like(oh)
     r_before = res.clone()
     hip.rms_norm(x, w, 1e-5, oh, residual=res, rows=rows)
@@ -75,15 +89,15 @@ def test_rms_norm_plain_and_fused(hip, twin, dtype, wdtype, tokens, hidden):
 
 def test_rms_norm_refuses_wide_rows(hip):
     from sparseengine_amd.kernels.hip_ops import KernelShapeError
-    x = torch.zeros(1, 16384, device="cuda")
+    x = torch.zeros(1, 16384, device=DEV)
     with pytest.raises(KernelShapeError):
-        hip.rms_norm(x, torch.ones(16384, device="cuda"), 1e-6, torch.empty_like(x))
+        hip.rms_norm(x, torch.ones(16384, device=DEV), 1e-6, torch.empty_like(x))
 
 
 def rope_table(max_pos, rotary_dim, theta):
     inv = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
     f = torch.arange(max_pos, dtype=torch.float32)[:, None] * inv[None]
-    return torch.cat((f.cos(), f.sin()), -1).cuda()
+    return torch.cat((f.cos(), f.sin()), -1).to(DEV)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -94,13 +108,13 @@ def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary,
     tokens, pages = 9, 7
     width = (heads + 2 * kv_heads) * head_dim
     qkv = randn(tokens, width, dtype=dtype, seed=3)
-    positions = torch.tensor([0, 1, 17, 127, 1023, 5, 6, 7, 300], dtype=torch.int32).cuda()
-    table = rope_table(2048, rotary, 5e6) if rotary else torch.zeros(1, 1, device="cuda")
-    qw = (1 + 0.1 * torch.randn(heads * head_dim)).to(dtype).cuda() if norm else None
-    kw = (1 + 0.1 * torch.randn(kv_heads * head_dim)).to(dtype).cuda() if norm else None
+    positions = torch.tensor([0, 1, 17, 127, 1023, 5, 6, 7, 300], dtype=torch.int32).to(DEV)
+    table = rope_table(2048, rotary, 5e6) if rotary else torch.zeros(1, 1, device=DEV)
+    qw = (1 + 0.1 * torch.randn(heads * head_dim)).to(dtype).to(DEV) if norm else None
+    kw = (1 + 0.1 * torch.randn(kv_heads * head_dim)).to(dtype).to(DEV) if norm else None
     slots = torch.tensor([3 * page + 1, 0, page - 1, 5 * page, -1, 2 * page + 3, 2 * page + 4, 6 * page + page - 1, page],
-                         dtype=torch.int32).cuda()
-    cache_h = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device="cuda")
+                         dtype=torch.int32).to(DEV)
+    cache_h = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device=DEV)
     cache_t = cache_h.clone()
     a, b = qkv.clone(), qkv.clone()
     hip.qk_norm_rope_store(a, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_h, slots, page)
@@ -117,23 +131,41 @@ def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary,
     for t in range(tokens):
         s = int(slots[t])
         if s >= 0:
-            at = (torch.tensor([s // page]).cuda(), torch.tensor([s % page]).cuda())
+            at = (torch.tensor([s // page]).to(DEV), torch.tensor([s % page]).to(DEV))
             assert torch.equal(layout.read_keys(cache_h, *at)[0], kq[t])
             assert torch.equal(layout.read_values(cache_h, *at)[0], a[t, (heads + kv_heads) * head_dim:].view(kv_heads, head_dim))
 
 
-def make_paged(dtype, kv_heads, head_dim, page, lens, seed=0, extra_pages=3):
-    """Random k/v for requests of the given lengths scattered over shuffled pages."""
+def make_paged(dtype, kv_heads, head_dim, page, lens, seed=0, extra_pages=3, window=0, q_lens=None):
+    """Random k/v for requests of the given lengths scattered over shuffled pages, as the cache
+    manager leaves them: with a window, the pages that lie wholly before the window of a request's
+    first new token (``q_lens`` new tokens each) have been given back, so their table entries are -1;
+    pages that no table names, the given-back ones among them, and the slots past a request's last
+    key hold not-a-number.  A kernel that looks up a page it must not, or reads a slot it must not,
+    shows it in its output (and faults under the emulated backend, whose tables end at a guard page)."""
     g = torch.Generator().manual_seed(seed)
     need = [(n + page - 1) // page for n in lens]
     total = sum(need) + extra_pages
     perm = torch.randperm(total, generator=g).tolist()
-    cache = (torch.randn(total, 2, kv_heads, page, head_dim, generator=g)).to(dtype).cuda()
+    cache = torch.randn(total, 2, kv_heads, page, head_dim, generator=g).to(dtype)
     table = torch.full((len(lens), max(need) + 1), -1, dtype=torch.int32)
+    named = torch.zeros(total, dtype=torch.bool)
     for r, n in enumerate(need):
+        first_live = 0
+        if window and q_lens is not None:
+            first_live = max(0, lens[r] - q_lens[r] - window + 1) // page       # cache/manager.py: _plan
         for j in range(n):
-            table[r, j] = perm.pop()
-    return cache, table.cuda()
+            p = perm.pop()
+            if j >= first_live:
+                table[r, j] = p
+                named[p] = True
+        last, used = int(table[r, n - 1]), lens[r] - (n - 1) * page
+        if used < page:
+            beyond = torch.arange(used, page)
+            layout.keys_view(cache)[last, :, beyond] = float("nan")
+            layout.values_view(cache)[last, :, beyond // 8, beyond % 8] = float("nan")
+    cache[~named] = float("nan")
+    return cache.to(DEV), table.to(DEV)
 
 
 def make_meta(table, ctx_lens, q_lens):
@@ -144,16 +176,16 @@ def make_meta(table, ctx_lens, q_lens):
         token_row += [r] * ql
         positions += list(range(n - ql, n))
     q_start = np.concatenate(([0], np.cumsum(q_lens)[:-1])).astype(np.int32)
-    item_meta = torch.tensor(np.stack([q_start, np.asarray(q_lens), np.asarray(ctx_lens)]), dtype=torch.int32).cuda()
-    return SimpleNamespace(block_table=table, token_row=torch.tensor(token_row, dtype=torch.int32).cuda(),
-                           positions=torch.tensor(positions, dtype=torch.int32).cuda(), item_meta=item_meta,
+    item_meta = torch.tensor(np.stack([q_start, np.asarray(q_lens), np.asarray(ctx_lens)]), dtype=torch.int32).to(DEV)
+    return SimpleNamespace(block_table=table, token_row=torch.tensor(token_row, dtype=torch.int32).to(DEV),
+                           positions=torch.tensor(positions, dtype=torch.int32).to(DEV), item_meta=item_meta,
                            item_q_len=np.asarray(q_lens), item_ctx_len=np.asarray(ctx_lens), work={})
 
 
 def dense_attention(q, cache, table, row, pos, scale, window, page):
     """Reference through the library routine: gather the request's keys, call SDPA for one query."""
     first = max(0, pos - window + 1) if window else 0
-    n = torch.arange(first, pos + 1, device="cuda")
+    n = torch.arange(first, pos + 1, device=DEV)
     pages = table[row, n // page].long()
     k = layout.read_keys(cache, pages, n % page).float().transpose(0, 1)   # [Hkv, n, D]
     v = layout.read_values(cache, pages, n % page).float().transpose(0, 1)
@@ -174,7 +206,7 @@ def test_paged_attention_mixed_batch(hip, twin, dtype, heads, kv_heads, head_dim
     # three requests: a whole prompt, a portion on top of a cached prefix, a single decoded token
     lens = [37, 150, 301]
     q_lens = [37, 23, 1]
-    cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=heads)
+    cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=heads, window=window, q_lens=q_lens)
     token_row, positions = [], []
     for r, (n, ql) in enumerate(zip(lens, q_lens)):
         token_row += [r] * ql
@@ -184,7 +216,7 @@ def test_paged_attention_mixed_batch(hip, twin, dtype, heads, kv_heads, head_dim
     qkv = randn(T, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=9)
     q = qkv[:, :heads * head_dim].view(T, heads, head_dim)
     scale = head_dim ** -0.5
-    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device="cuda")
+    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device=DEV)
     out_t = torch.empty_like(out_h)
     hip.paged_attention(q, cache, meta, out_h, scale, window)
     twin.paged_attention(q, cache, meta, out_t, scale, window)
@@ -211,7 +243,7 @@ def test_paged_attention_finds_one_far_key(hip, dtype):
             qh = q[0, kvh * (heads // kv_heads)].float()
             layout.keys_view(c)[pg, kvh, off] = (qh / qh.norm() * 60).to(dtype).view(-1, 8)
         meta = make_meta(table, [n], [1])
-        out = torch.empty(1, heads * head_dim, dtype=dtype, device="cuda")
+        out = torch.empty(1, heads * head_dim, dtype=dtype, device=DEV)
         hip.paged_attention(q, c, meta, out, 1.0, 0)
         for kvh in range(kv_heads):
             head = kvh * (heads // kv_heads)
@@ -226,7 +258,7 @@ def test_router_logits_are_float_products(hip, dtype, tokens, experts, k):
     """Few tokens take the small kernel (activations widened on the fly), more the library."""
     x = randn(tokens, k, dtype=dtype, seed=3)
     w = randn(experts, k, dtype=torch.float32, scale=k ** -0.5, seed=4)
-    out = torch.empty(tokens, experts, dtype=torch.float32, device="cuda")
+    out = torch.empty(tokens, experts, dtype=torch.float32, device=DEV)
     hip.router_logits(x, w, out)
     ref = (x.double() @ w.double().T).float()
     torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
@@ -239,10 +271,10 @@ def test_router_logits_are_float_products(hip, dtype, tokens, experts, k):
 def test_router_matches_library_topk(hip, twin):
     torch.manual_seed(27)
     for tokens, experts, k in [(4096, 256, 8), (33, 8, 2), (17, 16, 4), (5, 100, 7), (3, 1, 1), (9, 1000, 16)]:
-        logits = (torch.randn(tokens, experts) * 3).cuda()
-        bias = (torch.randn(experts) * 0.1).cuda()
-        ids = torch.empty(tokens, k, dtype=torch.int32, device="cuda")
-        w = torch.empty(tokens, k, device="cuda")
+        logits = (torch.randn(tokens, experts) * 3).to(DEV)
+        bias = (torch.randn(experts) * 0.1).to(DEV)
+        ids = torch.empty(tokens, k, dtype=torch.int32, device=DEV)
+        w = torch.empty(tokens, k, device=DEV)
         hip.router_topk(logits, bias, k, ids, w)
         s = torch.sigmoid(logits)
         ref_ids = torch.topk(s + bias, k, dim=-1).indices
@@ -260,12 +292,12 @@ def test_router_with_grouping_in_one_launch(hip, tokens, experts, k):
     """Few tokens: routing and grouping in one launch give what the two launches give."""
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     torch.manual_seed(tokens + experts)
-    logits = (torch.randn(tokens, experts) * 3).cuda()
-    bias = (torch.randn(experts) * 0.1).cuda()
-    ids_a = torch.empty(tokens, k, dtype=torch.int32, device="cuda"); w_a = torch.empty(tokens, k, device="cuda")
+    logits = (torch.randn(tokens, experts) * 3).to(DEV)
+    bias = (torch.randn(experts) * 0.1).to(DEV)
+    ids_a = torch.empty(tokens, k, dtype=torch.int32, device=DEV); w_a = torch.empty(tokens, k, device=DEV)
     ids_b = torch.empty_like(ids_a); w_b = torch.empty_like(w_a)
-    ws_a = MoeWorkspace(tokens, k, experts, 128, 128, torch.bfloat16, "cuda")
-    ws_b = MoeWorkspace(tokens, k, experts, 128, 128, torch.bfloat16, "cuda")
+    ws_a = MoeWorkspace(tokens, k, experts, 128, 128, torch.bfloat16, DEV)
+    ws_b = MoeWorkspace(tokens, k, experts, 128, 128, torch.bfloat16, DEV)
     hip.router_topk(logits, bias, k, ids_a, w_a)
     tiles_a = hip.moe_align(ids_a, experts, ws_a, 16)
     hip.router_topk(logits, bias, k, ids_b, w_b, workspace=ws_b)
@@ -298,14 +330,14 @@ def test_whole_router(hip, dtype, tokens, experts, k, hidden):
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     w = randn(experts, hidden, dtype=torch.float32, scale=3 * hidden ** -0.5, seed=40 + tokens)
     bias = randn(experts, dtype=torch.float32, scale=0.1, seed=41)
-    ws_a = MoeWorkspace(16, k, experts, 128, 128, torch.bfloat16, "cuda")
-    ws_b = MoeWorkspace(16, k, experts, 128, 128, torch.bfloat16, "cuda")
+    ws_a = MoeWorkspace(16, k, experts, 128, 128, torch.bfloat16, DEV)
+    ws_b = MoeWorkspace(16, k, experts, 128, 128, torch.bfloat16, DEV)
     for call in range(3):
         wide = randn(tokens, hidden + 8, dtype=dtype, seed=50 + call)
         x = wide[:, :hidden] if call == 1 else wide[:, :hidden].contiguous()     # also a view with a row stride
-        logits_a = torch.empty(tokens, experts, dtype=torch.float32, device="cuda")
+        logits_a = torch.empty(tokens, experts, dtype=torch.float32, device=DEV)
         logits_b = torch.full_like(logits_a, float("nan"))
-        ids_a = torch.empty(tokens, k, dtype=torch.int32, device="cuda"); w_a = torch.empty(tokens, k, device="cuda")
+        ids_a = torch.empty(tokens, k, dtype=torch.int32, device=DEV); w_a = torch.empty(tokens, k, device=DEV)
         ids_b = torch.full_like(ids_a, -1); w_b = torch.full_like(w_a, float("nan"))
         hip.router_logits(x, w, logits_a)
         hip.router_topk(logits_a, bias, k, ids_a, w_a)
@@ -323,12 +355,12 @@ def test_whole_router(hip, dtype, tokens, experts, k, hidden):
 
 def test_router_ties_nonfinite_and_bias(hip, twin):
     # tie order and non-finite rows as in the reference's tests/test_minimax_m2_router.py:68-122
-    logits = torch.zeros(4, 256).cuda()
+    logits = torch.zeros(4, 256).to(DEV)
     logits[1, :9] = 1
     logits[2, 120:129] = 1
-    logits[3] = (torch.arange(256).cuda() // 8).float()
-    bias = torch.zeros(256).cuda()
-    ids = torch.empty(4, 8, dtype=torch.int32, device="cuda"); w = torch.empty(4, 8, device="cuda")
+    logits[3] = (torch.arange(256).to(DEV) // 8).float()
+    bias = torch.zeros(256).to(DEV)
+    ids = torch.empty(4, 8, dtype=torch.int32, device=DEV); w = torch.empty(4, 8, device=DEV)
     hip.router_topk(logits, bias, 8, ids, w)
     assert ids[0].tolist() == list(range(8))
     assert ids[1].tolist() == list(range(8))
@@ -336,28 +368,28 @@ def test_router_ties_nonfinite_and_bias(hip, twin):
     s3 = torch.sigmoid(logits[3])   # saturates to 1.0 from index 136 on: the ties go to the lowest indices
     assert ids[3].tolist() == torch.nonzero(s3 == s3.max()).flatten()[:8].tolist()
     torch.testing.assert_close(w, torch.full_like(w, 0.125))
-    logits = torch.zeros(6, 256).cuda()
+    logits = torch.zeros(6, 256).to(DEV)
     logits[0, 3] = float("nan"); logits[1, 7] = float("inf"); logits[2, 9] = -float("inf")
     logits[3] = 100; logits[4] = -100
     bias2 = bias.clone(); bias2[5] = float("nan")
-    hip.router_topk(logits[:5], bias, 8, ids := torch.empty(5, 8, dtype=torch.int32, device="cuda"),
-                    w := torch.empty(5, 8, device="cuda"))
+    hip.router_topk(logits[:5], bias, 8, ids := torch.empty(5, 8, dtype=torch.int32, device=DEV),
+                    w := torch.empty(5, 8, device=DEV))
     assert 3 in ids[0].tolist() and torch.isnan(w[0]).all()
     assert 7 in ids[1].tolist() and 9 not in ids[2].tolist()
     assert ids[3].tolist() == list(range(8)) and ids[4].tolist() == list(range(8))
-    hip.router_topk(logits[5:], bias2, 8, ids6 := torch.empty(1, 8, dtype=torch.int32, device="cuda"),
-                    w6 := torch.empty(1, 8, device="cuda"))
+    hip.router_topk(logits[5:], bias2, 8, ids6 := torch.empty(1, 8, dtype=torch.int32, device=DEV),
+                    w6 := torch.empty(1, 8, device=DEV))
     assert ids6[0].tolist() == [5, 0, 1, 2, 3, 4, 6, 7]
     # a bias of +2 on experts 0..7 selects exactly them and leaves the weights unbiased
-    logits = torch.linspace(-4, 4, 256)[None].cuda()
-    bias3 = torch.zeros(256).cuda(); bias3[:8] = 2
+    logits = torch.linspace(-4, 4, 256)[None].to(DEV)
+    bias3 = torch.zeros(256).to(DEV); bias3[:8] = 2
     hip.router_topk(logits, bias3, 8, ids6, w6)
     assert sorted(ids6[0].tolist()) == list(range(8))
     s = torch.sigmoid(logits[0, :8])
     torch.testing.assert_close(w6[0].sort().values, (s / s.sum()).sort().values)
     # softmax scoring, no renormalisation, scaling
-    logits = torch.randn(7, 40).cuda()
-    ids7 = torch.empty(7, 3, dtype=torch.int32, device="cuda"); w7 = torch.empty(7, 3, device="cuda")
+    logits = torch.randn(7, 40).to(DEV)
+    ids7 = torch.empty(7, 3, dtype=torch.int32, device=DEV); w7 = torch.empty(7, 3, device=DEV)
     hip.router_topk(logits, None, 3, ids7, w7, scoring="softmax", normalize=False, scaling=2.5)
     ref = torch.topk(torch.softmax(logits, -1), 3)
     assert torch.equal(ids7.long().sort(-1).values, ref.indices.sort(-1).values)
@@ -367,8 +399,8 @@ def test_router_ties_nonfinite_and_bias(hip, twin):
 def test_moe_align_groups_every_assignment_once(hip):
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     for tokens, k, experts in [(1, 8, 256), (2048, 8, 256), (33, 2, 8), (100, 4, 16), (7, 1, 1)]:
-        ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
-        ws = MoeWorkspace(tokens, k, experts, 16, 16, torch.float32, "cuda")
+        ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).to(DEV)
+        ws = MoeWorkspace(tokens, k, experts, 16, 16, torch.float32, DEV)
         for rows in (16, 32, 64):
             ws.sorted.fill_(-7); ws.tile_expert.fill_(-7)
             hip.moe_align(ids, experts, ws, rows)
@@ -395,14 +427,15 @@ def test_moe_align_groups_every_assignment_once(hip):
     # hundreds of rows per expert: tiles of 128 rows x 256 weight rows
     (2048, 256, 128, 8, 8), (1000, 512, 384, 6, 3), (777, 768, 256, 3, 1)])
 def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
+    emulator_skips(tokens * k * hidden * inter, 1.2e9)
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     x = randn(tokens, hidden, dtype=dtype, seed=11)
     w13 = randn(experts, 2 * inter, hidden, dtype=dtype, scale=hidden ** -0.5, seed=12)
     w2 = randn(experts, hidden, inter, dtype=dtype, scale=inter ** -0.5, seed=13)
-    ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
-    weights = torch.rand(tokens, k).cuda()
+    ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).to(DEV)
+    weights = torch.rand(tokens, k).to(DEV)
     weights = weights / weights.sum(-1, keepdim=True)
-    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, DEV)
     out_h = torch.empty_like(x); out_t = torch.empty_like(x)
     hip.moe_experts(x, w13, w2, ids, weights, out_h, ws)
     twin.moe_experts(x, w13, w2, ids, weights, out_t)
@@ -422,7 +455,7 @@ def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_silu_mul(hip, twin, dtype):
     x = randn(13, 2 * 72, dtype=dtype, seed=4)
-    a = torch.empty(13, 72, dtype=dtype, device="cuda"); b = torch.empty_like(a)
+    a = torch.empty(13, 72, dtype=dtype, device=DEV); b = torch.empty_like(a)
     hip.silu_mul(x, a); twin.silu_mul(x, b)
     torch.testing.assert_close(a, b, **tol(dtype))
     torch.testing.assert_close(a.float(), torch.nn.functional.silu(x[:, :72].float()) * x[:, 72:].float(), **tol(dtype))
@@ -431,56 +464,57 @@ def test_silu_mul(hip, twin, dtype):
 def test_sampling(hip, twin):
     torch.manual_seed(3)
     rows, vocab = 6, 1000
-    logits = (torch.randn(rows, vocab) * 2).cuda()
-    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    logits = (torch.randn(rows, vocab) * 2).to(DEV)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
     # greedy, top_k = 1 and a tiny top_p all give the arg-max (reference tests/test_sampler.py:39-58)
     hip.sample(logits, None, None, None, None, out)
     assert torch.equal(out.long(), logits.argmax(-1))
-    temp = torch.full((rows,), 0.7).cuda()
-    seeds = torch.arange(rows, dtype=torch.int64).cuda() * 7919 + 1
-    hip.sample(logits, temp, torch.ones(rows, dtype=torch.int32).cuda(), None, seeds, out)
+    temp = torch.full((rows,), 0.7).to(DEV)
+    seeds = torch.arange(rows, dtype=torch.int64).to(DEV) * 7919 + 1
+    hip.sample(logits, temp, torch.ones(rows, dtype=torch.int32).to(DEV), None, seeds, out)
     assert torch.equal(out.long(), logits.argmax(-1))
-    hip.sample(logits, temp, None, torch.full((rows,), 0.01).cuda(), seeds, out)
+    hip.sample(logits, temp, None, torch.full((rows,), 0.01).to(DEV), seeds, out)
     assert torch.equal(out.long(), logits.argmax(-1))
     # mixed rows against the twin: same noise, same choice
-    temp = torch.tensor([0.0, 0.8, 1.0, 0.7, 1.3, 0.5]).cuda()
-    top_k = torch.tensor([0, 0, 5, 0, 50, 3], dtype=torch.int32).cuda()
-    top_p = torch.tensor([1.0, 1.0, 1.0, 0.6, 0.9, 0.5]).cuda()
+    temp = torch.tensor([0.0, 0.8, 1.0, 0.7, 1.3, 0.5]).to(DEV)
+    top_k = torch.tensor([0, 0, 5, 0, 50, 3], dtype=torch.int32).to(DEV)
+    top_p = torch.tensor([1.0, 1.0, 1.0, 0.6, 0.9, 0.5]).to(DEV)
     ref = torch.empty_like(out)
     hip.sample(logits, temp, top_k, top_p, seeds, out)
     twin.sample(logits, temp, top_k, top_p, seeds, ref)
     assert torch.equal(out, ref)
     # without filters the many-block path is taken: same noise, same choice as the one-block kernel
-    big = (torch.randn(5, 20011) * 2).cuda()
-    t5 = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.3]).cuda()
+    big = (torch.randn(5, 20011) * 2).to(DEV)
+    t5 = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.3]).to(DEV)
     s5 = seeds[:5].contiguous()
-    fast = torch.empty(5, dtype=torch.int32, device="cuda"); slow = torch.empty_like(fast)
+    fast = torch.empty(5, dtype=torch.int32, device=DEV); slow = torch.empty_like(fast)
     hip.sample(big, t5, None, None, s5, fast)
-    hip.sample(big, t5, torch.zeros(5, dtype=torch.int32).cuda(), None, s5, slow)
+    hip.sample(big, t5, torch.zeros(5, dtype=torch.int32).to(DEV), None, s5, slow)
     assert torch.equal(fast, slow) and int(fast[0]) == int(big[0].argmax())
     # a row's draw does not depend on the rest of the batch
-    one = torch.empty(1, dtype=torch.int32, device="cuda")
+    one = torch.empty(1, dtype=torch.int32, device=DEV)
     for r in range(rows):
         hip.sample(logits[r:r + 1], temp[r:r + 1], top_k[r:r + 1], top_p[r:r + 1], seeds[r:r + 1], one)
         assert int(one) == int(out[r])
 
 
 def test_sampling_distribution(hip):
+    emulator_skips(float("inf"))
     # 32768 draws at temperature 0.7 stay within 0.015 of softmax(l / 0.7) (reference tests/test_sampler.py:351-367)
     torch.manual_seed(5)
     vocab, draws = 12, 32768
     row = torch.randn(vocab) * 1.5
-    logits = row[None].repeat(draws, 1).cuda()
-    temp = torch.full((draws,), 0.7).cuda()
-    seeds = (torch.arange(draws, dtype=torch.int64) * 0x9E3779B1 + 12345).cuda()
-    out = torch.empty(draws, dtype=torch.int32, device="cuda")
+    logits = row[None].repeat(draws, 1).to(DEV)
+    temp = torch.full((draws,), 0.7).to(DEV)
+    seeds = (torch.arange(draws, dtype=torch.int64) * 0x9E3779B1 + 12345).to(DEV)
+    out = torch.empty(draws, dtype=torch.int32, device=DEV)
     hip.sample(logits, temp, None, None, seeds, out)
     freq = torch.bincount(out.long().cpu(), minlength=vocab).float() / draws
     assert (freq - torch.softmax(row / 0.7, -1)).abs().max() < 0.015
     # top-k then top-p: the nucleus is taken over the survivors of top-k (tests/test_sampler.py:332-349)
-    logits = torch.tensor([[3.0, 2.0, 1.0, 0.0, -1.0]]).repeat(draws, 1).cuda()
-    hip.sample(logits, torch.ones(draws).cuda(), torch.full((draws,), 3, dtype=torch.int32).cuda(),
-               torch.full((draws,), 0.7).cuda(), seeds, out)
+    logits = torch.tensor([[3.0, 2.0, 1.0, 0.0, -1.0]]).repeat(draws, 1).to(DEV)
+    hip.sample(logits, torch.ones(draws).to(DEV), torch.full((draws,), 3, dtype=torch.int32).to(DEV),
+               torch.full((draws,), 0.7).to(DEV), seeds, out)
     freq = torch.bincount(out.long().cpu(), minlength=5).float() / draws
     p3 = torch.softmax(torch.tensor([3.0, 2.0, 1.0]), -1)   # 0.665, 0.245, 0.090: nucleus 0.7 keeps two
     expect = torch.tensor([p3[0], p3[1], 0, 0, 0]) / (p3[0] + p3[1])
@@ -490,6 +524,7 @@ def test_sampling_distribution(hip):
 @pytest.mark.parametrize("batch,ctx,q_len", [(1, 2049, 1), (3, 700, 1), (64, 300, 1), (2, 1500, 130), (1, 4100, 1)])
 def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     """Few rows and long contexts: the key ranges are split over many wavefronts and merged."""
+    emulator_skips(batch * ctx * q_len * 48 * 128, 6e8)
     heads, kv_heads, head_dim, page = 48, 8, 128, 64
     dtype = torch.bfloat16
     lens = [ctx - 3 * i for i in range(batch)]
@@ -497,7 +532,7 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     meta = make_meta(table, lens, [q_len] * batch)
     T = batch * q_len
     q = randn(T, heads, head_dim, dtype=dtype, seed=2)
-    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device="cuda")
+    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device=DEV)
     hip.paged_attention(q, cache, meta, out_h, head_dim ** -0.5, 0)
     assert meta.work[(heads // kv_heads, 0)].num_tasks > 0 or batch * q_len >= 64, "expected split units"
     for t in sorted({0, T // 2, T - 1}):
@@ -521,19 +556,15 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     (8, 8, 32, 8, 0, [17000], [4100])])                          # more pages than the kernel keeps ids of at once
 def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, page, window, lens, q_lens):
     """Steps with many rows: blocks share each step's keys and values through shared memory."""
+    emulator_skips(sum(q * (min(n, window + q) if window else n) for q, n in zip(q_lens, lens)) * heads * head_dim, 2.5e9)
     dtype = torch.bfloat16
-    cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=heads + head_dim)
-    # a page's slots past a request's end may hold anything an earlier owner left, even NaN
-    last_page = int(table[0, (lens[0] - 1) // page])
-    if lens[0] % page:
-        beyond = torch.arange(lens[0] % page, page, device="cuda")
-        layout.keys_view(cache)[last_page, :, beyond] = float("nan")
-        layout.values_view(cache)[last_page, :, beyond // 8, beyond % 8] = float("nan")
+    # pages the window has passed are given back (-1 in the table); whatever no request holds is not-a-number
+    cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=heads + head_dim, window=window, q_lens=q_lens)
     meta = make_meta(table, lens, q_lens)
     T = sum(q_lens)
     q = randn(T, heads, head_dim, dtype=dtype, seed=3)
     scale = head_dim ** -0.5
-    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device="cuda")
+    out_h = torch.empty(T, heads * head_dim, dtype=dtype, device=DEV)
     out_t = torch.empty_like(out_h)
     hip.paged_attention(q, cache, meta, out_h, scale, window)
     work = meta.work[(heads // kv_heads, window)]
@@ -552,9 +583,10 @@ def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, p
                                       (64, 200064, 3072), (5, 50, 128), (3, 64, 96)])
 def test_skinny_linear(hip, rows, n, k):
     """Few rows against a large matrix: the streaming kernel where its sizes fit, the library otherwise."""
+    emulator_skips(rows * n * k, 4e8)
     x = randn(rows, k, dtype=torch.bfloat16, seed=1)
     w = randn(n, k, dtype=torch.bfloat16, scale=k ** -0.5, seed=2)
-    out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device=DEV)
     hip.linear(x, w, out)
     ref = x.float() @ w.float().T
     torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1.6e-2)
@@ -575,8 +607,8 @@ def test_rounding_to_bfloat16_is_to_nearest_even(hip):
     b[:6] = torch.tensor([1.5, 1.5, 1.5, 3.0, 1.0, 2 ** -20]).bfloat16()
     x = torch.zeros(rows, k, dtype=torch.bfloat16); x[:, 0] = a
     w = torch.zeros(n, k, dtype=torch.bfloat16); w[:, 0] = b
-    out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
-    hip.linear(x.cuda(), w.cuda(), out)
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device=DEV)
+    hip.linear(x.to(DEV), w.to(DEV), out)
     ref = (a.float()[:, None] * b.float()[None, :]).bfloat16()
     finite = torch.isfinite(ref.float())
     assert torch.equal(out.cpu()[finite].view(torch.int16), ref[finite].view(torch.int16))
@@ -589,47 +621,49 @@ def test_cache_pages_beyond_four_gigabytes(hip, twin, dtype):
     """A layer's cache tensor larger than 2^32 bytes and 2^31 elements: the write and both
     attention kernels must address its last pages with 64-bit offsets (a 32-bit offset would wrap
     into the first pages, which stay zero here)."""
+    emulator_skips(float("inf"))
     heads, kv_heads, head_dim, page, rotary = 48, 8, 128, 64, 64
     pages = 17000
     assert pages * 2 * kv_heads * page * head_dim > 2 ** 31
-    cache = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device="cuda")
+    cache = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device=DEV)
     lens, q_lens = [700, 130], [200, 1]
     need = [-(-n // page) for n in lens]
     ids = [list(range(16990, 16990 - need[0], -1)), list(range(16900, 16900 + need[1]))]
     table = torch.full((2, max(need) + 1), -1, dtype=torch.int32)
     for r, row in enumerate(ids):
         table[r, :len(row)] = torch.tensor(row, dtype=torch.int32)
-    table = table.cuda()
+    table = table.to(DEV)
     T = sum(lens)
     width = (heads + 2 * kv_heads) * head_dim
     qkv = randn(T, width, dtype=dtype, seed=11)
-    positions = torch.cat([torch.arange(n) for n in lens]).to(torch.int32).cuda()
+    positions = torch.cat([torch.arange(n) for n in lens]).to(torch.int32).to(DEV)
     slots = torch.cat([torch.tensor([ids[r][p // page] * page + p % page for p in range(n)]) for r, n in enumerate(lens)])
     used = sorted(set(sum(ids, [])))
     remap = {p: i for i, p in enumerate(used)}
-    small_slots = torch.tensor([remap[int(s) // page] * page + int(s) % page for s in slots], dtype=torch.int32).cuda()
-    slots = slots.to(torch.int32).cuda()
+    small_slots = torch.tensor([remap[int(s) // page] * page + int(s) % page for s in slots], dtype=torch.int32).to(DEV)
+    slots = slots.to(torch.int32).to(DEV)
     cos_sin = rope_table(2048, rotary, 5e6)
-    qw = (1 + 0.1 * torch.randn(heads * head_dim)).to(dtype).cuda()
-    kw = (1 + 0.1 * torch.randn(kv_heads * head_dim)).to(dtype).cuda()
-    small = torch.zeros(len(used), 2, kv_heads, page, head_dim, dtype=dtype, device="cuda")
+    qw = (1 + 0.1 * torch.randn(heads * head_dim)).to(dtype).to(DEV)
+    kw = (1 + 0.1 * torch.randn(kv_heads * head_dim)).to(dtype).to(DEV)
+    small = torch.zeros(len(used), 2, kv_heads, page, head_dim, dtype=dtype, device=DEV)
     a, b = qkv.clone(), qkv.clone()
     hip.qk_norm_rope_store(a, positions, cos_sin, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache, slots, page)
     twin.qk_norm_rope_store(b, positions, cos_sin, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, small, small_slots, page)
-    torch.testing.assert_close(cache[torch.tensor(used).cuda()], small, **tol(dtype))
+    torch.testing.assert_close(cache[torch.tensor(used).to(DEV)], small, **tol(dtype))
     assert float(cache[:16384].abs().max()) == 0.0                 # nothing wrapped into the low pages
     # attention over these pages: a prompt portion (blocks of tiles in bfloat16) and a decoded token
-    rows = torch.cat([torch.arange(lens[0] - q_lens[0], lens[0]), torch.tensor([T - 1])]).cuda()
+    rows = torch.cat([torch.arange(lens[0] - q_lens[0], lens[0]), torch.tensor([T - 1])]).to(DEV)
     q = a[rows, :heads * head_dim].reshape(-1, heads, head_dim).contiguous()
     meta = make_meta(table, lens, q_lens)
-    out = torch.empty(q.shape[0], heads * head_dim, dtype=dtype, device="cuda")
+    out = torch.empty(q.shape[0], heads * head_dim, dtype=dtype, device=DEV)
     hip.paged_attention(q, cache, meta, out, head_dim ** -0.5, 0)
     for t in (0, 77, 199, 200):
         row, pos = int(meta.token_row[t]), int(meta.positions[t])
         ref = dense_attention(q[t], cache, table, row, pos, head_dim ** -0.5, 0, page)
         torch.testing.assert_close(out[t].float(), ref, rtol=1.6e-2, atol=1.6e-2)
     del cache
-    torch.cuda.empty_cache()
+    if DEV == "cuda":
+        torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("tokens", [3, 40, 600])
@@ -637,20 +671,21 @@ def test_expert_weights_beyond_two_to_the_31_elements(hip, twin, tokens):
     """MiniMax-M2's expert tables hold 2.4e9 and 1.2e9 elements; the last experts lie beyond a
     32-bit element offset (and, in bytes, beyond 2^32).  Only those are chosen here, in the
     streaming, the tall and the wide kernel."""
+    emulator_skips(float("inf"))
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     dtype, experts, hidden, inter, k = torch.bfloat16, 256, 3072, 1536, 2
     assert (experts - 3) * 2 * inter * hidden > 2 ** 31
-    w13 = torch.zeros(experts, 2 * inter, hidden, dtype=dtype, device="cuda")
-    w2 = torch.zeros(experts, hidden, inter, dtype=dtype, device="cuda")
-    g = torch.Generator(device="cuda").manual_seed(5)
+    w13 = torch.zeros(experts, 2 * inter, hidden, dtype=dtype, device=DEV)
+    w2 = torch.zeros(experts, hidden, inter, dtype=dtype, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(5)
     for e in (experts - 3, experts - 2, experts - 1):
-        w13[e] = (torch.randn(2 * inter, hidden, generator=g, device="cuda") * hidden ** -0.5).to(dtype)
-        w2[e] = (torch.randn(hidden, inter, generator=g, device="cuda") * inter ** -0.5).to(dtype)
+        w13[e] = (torch.randn(2 * inter, hidden, generator=g, device=DEV) * hidden ** -0.5).to(dtype)
+        w2[e] = (torch.randn(hidden, inter, generator=g, device=DEV) * inter ** -0.5).to(dtype)
     x = randn(tokens, hidden, dtype=dtype, seed=21)
-    ids = torch.stack([experts - 3 + torch.randperm(3)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
-    weights = torch.rand(tokens, k).cuda()
+    ids = torch.stack([experts - 3 + torch.randperm(3)[:k] for _ in range(tokens)]).to(torch.int32).to(DEV)
+    weights = torch.rand(tokens, k).to(DEV)
     weights = weights / weights.sum(-1, keepdim=True)
-    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, DEV)
     out_h = torch.empty_like(x)
     hip.moe_experts(x, w13, w2, ids, weights, out_h, ws)
     # the twin on the three used experts alone
@@ -659,7 +694,8 @@ def test_expert_weights_beyond_two_to_the_31_elements(hip, twin, tokens):
     assert float(out_t.abs().max()) > 0.1
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
     del w13, w2
-    torch.cuda.empty_cache()
+    if DEV == "cuda":
+        torch.cuda.empty_cache()
 
 
 def test_expert_tables_arranged_in_place_are_the_tiled_copy(hip, twin):
@@ -683,9 +719,9 @@ def test_expert_tables_arranged_in_place_are_the_tiled_copy(hip, twin):
     odd = randn(2, 2 * 72, 200, dtype=dtype, seed=3)
     assert hip.arrange_expert_weights(odd, randn(2, 200, 72, dtype=dtype, seed=4)) is False   # sizes of the general kernel
     x = randn(tokens, hidden, dtype=dtype, seed=11)
-    ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).cuda()
-    weights = torch.rand(tokens, k).cuda()
-    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+    ids = torch.stack([torch.randperm(experts)[:k] for _ in range(tokens)]).to(torch.int32).to(DEV)
+    weights = torch.rand(tokens, k).to(DEV)
+    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, DEV)
     out_h, out_t = torch.empty_like(x), torch.empty_like(x)
     hip.moe_experts(x, a13, a2, ids, weights, out_h, ws, tiled=True)
     twin.moe_experts(x, w13, w2, ids, weights, out_t)
@@ -710,11 +746,11 @@ def test_attention_on_random_shapes(hip):
             n = rng.choice([1, 2, 31, 32, 33, 64, 100, 255, 256, 500, 1000, 2500])
             lens.append(n)
             q_lens.append(max(1, min(n, rng.choice([1, 1, 2, 16, 65, n]))))
-        cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=case)
+        cache, table = make_paged(dtype, kv_heads, head_dim, page, lens, seed=case, window=window, q_lens=q_lens)
         meta = make_meta(table, lens, q_lens)
         T = sum(q_lens)
         q = randn(T, heads, head_dim, dtype=dtype, seed=case + 1)
-        out = torch.full((T, heads * head_dim), float("nan"), dtype=dtype, device="cuda")
+        out = torch.full((T, heads * head_dim), float("nan"), dtype=dtype, device=DEV)
         scale = head_dim ** -0.5
         hip.paged_attention(q, cache, meta, out, scale, window)
         what = f"case {case}: heads {heads}/{kv_heads}, head_dim {head_dim}, page {page}, window {window}, lens {lens}, new {q_lens}"
@@ -738,14 +774,14 @@ def test_experts_on_random_shapes_and_lumpy_routing(hip, twin):
         hidden, inter = rng.choice([256, 512, 768]), rng.choice([128, 256, 384])
         tokens = rng.choice([1, 2, 7, 16, 17, 33, 64, 100, 255, 256, 257, 500, 1000, 2100])
         g = torch.Generator().manual_seed(case)
-        x = torch.randn(tokens, hidden, generator=g).to(dtype).cuda()
-        w13 = (torch.randn(experts, 2 * inter, hidden, generator=g) * hidden ** -0.5).to(dtype).cuda()
-        w2 = (torch.randn(experts, hidden, inter, generator=g) * inter ** -0.5).to(dtype).cuda()
+        x = torch.randn(tokens, hidden, generator=g).to(dtype).to(DEV)
+        w13 = (torch.randn(experts, 2 * inter, hidden, generator=g) * hidden ** -0.5).to(dtype).to(DEV)
+        w2 = (torch.randn(experts, hidden, inter, generator=g) * inter ** -0.5).to(dtype).to(DEV)
         liking = torch.rand(experts, generator=g) ** 3 + 1e-3
-        ids = torch.stack([torch.multinomial(liking, k, generator=g) for _ in range(tokens)]).to(torch.int32).cuda()
-        weights = torch.rand(tokens, k, generator=g).cuda()
+        ids = torch.stack([torch.multinomial(liking, k, generator=g) for _ in range(tokens)]).to(torch.int32).to(DEV)
+        weights = torch.rand(tokens, k, generator=g).to(DEV)
         weights = weights / weights.sum(-1, keepdim=True)
-        ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, "cuda")
+        ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, DEV)
         ref = torch.empty_like(x)
         twin.moe_experts(x, w13, w2, ids, weights, ref)
         a13, a2 = w13.clone(), w2.clone()

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests import traces
+from tests import backends, traces
 from tests.helpers import CONFIGS, make_folder, random_tokens
 from tests.plain.minimax_m2 import PlainMiniMaxM2
 
@@ -18,6 +18,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 LENGTHS = {"A": [5, 17, 31, 100, 64, 129, 250, 1, 48], "B": [1, 9, 40, 100, 200, 333, 65, 16, 500],
            "C": [3, 40, 130, 700, 64, 257, 1, 33, 520]}
+# the emulated backend runs a thousand times slower: fewer and shorter requests, the same edges
+# (one token, a page's edge, one past it, several pages)
+SHORT_LENGTHS = {"A": [5, 17, 64, 1, 100], "B": [1, 9, 65, 16, 130], "C": [3, 40, 130, 1, 64]}
 
 
 def bound(dtype, ref):
@@ -33,7 +36,8 @@ def model(request, tmp_path_factory):
     key = request.param
     folder = make_folder(tmp_path_factory.mktemp("models"), key)
     vocab = CONFIGS[key][0]["vocab_size"]
-    requests = {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate(LENGTHS[key[0]])}
+    lengths = (SHORT_LENGTHS if backends.ACTIVE.slow else LENGTHS)[key[0]]
+    requests = {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate(lengths)}
     plain = PlainMiniMaxM2(folder)
     expected = {rid: plain.logits(toks).numpy() for rid, toks in requests.items()}
     return folder, requests, expected, plain
@@ -49,7 +53,8 @@ def run_records(folder, dtype, records, max_tokens, page_size):
     from sparseengine_amd.engine.replay import replay_step
     from sparseengine_amd.engine.runner import ModelRunner
     runner = ModelRunner.from_folder(folder, dtype=dtype, kv_page_size=page_size,
-                                     num_kvcache_tokens=-(-max_tokens // 64) * 64, max_num_seqs=4)
+                                     num_kvcache_tokens=-(-max_tokens // 64) * 64, max_num_seqs=4,
+                                     **backends.ACTIVE.runner_kwargs())
     out, routing = {}, {}
     for rec in records:
         taps = {}
@@ -145,10 +150,13 @@ def test_trace_run_program(model, dtype, tmp_path):
     folder, requests, expected, plain = model
     records, peak = traces.mixed(requests, seed=3)
     out_dir = tmp_path / "out"
+    env = dict(os.environ)
+    if backends.ACTIVE.name == "emu":      # the program builds its engine itself: name the kernels' stand-in
+        env.update(SPARSEENGINE_AMD_KERNELS="tests.emu.kernels:EmulatedProgramKernels", PYTHONPATH=ROOT)
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
          "--out", str(out_dir), "--max-tokens", str(peak), "--page-size", "16"],
-        input="".join(json.dumps(r) + "\n" for r in records), capture_output=True, text=True, timeout=600)
+        input="".join(json.dumps(r) + "\n" for r in records), capture_output=True, text=True, timeout=1800, env=env)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {r['step']}" for r in records]
     vocab = next(iter(expected.values())).shape[1]
@@ -162,7 +170,8 @@ def test_trace_run_program(model, dtype, tmp_path):
         proc = subprocess.run(
             [sys.executable, "-m", "sparseengine_amd", "replay", "--model", folder, "--dtype", dtype, "--out", str(other),
              "--max-tokens", str(peak), "--page-size", "16"], cwd=ROOT,
-            input="".join(json.dumps(r) + "\n" for r in records[:6]), capture_output=True, text=True, timeout=600)
+            input="".join(json.dumps(r) + "\n" for r in records[:6]), capture_output=True, text=True, timeout=1800,
+            env=env)
         assert proc.returncode == 0, proc.stderr[-2000:]
         for r in records[:6]:
             assert np.array_equal(np.fromfile(other / f"{r['step']}.f32", dtype="<f4").reshape(-1, vocab), logits[r["step"]])
@@ -177,14 +186,16 @@ def test_matrix_core_sizes_take_the_matrix_core_kernels(tmp_path):
     from sparseengine_amd.kernels.hip_ops import HipKernels
     folder = make_folder(tmp_path, "C_loud")
     stored = load_file(os.path.join(folder, "model.safetensors"))
-    w1 = stored["model.layers.0.block_sparse_moe.experts.3.w1.weight"].cuda()
-    half = ModelRunner.from_folder(folder, dtype="bfloat16", kv_page_size=16, num_kvcache_tokens=256, max_num_seqs=2)
+    w1 = stored["model.layers.0.block_sparse_moe.experts.3.w1.weight"].to(backends.ACTIVE.device)
+    half = ModelRunner.from_folder(folder, dtype="bfloat16", kv_page_size=16, num_kvcache_tokens=256, max_num_seqs=2,
+                                   **backends.ACTIVE.runner_kwargs())
     ffn = half.model.layers[0].ffn
     assert ffn._tiled is True
     inter = w1.shape[0]
-    tiled_expert = HipKernels.tile_expert_weights(torch.cat([w1, stored["model.layers.0.block_sparse_moe.experts.3.w3.weight"].cuda()])[None])
+    tiled_expert = HipKernels.tile_expert_weights(torch.cat([w1, stored["model.layers.0.block_sparse_moe.experts.3.w3.weight"].to(backends.ACTIVE.device)])[None])
     assert torch.equal(ffn.params["w13"][3:4], tiled_expert) and not torch.equal(ffn.params["w13"][3, :inter], w1)
-    full = ModelRunner.from_folder(folder, dtype="float32", kv_page_size=16, num_kvcache_tokens=256, max_num_seqs=2)
+    full = ModelRunner.from_folder(folder, dtype="float32", kv_page_size=16, num_kvcache_tokens=256, max_num_seqs=2,
+                                   **backends.ACTIVE.runner_kwargs())
     assert full.model.layers[0].ffn._tiled is False
     assert torch.equal(full.model.layers[0].ffn.params["w13"][3, :inter], w1.float())
     spec = half.spec.layers[0].mixer

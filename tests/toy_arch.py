@@ -80,6 +80,8 @@ class SignRoutedFFN(Part):
     def forward(self, fb, x):
         p = self.params
         choice = (x.float() @ p["probe"].float() > 0).long()                   # [T]
+        if fb.taps is not None:
+            fb.taps.setdefault("toy_sign", []).append(choice.clone())
         up, down = p["up"].float()[choice], p["down"].float()[choice]          # [T, i, h], [T, h, i]
         hidden = torch.nn.functional.silu(torch.einsum("tih,th->ti", up, x.float()))
         return torch.einsum("thi,ti->th", down, hidden).to(x.dtype)
@@ -202,8 +204,12 @@ class PlainToy:
         self.cfg = json.load(open(os.path.join(folder, "config.json")))
         self.w = {k[4:]: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
 
-    def logits(self, tokens):
+    def logits(self, tokens, forced=None):
+        """``forced``: {"router": [ids [T, k] per routed layer in run order], "sign": [choice [T] per
+        sign-routed layer]}: the choices of a run in reduced precision, whose near-ties may tip."""
         cfg, w = self.cfg, self.w
+        forced = forced or {}
+        routers, signs = iter(forced.get("router", [])), iter(forced.get("sign", []))
         T = len(tokens)
         pos = torch.arange(T)
         x = w["embed.weight"][torch.as_tensor(tokens)]
@@ -247,14 +253,18 @@ class PlainToy:
                 gu = m @ w[p + "ffn.gate_up"].T
                 x = (torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]) @ w[p + "ffn.down"].T
             elif layer["ffn"] == "sign":
-                x = torch.stack([
-                    w[p + "ffn.down"][int(t @ w[p + "ffn.probe"] > 0)]
-                    @ torch.nn.functional.silu(w[p + "ffn.up"][int(t @ w[p + "ffn.probe"] > 0)] @ t) for t in m])
+                choice = next(signs, None)
+                if choice is None:
+                    choice = (m @ w[p + "ffn.probe"] > 0).long()
+                x = torch.stack([w[p + "ffn.down"][int(c)] @ torch.nn.functional.silu(w[p + "ffn.up"][int(c)] @ t)
+                                 for t, c in zip(m, choice)])
             else:
                 logits = m @ w[p + "ffn.router"].T
                 scores = torch.softmax(logits, -1) if layer.get("scoring") == "softmax" else torch.sigmoid(logits)
                 sel = scores + w[p + "ffn.router_bias"] if layer.get("bias", True) else scores
-                ids = torch.topk(sel, layer["top_k"], dim=-1).indices
+                ids = next(routers, None)
+                if ids is None:
+                    ids = torch.topk(sel, layer["top_k"], dim=-1).indices
                 wts = scores.gather(1, ids)
                 if layer.get("normalize", True):
                     wts = wts / wts.sum(-1, keepdim=True)
