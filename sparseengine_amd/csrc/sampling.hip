@@ -8,6 +8,7 @@
 // The noise of token i is a pure function of (seed of the row, i): a row's draw does not depend
 // on which other rows share the launch.
 #include "common.h"
+#include "no_alloc.h"
 
 #define SAMPLE_THREADS 1024
 
@@ -229,6 +230,42 @@ extern "C" int se_sample(const float* logits, int64_t stride, int rows, int voca
   if (vocab <= 0) return SE_ERR_SHAPE;
   sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, stride, vocab, temperature, top_k,
                                                      top_p, seeds, out);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+// ---------------------------------------------------------------------------------------- //
+// The same arg-max sampling for callers that cannot allocate (no_alloc.h): the partial maxima go
+// to a fixed array in device memory instead of a workspace of the caller's.
+// ---------------------------------------------------------------------------------------- //
+static __device__ __align__(256) unsigned char scratch[SE_NO_ALLOC_SAMPLE_SLOTS * (sizeof(float) + sizeof(int32_t))];
+
+#define SE_NO_ALLOC_MAX_DEVICES 64
+static unsigned char* scratch_of_device[SE_NO_ALLOC_MAX_DEVICES];   // the array's address on each GPU, once asked for
+
+extern "C" int se_sample_unfiltered_no_alloc(const float* logits, int64_t stride, int rows, int vocab,
+                                             const float* temperature, const uint64_t* seeds,
+                                             int32_t* out, hipStream_t stream) {
+  if (rows <= 0) return SE_OK;
+  if (vocab <= 0) return SE_ERR_SHAPE;
+  const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  if (chunks > 65535 || static_cast<int64_t>(rows) * chunks > SE_NO_ALLOC_SAMPLE_SLOTS) return SE_ERR_SHAPE;
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= SE_NO_ALLOC_MAX_DEVICES) return SE_ERR_LAUNCH;
+  if (!scratch_of_device[device]) {
+    // in host code the array's name is a stand-in, not a device address: every GPU holds its own
+    // copy at its own address, which is asked for once with that GPU current
+    void* address = nullptr;
+    if (hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)) != hipSuccess || !address) return SE_ERR_LAUNCH;
+    scratch_of_device[device] = static_cast<unsigned char*>(address);
+  }
+  // every slot a call reads has been written by the same call: nothing has to start at zero
+  float* part_value = reinterpret_cast<float*>(scratch_of_device[device]);
+  int32_t* part_index = reinterpret_cast<int32_t*>(scratch_of_device[device] + SE_NO_ALLOC_SAMPLE_SLOTS * sizeof(float));
+  sample_partial_kernel<<<dim3(rows, chunks), SAMPLE_THREADS, 0, stream>>>(
+      logits, stride, vocab, temperature, seeds, part_value, part_index, chunks);
+  SE_CHECK_LAUNCH();
+  sample_final_kernel<<<rows, SE_WAVE, 0, stream>>>(part_value, part_index, chunks, out);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -44,16 +44,19 @@ def _on_gpu(item) -> bool:
     return "gpu" in item.keywords and not any(m.name == "skip" for m in item.iter_markers())
 
 
-def pytest_runtest_logstart(nodeid, location):
-    """The name of every GPU test goes out, flushed, before the test touches the GPU: if the
-    process dies under it, the last name printed is the test that was running."""
-    if "gpu" in nodeid or os.environ.get("SPARSEENGINE_AMD_NAME_TESTS"):
+@pytest.hookimpl(hookwrapper=True, tryfirst=True)
+def pytest_runtest_protocol(item, nextitem):
+    """The name of every GPU test goes out, flushed, before the test touches the GPU (and before
+    output is captured for it): if the process dies under it, the last name printed is the test
+    that was running."""
+    if _on_gpu(item):
         for stream in (sys.__stdout__, sys.__stderr__):
             try:
-                stream.write(f"\n[test] {nodeid}\n")
+                stream.write(f"\n[test] {item.nodeid}\n")
                 stream.flush()
             except (OSError, ValueError):
                 pass
+    yield
 
 
 @pytest.hookimpl(trylast=True)

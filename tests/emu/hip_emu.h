@@ -40,7 +40,7 @@
 #define __forceinline__ inline
 #define __shared__ static
 #define __launch_bounds__(...)
-#define __align__(n) alignas(n)
+#define __align__(n) __attribute__((aligned(n)))
 
 // ---------------------------------------------------------------------------------------------
 // runtime shared by all emulated libraries (tests/emu/emu_rt.cpp, loaded first and globally)
@@ -77,6 +77,16 @@ enum hipError_t { hipSuccess = 0, hipErrorUnknown = 999 };
 enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize = 8 };
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
+inline hipError_t hipGetDevice(int* device) {
+  *device = 0;
+  return hipSuccess;
+}
+// a __device__ variable is an ordinary one here: its name is its address
+#define HIP_SYMBOL(x) x
+inline hipError_t hipGetSymbolAddress(void** address, const void* symbol) {
+  *address = const_cast<void*>(symbol);
+  return hipSuccess;
+}
 
 namespace {
 
