@@ -7,9 +7,15 @@ top-8 of width 1536, vocabulary 200064) cut to 16 of its 62 layers, random weigh
 A "step" is one decode step of a batch of 8 requests whose prompts were 2048 random token ids
 (sampling greedily, token ids read back each step).  One JSON line is printed: ``value`` is decoded
 tokens per second at batch 8; ``prefill`` is a 2048-token prompt in one step (``frac``: its flops
-against the matrix peak, ``hbm_frac``: the bytes it has to read against 8 TB/s); ``points`` holds
-decode at batch 1 and 64 and the prefill of eight 2048-token prompts in one step; ``roofline``
-prices the batch-8 decode step against 8 TB/s.
+against the matrix peak, ``hbm_frac``: the bytes it has to read against 8 TB/s, ``experts_touched``:
+the mean number of experts per layer that its tokens chose); ``points`` holds decode at batch 1 and
+64 and the prefill of eight 2048-token prompts in one step; ``roofline`` prices the batch-8 decode
+step against 8 TB/s and ``point_rooflines`` the other decode points the same way (every weight the
+step uses once - the experts it touched are counted from the step's own routing - and the cache of
+the live requests).  With random weights the tokens of a prompt agree on a few dozen experts past
+the first layer, which makes a prompt cheaper than real weights would: ``prefill_uniform`` is the
+same step with every token sent to eight experts drawn evenly from all 256 (the routing is replaced
+after the router has run, so the router's own work is still in the time).
 """
 from __future__ import annotations
 
@@ -25,7 +31,7 @@ MODEL = dict(
     architectures=["MiniMaxM2ForCausalLM"], model_type="minimax_m2", hidden_size=3072,
     num_attention_heads=48, num_key_value_heads=8, head_dim=128, rotary_dim=64, rope_theta=5000000.0,
     num_local_experts=256, num_experts_per_tok=8, intermediate_size=1536, vocab_size=200064,
-    rms_norm_eps=1e-6, use_qk_norm=True, max_position_embeddings=8192, tie_word_embeddings=False)
+    rms_norm_eps=1e-6, use_qk_norm=True, max_position_embeddings=204800, tie_word_embeddings=False)
 FULL_MODEL_LAYERS = 62
 PROMPT_LEN = 2048
 CONTEXT_LEN = 8192
@@ -144,7 +150,8 @@ def main() -> int:
         runner.release(f"p{i}")
     prefill_s = min(times[1:])
     T = PROMPT_LEN
-    prefill_bytes = None
+    prefill_bytes = touched = None
+    uniform_s = uniform_bytes = None
     if not args.no_prefill:     # untimed: the experts the prompt touches, layer by layer, are what it has to read
         taps = {}
         runner.step([StepEntry("p_taps", prompt(), [PROMPT_LEN - 1])], taps=taps)
@@ -152,6 +159,21 @@ def main() -> int:
         touched = [int(torch.unique(i).numel()) for i, _ in taps["router"]]
         prefill_bytes = L * dense_layer + sum(touched) * expert_bytes + V * h * itemsize
         del taps
+        # the same step with even expert load: eight distinct experts per token, drawn uniformly
+        dev_gen = torch.Generator(device="cuda").manual_seed(1)
+        even = [torch.rand(T, E, generator=dev_gen, device="cuda").topk(K, dim=-1).indices.to(torch.int32).contiguous()
+                for _ in range(L)]
+        uniform_times = []
+        for i in range(3):
+            sync()
+            t = time.perf_counter()
+            runner.step([StepEntry(f"u{i}", prompt(), [PROMPT_LEN - 1])], forced_routing=even)
+            sync()
+            uniform_times.append(time.perf_counter() - t)
+            runner.release(f"u{i}")
+        uniform_s = min(uniform_times[1:])
+        uniform_bytes = L * dense_layer + L * min(E, T * K) * expert_bytes + V * h * itemsize
+        del even
     prefill_flops = L * (2 * T * h * (H + 2 * Hkv) * D + 2 * T * H * D * h + 2 * T * h * E + 2 * T * K * 3 * I * h
                          + 4 * H * D * T * (T + 1) / 2) + 2 * V * h
     peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
@@ -179,11 +201,13 @@ def main() -> int:
         return 0
     step_s, distinct, context = decode(args.batch, args.steps, args.warmup, "d")
     print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
-    points = {}
+    points, point_rooflines = {}, {}
     for b in [int(x) for x in args.points.split(",") if x]:
-        s, _, _ = decode(b, max(8, args.steps // 2), max(2, args.warmup // 2), f"b{b}_")
+        s, d, c = decode(b, max(8, args.steps // 2), max(2, args.warmup // 2), f"b{b}_")
         points[f"decode_b{b}"] = round(b / s, 1)
-        print(f"[bench] decode batch {b}: {s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+        point_rooflines[f"decode_b{b}"] = round(decode_bytes(b, d, c) / s / HBM_PEAK, 4)
+        print(f"[bench] decode batch {b}: {s * 1e3:.2f} ms/step, {sum(d) / len(d):.0f} experts touched per layer, "
+              f"{decode_bytes(b, d, c) / s / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
 
     if many_prompts:
         points[many_prompts[0]] = many_prompts[1]
@@ -197,14 +221,22 @@ def main() -> int:
                    "global_batch": args.batch, "seq_len": CONTEXT_LEN, "prompt_len": PROMPT_LEN, "hidden_size": h,
                    "num_attention_heads": H, "num_key_value_heads": Hkv, "head_dim": D, "rotary_dim": cfg["rotary_dim"],
                    "num_local_experts": E, "num_experts_per_tok": K, "intermediate_size": I, "vocab_size": V,
-                   "kv_page_size": 64, "kv_cache_tokens": args.kv_requests * CONTEXT_LEN, "parallelism": "single GPU"},
+                   "kv_page_size": 64, "kv_cache_tokens": args.kv_requests * CONTEXT_LEN,
+                   "max_position_embeddings": cfg["max_position_embeddings"], "parallelism": "single GPU"},
         "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops / prefill_s / peak, 5),
                     # a 2048-token step reads every expert it touches for a few dozen rows each: memory bound too
-                    "hbm_frac": None if prefill_bytes is None else round(prefill_bytes / prefill_s / HBM_PEAK, 4)},
+                    "hbm_frac": None if prefill_bytes is None else round(prefill_bytes / prefill_s / HBM_PEAK, 4),
+                    "flops": prefill_flops, "bytes": prefill_bytes,
+                    "experts_touched": None if touched is None else round(sum(touched) / len(touched), 1)},
+        "prefill_uniform": None if uniform_s is None else {
+            "value": round(T / uniform_s, 1), "tokens": T, "ms": round(uniform_s * 1e3, 3),
+            "frac": round(prefill_flops / uniform_s / peak, 5), "hbm_frac": round(uniform_bytes / uniform_s / HBM_PEAK, 4),
+            "bytes": uniform_bytes, "experts_touched": min(E, T * K)},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
+        "point_rooflines": point_rooflines,
     }
     print(json.dumps(line), flush=True)
     return 0

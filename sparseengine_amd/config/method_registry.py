@@ -13,19 +13,48 @@ PREFILL_POLICY_AUTO = "auto"
 METHOD_ALIASES = {"vanilla": "", "none": "", "dense": "", "full": ""}
 
 
-class PassThroughMethod:
-    """The dense method: every hook is the identity."""
+class MethodRuntime:
+    """What a sparse method may do in a step, and the defaults of the dense method.
+
+    One object per engine.  The step function and the attention mixer call it at fixed places:
+
+    ``bind(cache)``                once, with the engine's cache manager;
+    ``prepare_step(fb)``           after the step's batch is built, before the first layer;
+    ``select(position, meta)``     per cache-keeping schedule position, just before attention: the
+                                   view of the request's pages the layer may read (a ``GroupMeta``, or
+                                   anything with its fields); the dense method hands back what it gets;
+    ``after_attention(position, fb)`` per such position, after its attention has read the cache;
+    ``finish_step(fb)``            after the last layer, before logits leave the step;
+    ``extra_pages(row, new_tokens)`` pages per group index the method needs for itself on top of
+                                   what the cache manager counts for an append (temporary slots);
+                                   the scheduler's capacity questions add them.
+
+    (Reference: engine/sparse_methods/base.py:324-500 prepare_step / build_*_selection /
+    on_attention_end / finish_step; engine/cache_manager/base.py:1335-1361 the cache-side hooks.)
+    """
     name = ""
 
+    def bind(self, cache) -> None:
+        self.cache = cache
+
+    def prepare_step(self, fb) -> None:
+        pass
+
     def select(self, position: int, meta):
-        """The keys a layer may read: all of them."""
         return meta
 
     def after_attention(self, position: int, fb) -> None:
         pass
 
-    def after_step(self, fb) -> None:
+    def finish_step(self, fb) -> None:
         pass
+
+    def extra_pages(self, row: int | None, new_tokens: int) -> dict[int, int]:
+        return {}
+
+
+class PassThroughMethod(MethodRuntime):
+    """The dense method: every hook is the identity (reference engine/sparse_methods/passthrough.py:11-32)."""
 
 
 @dataclass(frozen=True)

@@ -60,6 +60,14 @@ class ForwardBatch:
         self.token_item = None         # int32 [T]
         self.item_rows = None          # int32 [items]: the cache row (state slot) of every item
         self.item_rows_host = None
+        # where every item's tokens lie in the step and how long its request is with them: host
+        # copies (int32 numpy [items]) and one device tensor [3, items] = q_start, q_len, ctx_len.
+        # They belong to the step, not to a cache group: a mixer that keeps state only reads them too.
+        self.item_q_start = None
+        self.item_q_len = None
+        self.item_ctx_len = None
+        self.item_meta = None
+        self.method = None             # the sparse method's runtime (config/method_registry.py)
         self.want_index = None         # int32 [wanted] token indices whose logits are returned
         self.groups: dict[int, GroupMeta] = {}
         self.taps: dict | None = None
@@ -175,6 +183,7 @@ class BatchBuilder:
         fb.item_rows, fb.item_rows_host = view(3), rows
         fb.want_index = view(5)
         item_meta = view(4, (3, B))
+        fb.item_q_start, fb.item_q_len, fb.item_ctx_len, fb.item_meta = q_start, q_len, ctx_len, item_meta
         for gi, group in enumerate(cache.groups):
             fb.groups[group.index] = GroupMeta(
                 block_table=view(6 + 2 * gi + 1, tables[group.index].shape),

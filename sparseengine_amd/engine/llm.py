@@ -26,8 +26,9 @@ from .sequence import Sequence
 class CacheOracle(MemoryOracle):
     """The scheduler's view of the cache manager, in pages of the tightest group."""
 
-    def __init__(self, cache):
+    def __init__(self, cache, method=None):
         self.cache = cache
+        self.method = method
 
     def free_pages(self):
         return min(g.pool.free_count for g in self.cache.groups) if self.cache.groups else 1 << 30
@@ -44,9 +45,14 @@ class CacheOracle(MemoryOracle):
     def pages_to_append(self, seq_id, new_tokens):
         if new_tokens <= 0:
             return 0
-        if not self.cache.has_row(seq_id):
-            return self.cache.pages_for_tokens(new_tokens)
-        needed = self.cache.pages_needed(self.cache.row_of(seq_id), new_tokens)
+        row = self.cache.row_of(seq_id) if self.cache.has_row(seq_id) else None
+        if row is None:
+            needed = {g.index: self.cache.pages_for_tokens(new_tokens) for g in self.cache.groups}
+        else:
+            needed = self.cache.pages_needed(row, new_tokens)
+        if self.method is not None:       # what the sparse method keeps for itself on top
+            for group, pages in self.method.extra_pages(row, new_tokens).items():
+                needed[group] = needed.get(group, 0) + pages
         return max(needed.values()) if needed else 0
 
     def tokens_that_fit(self, seq_id, pages):
@@ -133,7 +139,7 @@ class LLM:
         cache_tokens = config.num_kvcache_slots
         common = dict(dtype=config.dtype, device=device, kv_page_size=config.kv_page_size,
                       max_num_seqs=config.max_num_seqs_in_gpu, max_model_len=config.max_model_len,
-                      mlp_chunk_size=config.mlp_chunk_size, kernels=kernels)
+                      mlp_chunk_size=config.mlp_chunk_size, kernels=kernels, method=self.method)
         if config.tiny_random:
             self.runner = ModelRunner.from_random(config.raw_model_config, seed=config.tiny_random_seed,
                                                   on_device=config.tiny_random_on_device,
@@ -142,7 +148,7 @@ class LLM:
         else:
             self.runner = ModelRunner.from_folder(model, num_kvcache_tokens=cache_tokens,
                                                   gpu_memory_utilization=config.gpu_memory_utilization, **common)
-        self.oracle = CacheOracle(self.runner.cache)
+        self.oracle = CacheOracle(self.runner.cache, self.method)
         self.scheduler = Scheduler(
             self.oracle, max_num_batched_tokens=config.max_num_batched_tokens,
             max_num_seqs_in_batch=config.max_num_seqs_in_batch, max_decoding_seqs=config.max_decoding_seqs,
@@ -181,11 +187,11 @@ class LLM:
         bad = [t for t in ids if not 0 <= t < self.vocab_size]
         if bad:
             raise ValueError(f"prompt token {bad[0]} is outside the vocabulary [0, {self.vocab_size})")
-        if len(ids) + sampling_params.max_tokens > self.config.max_model_len:
+        longest = len(ids) + sampling_params.max_tokens
+        if longest > self.config.max_model_len:
             raise ValueError(
-                f"Prompt length + max_tokens exceeds max_model_len: {len(ids)} + {sampling_params.max_tokens} "
-                f"> {self.config.max_model_len}. Reduce prompt/decoding length or increase max_model_len "
-                "if the model supports it.")
+                f"this request may grow to {longest} tokens ({len(ids)} of prompt, max_tokens = "
+                f"{sampling_params.max_tokens}), more than max_model_len = {self.config.max_model_len} allows")
         sampling_params.validate_for_vocab(self.vocab_size)
         seq = Sequence(ids, sampling_params)
         self.scheduler.add(seq)
@@ -223,7 +229,6 @@ class LLM:
                 for s, t, c, top in zip(wanting, tokens, chosen, tops):
                     sampled[s.seq_id] = t
                     logprobs[s.seq_id] = (c, top)
-            self.method.after_step(None)
             times.section("sample")
         except Exception:
             self.scheduler.fail_step(schedule)

@@ -61,7 +61,7 @@ class StepEntry:
 class ModelRunner:
     def __init__(self, arch: Architecture, cfg, params_factory, *, dtype, device="cuda", kv_page_size=64,
                  num_kvcache_tokens: int | None = None, max_num_seqs: int = 8, max_model_len: int | None = None,
-                 mlp_chunk_size: int = 16384, kernels=None, gpu_memory_utilization: float = 0.9):
+                 mlp_chunk_size: int = 16384, kernels=None, gpu_memory_utilization: float = 0.9, method=None):
         self.arch, self.model_config = arch, cfg
         self.dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
@@ -79,15 +79,15 @@ class ModelRunner:
         if getattr(kernels, "libraries", None):
             from ..kernels import library
             library.ensure_built(sorted(self.model.all_kernel_libraries()))
-        decls = self.model.all_param_decls()
-        self.params = params_factory(decls, self.dtype, self.device)
-        self.model.bind_all(self.params)
-        self.model.finalize_all(kernels)
-
         self.max_model_len = int(max_model_len or self.spec.max_position)
         if self.max_model_len > self.spec.max_position:
             raise ValueError(f"max_model_len {self.max_model_len} exceeds the model's "
                              f"max_position_embeddings {self.spec.max_position}")
+        self.model.limit_positions(self.max_model_len)
+        decls = self.model.all_param_decls()
+        self.params = params_factory(decls, self.dtype, self.device)
+        self.model.bind_all(self.params)
+        self.model.finalize_all(kernels)
         self.kv_page_size = int(kv_page_size)
         requests = self.model.cache_requests()
         if num_kvcache_tokens is None or int(num_kvcache_tokens) <= 0:
@@ -104,6 +104,11 @@ class ModelRunner:
                     shapes.setdefault(self.cache.group_of_position[position], set()).add(key())
         self.builder = BatchBuilder(kernels, self.cache, self.dtype, self.device, self.spec.vocab_size,
                                     attention_shapes=shapes)
+        if method is None:
+            from ..config.method_registry import PassThroughMethod
+            method = PassThroughMethod()
+        self.method = method
+        method.bind(self.cache)
 
     def derive_cache_tokens(self, requests, max_num_seqs: int, utilization: float) -> int:
         """Tokens of cache that fit the memory left after the weights: ``utilization`` of the card
@@ -163,19 +168,22 @@ class ModelRunner:
         need = {g.index: 0 for g in self.cache.groups}
         new_rows = 0
         for request_id, n in entries:
-            if self.cache.has_row(request_id):
-                for gi, pages in self.cache.pages_needed(self.cache.row_of(request_id), n).items():
+            row = self.cache.row_of(request_id) if self.cache.has_row(request_id) else None
+            if row is not None:
+                for gi, pages in self.cache.pages_needed(row, n).items():
                     need[gi] += pages
             else:
                 new_rows += 1
                 for gi in need:
                     need[gi] += self.cache.pages_for_tokens(n)
+            for gi, pages in self.method.extra_pages(row, n).items():
+                need[gi] += pages
         free = self.cache.free_pages()
         return new_rows <= self.cache.num_free_rows and all(need[g] <= free[g] for g in need)
 
     # ------------------------------------------------------------------ the step
     @torch.no_grad()
-    def step(self, entries: list[StepEntry], taps: dict | None = None) -> torch.Tensor:
+    def step(self, entries: list[StepEntry], taps: dict | None = None, forced_routing=None) -> torch.Tensor:
         """Run the entries' tokens as one batch; float32 logits ``[wanted, vocab]`` in the order
         of the entries and of their ``want`` lists.  A request that holds no row yet is admitted.
         If the cache cannot take the step, ``OutOfPages`` is raised and nothing has changed."""
@@ -193,4 +201,9 @@ class ModelRunner:
                 self.cache.free(request_id)
             raise
         fb.taps = taps
-        return self.model.forward(fb)
+        fb.forced_routing = forced_routing      # measurement and test seam (parts/feed_forward.py: _force)
+        fb.method = self.method
+        self.method.prepare_step(fb)
+        logits = self.model.forward(fb)
+        self.method.finish_step(fb)
+        return logits

@@ -55,24 +55,23 @@ class DeviceAttentionWork:
     tiles_per_block: int
 
 
-_native = None      # the compiled builder (csrc/host_work.hip), False if it cannot be had
+_native = None      # the compiled builder (csrc/host_work.hip)
 
 
 def _native_library():
+    """The compiled builder; like every other library of the kernels it is built at first use and
+    a failure to build or load it is an error (``KernelLibraryError``), not a quiet change of path."""
     global _native
     if _native is None:
-        try:
-            from . import library
-            lib = library.load("host_work")
-            i64p, i32p = ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32)
-            lib.se_attention_work_plan.argtypes = [i64p, i64p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                                   ctypes.c_int, ctypes.c_int, i64p, i64p, i64p]
-            lib.se_attention_work_fill.argtypes = [i64p, i64p, ctypes.c_int, ctypes.c_int, ctypes.c_int, i64p,
-                                                   i64p, i32p, i32p, i32p]
-            _native = lib
-        except Exception:       # no compiler, read-only tree ...: the numpy builder does the same work
-            _native = False
-    return _native or None
+        from . import library
+        lib = library.load("host_work")
+        i64p, i32p = ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32)
+        lib.se_attention_work_plan.argtypes = [i64p, i64p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                               ctypes.c_int, ctypes.c_int, i64p, i64p, i64p]
+        lib.se_attention_work_fill.argtypes = [i64p, i64p, ctypes.c_int, ctypes.c_int, ctypes.c_int, i64p,
+                                               i64p, i32p, i32p, i32p]
+        _native = lib
+    return _native
 
 
 _BAD_LENGTHS = "attention work: every item needs at least one new token and no more new tokens than its context holds"
@@ -80,11 +79,9 @@ _BAD_LENGTHS = "attention work: every item needs at least one new token and no m
 
 def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int = 0,
                          target_waves: int = TARGET_WAVES, head_dim: int = 0) -> AttentionWork:
-    """The work lists of one step; see ``build_attention_work_numpy`` for the rules.  The compiled
-    builder is used when it is there (it gives the same lists, about twenty times faster)."""
+    """The work lists of one step, from the compiled builder; ``build_attention_work_numpy`` states
+    the rules and gives the same lists (the tests compare the two), about twenty times slower."""
     lib = _native_library()
-    if lib is None:
-        return build_attention_work_numpy(q_len, ctx_len, group, kv_heads, window, target_waves, head_dim)
     q = np.ascontiguousarray(q_len, dtype=np.int64)
     c = np.ascontiguousarray(ctx_len, dtype=np.int64)
     rules = np.asarray([target_waves, MIN_SPLIT_KEYS, MAX_SPLITS, TILES_PER_BLOCK, TILED_MAX_HEAD_DIM,

@@ -37,6 +37,11 @@ class GQAAttention(Part):
             decls["k_norm"] = ParamDecl((self.kv_width,))
         return decls
 
+    def limit_positions(self, positions: int) -> None:
+        limit = getattr(self.position, "limit_positions", None)     # a position part of the tests may not have it
+        if limit is not None:
+            limit(positions)
+
     def bind(self, params):
         super().bind(params)
         self.position.prepare(params["qkv"].device)
@@ -58,7 +63,11 @@ class GQAAttention(Part):
             cache if write_cache else None, meta.slots if write_cache else None, meta.page_size)
         attended = fb.buffer("attn.out", (T, self.q_width))
         q = qkv[:, :self.q_width].view(T, s.num_heads, s.head_dim)
-        fb.kernels.paged_attention(q, cache, meta, attended, s.scale, s.window or 0)
+        method = getattr(fb, "method", None)
+        visible = meta if method is None else method.select(cache_position, meta)     # what this layer may read
+        fb.kernels.paged_attention(q, cache, visible, attended, s.scale, s.window or 0)
+        if method is not None:
+            method.after_attention(cache_position, fb)
         if fb.taps is not None:
             fb.taps.setdefault("attention_inputs", []).append(qkv.clone())
         return linear(attended, p["o"], out=fb.buffer("attn.proj", (T, self.hidden_size)), kernels=fb.kernels)

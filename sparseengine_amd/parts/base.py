@@ -59,6 +59,12 @@ class Part:
     def children(self) -> dict[str, "Part"]:
         return {}
 
+    def limit_positions(self, positions: int) -> None:
+        """Before ``bind``: the engine will never ask for a position at or beyond ``positions``
+        (parts with tables by position size them by this; the default hands it to the children)."""
+        for child in self.children().values():
+            child.limit_positions(positions)
+
     # flattened views over the tree of parts ---------------------------------------------
     def all_param_decls(self, prefix: str = "") -> dict[str, ParamDecl]:
         out = {prefix + name: decl for name, decl in self.param_decls().items()}

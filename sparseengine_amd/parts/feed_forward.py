@@ -61,12 +61,32 @@ class RoutedExperts(Part):
     def forward(self, fb, x):
         s, p, T = self.spec, self.params, x.shape[0]
         out = fb.buffer("ffn.out", (T, self.hidden_size))
+        forced = None
+        given = getattr(fb, "forced_routing", None)
+        if given is not None:       # measurement and test seam, see ``_force``
+            call = getattr(fb, "_routed_calls", 0)
+            fb._routed_calls = call + 1
+            forced = given[call] if call < len(given) else None
         for start in range(0, T, self.chunk_tokens):
             stop = min(T, start + self.chunk_tokens)
-            self._forward_chunk(fb, x[start:stop], out[start:stop])
+            self._forward_chunk(fb, x[start:stop], out[start:stop], None if forced is None else forced[start:stop])
         return out
 
-    def _forward_chunk(self, fb, x, out):
+    def _force(self, logits, forced, ids, weights):
+        """Measurement and test seam (``fb.forced_routing``: per routed layer of the step the experts
+        ``[T, top_k]`` every token is to take, or None): the router's choice is replaced, the weights
+        are the chosen experts' own scores as the router would have weighted them.  A run in reduced
+        precision can so be compared with one in float32 expert for expert, and a benchmark can
+        spread its tokens evenly over the experts; nothing in the product sets it."""
+        s = self.spec
+        scores = torch.sigmoid(logits) if s.scoring == "sigmoid" else torch.softmax(logits, dim=-1)
+        ids.copy_(forced)
+        chosen = scores.gather(1, forced.long())
+        if s.norm_topk_prob:
+            chosen = chosen / chosen.sum(-1, keepdim=True)
+        weights.copy_(chosen * s.routed_scaling_factor)
+
+    def _forward_chunk(self, fb, x, out, forced=None):
         s, p, T = self.spec, self.params, x.shape[0]
         logits = fb.buffer("moe.logits", (T, s.num_experts), torch.float32)
         ids = fb.buffer("moe.ids", (T, s.top_k), torch.int32)
@@ -75,6 +95,9 @@ class RoutedExperts(Part):
         ws = self._workspace_for(fb, T, w13.dtype)
         fb.kernels.route(x, p["router"], p.get("router_bias"), s.top_k, logits, ids, weights, scoring=s.scoring,
                          normalize=s.norm_topk_prob, scaling=s.routed_scaling_factor, workspace=ws)
+        if forced is not None:
+            self._force(logits, forced, ids, weights)
+            ws.grouped = None          # whatever the router's launch grouped were its own choices
         if fb.taps is not None:
             fb.taps.setdefault("router", []).append((ids.clone(), weights.clone()))
         if w13.dtype == x.dtype:

@@ -8,6 +8,7 @@ sin half in float32, built on the host exactly as the reference does
 from __future__ import annotations
 
 import math
+import weakref
 
 import torch
 
@@ -64,6 +65,21 @@ def rotary_inverse_frequencies(rotary_dim: int, theta: float, scaling: dict | No
                               "(default, linear, llama3, yarn)")
 
 
+# Tables by (spec, rows, device): layers with the same rotation share one tensor (a 62-layer model
+# with 204800 positions would hold 62 copies of the same 52 MB otherwise).  Entries go when the last
+# part that uses them goes.
+_SHARED_TABLES: "weakref.WeakValueDictionary" = weakref.WeakValueDictionary()
+
+
+def shared_table(key, build):
+    """The table stored under ``key``, built by ``build()`` if nobody holds it yet."""
+    table = _SHARED_TABLES.get(key)
+    if table is None:
+        table = build()
+        _SHARED_TABLES[key] = table
+    return table
+
+
 class RotaryPosition(Part):
     """Rotation of the leading ``rotary_dim`` dims of each head, NeoX pairing ``(d, d + R/2)``."""
 
@@ -76,14 +92,22 @@ class RotaryPosition(Part):
             raise ValueError("a rotary encoding needs max_position > 0")
         self.spec = spec
         self.rotary_dim = spec.rotary_dim
+        self.rows = spec.max_position
         self.table = None
 
+    def limit_positions(self, positions: int) -> None:
+        """No position at or beyond ``positions`` will be asked for: the table need not hold more rows."""
+        self.rows = max(1, min(self.spec.max_position, int(positions)))
+
     def prepare(self, device) -> None:
-        spec = self.spec
-        inv_freq, factor = rotary_inverse_frequencies(spec.rotary_dim, spec.theta,
-                                                      dict(spec.scaling) if spec.scaling else None)
-        angles = torch.arange(spec.max_position, dtype=torch.float32)[:, None] * inv_freq[None, :]
-        self.table = torch.cat((angles.cos() * factor, angles.sin() * factor), dim=-1).contiguous().to(device)
+        spec, rows = self.spec, self.rows
+
+        def build():
+            inv_freq, factor = rotary_inverse_frequencies(spec.rotary_dim, spec.theta,
+                                                          dict(spec.scaling) if spec.scaling else None)
+            angles = torch.arange(rows, dtype=torch.float32)[:, None] * inv_freq[None, :]
+            return torch.cat((angles.cos() * factor, angles.sin() * factor), dim=-1).contiguous().to(device)
+        self.table = shared_table((spec, rows, str(torch.device(device))), build)
 
 
 class NoPosition(Part):
@@ -94,6 +118,9 @@ class NoPosition(Part):
         pass
 
     def prepare(self, device) -> None:
+        pass
+
+    def limit_positions(self, positions: int) -> None:
         pass
 
 

@@ -72,6 +72,25 @@ class EmulatedBackend(Backend):
             yield
 
 
+class TwinBackend(Backend):
+    """The tensor-library twins of the kernels on the CPU: the host side of the engine alone."""
+    name = "twin"
+    device = "cpu"
+
+    def kernels(self):
+        from tests.twin_kernels import TwinKernels
+        return TwinKernels()
+
+    def runner_kwargs(self) -> dict:
+        return dict(device="cpu", kernels=self.kernels())
+
+    def llm_kwargs(self) -> dict:
+        return dict(_device="cpu", _kernels=self.kernels())
+
+    def available(self) -> bool:
+        return True
+
+
 def _from_environment() -> Backend:
     name = os.environ.get("SPARSEENGINE_AMD_TEST_BACKEND", "hip")
     if name == "emu":
@@ -89,7 +108,7 @@ def use(backend):
     """Run the block on another backend (an instance, or "emu" / "hip")."""
     global ACTIVE
     if isinstance(backend, str):
-        backend = EmulatedBackend() if backend == "emu" else Backend()
+        backend = {"emu": EmulatedBackend, "twin": TwinBackend, "hip": Backend}[backend]()
     saved = ACTIVE
     ACTIVE = backend
     try:

@@ -51,7 +51,7 @@ def rope_angles(positions: torch.Tensor, rotary_dim: int, theta: float):
     """cos/sin of ``p * theta^(-2d/R)``, ``d in [0, R/2)``; float32 as the reference
     builds its table.  layers/rotary_embedding.py:20-22,217-222.
     """
-    exponent = torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim
+    exponent = torch.arange(0, rotary_dim, 2, dtype=torch.float32, device=positions.device) / rotary_dim
     inv_freq = 1.0 / (theta ** exponent)
     freqs = positions.to(torch.float32)[:, None] * inv_freq[None, :]
     return freqs.cos(), freqs.sin()
@@ -84,7 +84,7 @@ def causal_gqa_attention(q, k, v, scale: float, window: int | None = None):
     Hkv = k.shape[1]
     group = H // Hkv
     out = torch.empty_like(q)
-    pos = torch.arange(T)
+    pos = torch.arange(T, device=q.device)
     allowed = pos[None, :] <= pos[:, None]
     if window is not None:
         allowed &= pos[None, :] > pos[:, None] - window
@@ -154,7 +154,10 @@ class PlainConfig:
     @classmethod
     def from_folder(cls, folder: str) -> "PlainConfig":
         with open(os.path.join(folder, "config.json")) as fh:
-            raw = json.load(fh)
+            return cls.from_dict(json.load(fh))
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "PlainConfig":
         rope_parameters = raw.get("rope_parameters") or {}
         theta = rope_parameters.get("rope_theta", raw.get("rope_theta", 10000.0))  # models/rope.py:37-43
         return cls(
@@ -181,6 +184,16 @@ class PlainMiniMaxM2:
             with safe_open(os.path.join(folder, name), framework="pt") as fh:
                 for key in fh.keys():
                     self.w[key] = fh.get_tensor(key).to(dtype)
+
+    @classmethod
+    def from_tensors(cls, raw_config: dict, tensors: dict[str, torch.Tensor], dtype: torch.dtype = torch.float32):
+        """The same model from checkpoint tensors by name that are in memory already (a model too
+        large to pass through a file); they may live on another device, where the forward pass then runs."""
+        self = cls.__new__(cls)
+        self.cfg = PlainConfig.from_dict(raw_config)
+        self.dtype = dtype
+        self.w = {name: t.to(dtype) for name, t in tensors.items()}
+        return self
 
     # one decoder layer: models/minimax_m2.py:334-397
     def attention_inputs(self, layer: int, u: torch.Tensor, positions: torch.Tensor):
@@ -215,7 +228,7 @@ class PlainMiniMaxM2:
             log[layer] = torch.sigmoid(logits) + bias
         if forced_ids is None:
             return biased_sigmoid_router(logits, bias, c.num_experts_per_tok)
-        ids = torch.as_tensor(forced_ids, dtype=torch.long)
+        ids = torch.as_tensor(forced_ids, dtype=torch.long, device=logits.device)
         weights = torch.sigmoid(logits).gather(1, ids)
         return weights / weights.sum(dim=-1, keepdim=True), ids
 
@@ -230,8 +243,9 @@ class PlainMiniMaxM2:
         """Final-normed hidden state of every token.  Residual wiring:
         models/minimax_m2.py:381-397, models/qwen3.py:291-325."""
         c = self.cfg
-        ids = torch.as_tensor(token_ids, dtype=torch.long)
-        positions = torch.arange(start_position, start_position + ids.numel())
+        device = self.w["model.embed_tokens.weight"].device      # the CPU, unless the tensors were handed over elsewhere
+        ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
+        positions = torch.arange(start_position, start_position + ids.numel(), device=device)
         x = self.w["model.embed_tokens.weight"][ids]
         residual = None
         for layer in range(c.num_hidden_layers):

@@ -115,7 +115,7 @@ def test_generate_is_the_plain_greedy_decoding(model):
     outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
     assert [o["token_ids"] for o in outs] == [plain.greedy(p, 8) for p in prompts]
     assert all(o["text"] == "" for o in outs)                       # no tokenizer in a random folder
-    with pytest.raises(ValueError, match="exceeds max_model_len"):
+    with pytest.raises(ValueError, match="more than max_model_len"):
         engine.add_request(prompts[0], SamplingParams(max_tokens=10 ** 6))
     with pytest.raises(ValueError, match="unknown configuration keys"):
         LLM(folder, not_an_option=1)
@@ -363,3 +363,159 @@ def test_engine_bench_counts_every_token_once(model, tmp_path, capsys):
         assert r["decode_tok_s"] > 0 and r["prefill_tok_s"] > 0 and r["total_s"] >= r["prefill_s"] + r["decode_s"] - 1e-3
     with pytest.raises(SystemExit):
         microbench.main(["--model_path", str(folder), "--lengths", "0"], llm_factory=lambda path, **kw: llm(path, **kw))
+
+
+# ------------------------------------------------------------------ what another architecture needs, without a GPU
+def test_toy_architecture_on_the_cpu(tmp_path):
+    """The toy architecture of the tests (a mixer with state of its own, a windowed cache group, a
+    layer that runs twice, a shared cache, its own feed-forward and rotation) registers, builds and
+    steps on the kernel twins: float32 logits equal its plain implementation under a mixed trace."""
+    from tests import backends
+    from tests.test_gpu_engine import run_toy_architecture
+    with backends.use("twin"):
+        run_toy_architecture(tmp_path, "float32", [70, 9, 33, 100, 1, 64])
+
+
+def test_an_architecture_with_state_only_and_no_cache_pages(tmp_path):
+    """Every layer keeps state of fixed size and none keeps keys and values: no cache group, no page
+    pool, no block table; item boundaries come from the step itself (``ForwardBatch.item_q_start``)."""
+    from sparseengine_amd.weights.random_weights import write_model_folder
+    from tests import toy_arch
+    config = dict(toy_arch.TOY_CONFIG, max_position_embeddings=256, layers=[
+        dict(mixer="decay", state_size=12, decay=0.8, ffn="dense", intermediate=40),
+        dict(mixer="decay", state_size=5, decay=0.5, ffn="sign", intermediate=24)],
+        schedule=[dict(layer=0), dict(layer=1), dict(layer=0)])
+    folder = write_model_folder(str(tmp_path / "state_only"), config, 4, {"std": 0.15})
+    plain = toy_arch.PlainToy(folder)
+    requests = {f"r{i}": random_tokens(n, 300, 70 + i) for i, n in enumerate([40, 3, 65, 1, 17])}
+    records, peak = traces.mixed(requests, seed=2)
+    runner = ModelRunner.from_folder(folder, dtype="float32", device="cpu", kv_page_size=16, num_kvcache_tokens=64,
+                                     max_num_seqs=4, kernels=TwinKernels())
+    assert runner.cache.groups == [] and sorted(runner.cache.state_positions) == [0, 1, 2]
+    out = {}
+    for rec in records:
+        logits = replay_step(runner, rec, None)
+        if logits is not None:
+            out[rec["step"]] = logits
+        runner.cache.check_invariants()
+    got = traces.gather(records, out)
+    for rid, toks in requests.items():
+        ref = plain.logits(toks).numpy()
+        assert np.abs(got[rid] - ref).max() < 2e-5 * max(1.0, np.abs(ref).max()), rid
+    assert runner.cache.num_free_rows == 4
+    # and through the entry point: the scheduler has no pages to count, only rows
+    engine = LLM(folder, dtype="float32", num_kvcache_slots=64, kv_page_size=16, max_num_seqs_in_batch=2,
+                 _kernels=TwinKernels(), _device="cpu")
+    prompts = [requests["r0"][:9], requests["r2"][:20], requests["r4"]]
+    outs = engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True), use_tqdm=False)
+    for prompt, o in zip(prompts, outs):
+        toks = list(prompt)
+        for t in o["token_ids"]:
+            assert t == int(plain.logits(toks)[-1].argmax())
+            toks.append(t)
+
+
+def test_a_second_sparse_method_gets_every_hook(model):
+    """A method registered from outside the package is resolved by name, bound to the cache and
+    called once per step (prepare, finish), once per cache-keeping layer (select, after attention)
+    and asked for its own pages; handing back the view it was given changes no token."""
+    from sparseengine_amd.config import method_registry
+    folder, requests, _, plain = model
+    calls = []
+
+    class Counting(method_registry.MethodRuntime):
+        name = "counting"
+
+        def bind(self, cache):
+            super().bind(cache)
+            calls.append(("bind", len(cache.groups)))
+
+        def prepare_step(self, fb):
+            calls.append(("prepare", fb.num_tokens))
+
+        def select(self, position, meta):
+            calls.append(("select", position))
+            return meta
+
+        def after_attention(self, position, fb):
+            calls.append(("after", position))
+
+        def finish_step(self, fb):
+            calls.append(("finish", fb.num_tokens))
+
+        def extra_pages(self, row, new_tokens):
+            calls.append(("extra", new_tokens))
+            return {0: 0}
+
+    method_registry.register_method("counting", Counting, "all_chunked")
+    try:
+        engine = llm(folder, sparse_method="counting")
+        prompt = list(requests.values())[1][:17]
+        out = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True), use_tqdm=False)
+        assert out[0]["token_ids"] == plain.greedy(prompt, 3)
+        layers = len(engine.runner.spec.schedule)
+        steps = [c for c in calls if c[0] == "prepare"]
+        assert calls[0] == ("bind", 1) and len(steps) == 3 and steps[0] == ("prepare", len(prompt)) and steps[1] == ("prepare", 1)
+        assert [c for c in calls if c[0] == "finish"] == [("finish", n) for _, n in steps]
+        assert [c[1] for c in calls if c[0] == "select"] == list(range(layers)) * 3
+        assert [c[1] for c in calls if c[0] == "after"] == list(range(layers)) * 3
+        assert any(c[0] == "extra" for c in calls)
+        with pytest.raises(ValueError, match="counting"):
+            llm(folder, sparse_method="counting", prefill_schedule_policy="something_else")
+    finally:
+        method_registry._METHODS.pop("counting", None)
+
+
+def test_replay_writes_the_pages_each_request_held(model, tmp_path):
+    """``pages.jsonl``: per step the page ids of the step's requests; under a pool of exactly the
+    peak need, pages of finished requests turn up again under later ones."""
+    folder, requests, _, _ = model
+    records, peak = traces.mixed(requests, seed=5)
+    runner = runner_for(folder, peak)
+    replay_stream(runner, (json.dumps(r) for r in records), str(tmp_path / "out"), report=open(os.devnull, "w"),
+                  with_taps=True)
+    lines = [json.loads(line) for line in open(tmp_path / "out" / "pages.jsonl")]
+    assert [l["step"] for l in lines] == [r["step"] for r in records]
+    owners: dict[int, set] = {}
+    fed: dict[str, int] = {}
+    for rec, line in zip(records, lines):
+        assert sorted(line["pages"]) == sorted(e["id"] for e in rec["entries"])
+        held_now = [p for groups in line["pages"].values() for p in groups["0"]]
+        assert len(held_now) == len(set(held_now)), "a page under two requests in one step"
+        for e in rec["entries"]:
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+            assert len(line["pages"][e["id"]]["0"]) == -(-fed[e["id"]] // 16)
+            for page in line["pages"][e["id"]]["0"]:
+                owners.setdefault(page, set()).add(e["id"])
+    assert any(len(ids) > 1 for ids in owners.values()), "no page was used again"
+    from safetensors.torch import load_file
+    taps = load_file(str(tmp_path / "out" / f"{records[0]['step']}.taps.safetensors"))
+    tokens = sum(len(e["tokens"]) for e in records[0]["entries"])
+    assert taps["layer_out.0"].shape[0] == tokens and taps["router.0.ids"].shape[0] == tokens
+
+
+def test_trace_run_program_on_the_cpu(model, tmp_path):
+    """``bin/trace_run`` itself, as a user calls it, with the kernel twins named through the test
+    seam: stdin in, logits files, ``done`` lines and the page log out; without the seam ``--device
+    cpu`` is refused (the engine's own kernels are the GPU's)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, requests, expected, _ = model
+    records, peak = traces.mixed(dict(list(requests.items())[:3]), seed=3)
+    cmd = [sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out",
+           str(tmp_path / "out"), "--max-tokens", str(peak), "--page-size", "16", "--device", "cpu"]
+    env = {k: v for k, v in os.environ.items() if k != "SPARSEENGINE_AMD_KERNELS"}
+    refused = subprocess.run(cmd, input="", capture_output=True, text=True, env=env)
+    assert refused.returncode != 0 and "SPARSEENGINE_AMD_KERNELS" in refused.stderr
+    env.update(SPARSEENGINE_AMD_KERNELS="tests.twin_kernels:TwinKernels", PYTHONPATH=root)
+    proc = subprocess.run(cmd, input="".join(json.dumps(r) + "\n" for r in records), capture_output=True, text=True,
+                          env=env, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {r['step']}" for r in records]
+    vocab = next(iter(expected.values())).shape[1]
+    logits = {r["step"]: np.fromfile(tmp_path / "out" / f"{r['step']}.f32", dtype="<f4").reshape(-1, vocab) for r in records}
+    got = traces.gather(records, logits)
+    for rid in got:
+        assert np.abs(got[rid] - expected[rid]).max() < 2e-5 * max(1.0, np.abs(expected[rid]).max())
+    assert len(open(tmp_path / "out" / "pages.jsonl").readlines()) == len(records)

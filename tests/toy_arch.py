@@ -44,10 +44,7 @@ class DecayMixer(Part):
         state = fb.state_view(cache_position)["s"]
         w_in, w_out = self.params["w_in"].float(), self.params["w_out"].float()
         out = torch.empty_like(x)
-        meta = next(iter(fb.groups.values())) if fb.groups else None
-        starts = meta.item_q_start if meta is not None else fb.toy_q_start
-        lens = meta.item_q_len if meta is not None else fb.toy_q_len
-        for row, start, n in zip(fb.item_rows_host.tolist(), starts.tolist(), lens.tolist()):
+        for row, start, n in zip(fb.item_rows_host.tolist(), fb.item_q_start.tolist(), fb.item_q_len.tolist()):
             s = state[row].clone()
             for t in range(start, start + n):          # a portion's tokens, in order
                 s = self.spec.decay * s + w_in @ x[t].float()
