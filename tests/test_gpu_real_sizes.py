@@ -8,15 +8,20 @@ engine stores them).  The float32 engine is first checked against the plain impl
 serves as the reference of the bfloat16 engine in every replay mode, with the bfloat16 engine's
 expert choices forced on it (a near-tie among 256 experts tips in bfloat16, which moves a logit by
 far more than rounding does; the choices themselves are checked to be top-8 up to a small slack).
-The bound: a bfloat16 rounding is off by 2^-9 / sqrt(3) = 0.11 % of the value (rms); sixteen
+The bound.  A bfloat16 rounding is off by 2^-9 / sqrt(3) = 0.11 % of the value (rms); sixteen
 roundings lie between the embedding and a logit of one layer (norms, projections, the five of the
 attention inputs and outputs, the stored residual, four in the experts, the slot sum, the head), so
-the hidden state that meets the head is off by about 0.45 % and a logit, being a product with that
-state, by 0.45 % of the logits' spread, plus its own rounding.  Allowed: 4 % of the spread (nine
-standard deviations: this test compares seven million logits) + 1 % of the logit itself.  (The
-reference compares its model with a float oracle at rtol 1e-2 / atol 2e-2 on logits of unit spread,
-tests/test_minimax_m2_model.py:95; the suite's general bfloat16 bound, 4 % of the largest logit, is
-four times wider than this one.)
+a logit should be off by about 0.45 % of the logits' spread (rms) at a position with few keys.
+Measured on MI355X: 0.41 % at the first positions, growing to 1.0 % at position 700 (attention
+averages more and more rounded keys and values), the same at every position of equal context,
+Gaussian (largest error of 1.4 million logits: 5.1 times the rms).  What a fault looks like is
+different: a wrong key, page or expert moves the logits of some positions by their whole spread.
+So the test asks for (1) an rms error of at most 1.5 % of the spread at every single position,
+(2) no single logit further off than 6.5 times the request's rms error (a Gaussian tail over a
+million samples ends at 5.2) and (3) 1 % of the logit's own size on top, for its own rounding.
+(The reference compares its model with a float oracle at rtol 1e-2 / atol 2e-2 on a tiny model,
+tests/test_minimax_m2_model.py:95; the suite's general bfloat16 bound, 4 % of the largest logit,
+is about 20 % of the spread.)
 """
 import numpy as np
 import pytest
@@ -128,10 +133,14 @@ def test_bfloat16_against_float32_at_real_layer_sizes():
         for rid in requests:
             scale = float(ref[rid].std())
             err = np.abs(got[rid] - ref[rid])
-            allowed = 4e-2 * scale + 1e-2 * np.abs(ref[rid])
-            print(f"[real sizes] {mode} {rid}: largest error {float((err / scale).max()):.4f} of the spread {scale:.3f}")
+            per_position = np.sqrt((err ** 2).mean(-1)) / scale
+            assert per_position.max() <= 0.015, (
+                f"{mode}, request {rid}: rms error {per_position.max():.4f} of the spread at position "
+                f"{int(per_position.argmax())} (median over positions {float(np.median(per_position)):.4f})")
+            rms = float(np.sqrt((err ** 2).mean()))
+            allowed = 6.5 * rms + 1e-2 * np.abs(ref[rid])
             worst = np.unravel_index(int((err - allowed).argmax()), err.shape)
             assert (err <= allowed).all(), (
                 f"{mode}, request {rid}: position {worst[0]}, token {worst[1]}: bfloat16 {got[rid][worst]:.4f}, "
-                f"float32 {ref[rid][worst]:.4f}, spread of the logits {scale:.3f}")
+                f"float32 {ref[rid][worst]:.4f}, rms error of the request {rms:.4f}, spread of the logits {scale:.3f}")
     assert half.cache.num_free_rows == 4 and full.cache.num_free_rows == 4
