@@ -501,12 +501,9 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   auto issue = [&](int step) {
     const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS + wave * DSTEPS) * 1024u;
     const bool over = next_key > kmax;
-    const bool under = next_key < low_clamp;     // only in a unit's first step
-    const int use_page = over ? clamp_page : (under ? low_page : next_page);
-    const int use_off = over ? clamp_off : (under ? low_off : next_off);
-    const int page = page_ids[use_page - window_base];
+    const int page = page_ids[(over ? clamp_page : next_page) - window_base];
     const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2) * plane + lane_base +
-                        static_cast<int64_t>(use_off) * off_scale;
+                        static_cast<int64_t>(over ? clamp_off : next_off) * off_scale;
 #pragma unroll
     for (int j = 0; j < DSTEPS; ++j) load16_to_lds(src + j * load_stride, dst + static_cast<uint32_t>(j) * 1024u);
     next_key += 32;
@@ -521,8 +518,21 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 
   const int nsteps = (key_end - k_first + 31) / 32;
   if (nsteps > 0) {
+    // Only a unit's first step can begin before `low_key` (it begins less than 32 keys before it): a
+    // lane whose key lies there takes `low_key`'s place for that one load and then goes on from its
+    // own key.  (Done here and not inside `issue`, which is the loop's hot path.)
+    const bool under = next_key < low_clamp;
+    if (under) {
+      next_page = low_page;
+      next_off = low_off;
+    }
+    issue(0);
+    if (under) {       // next_key has moved on by 32
+      next_page = next_key / page_size;
+      next_off = next_key % page_size;
+    }
 #pragma unroll
-    for (int j = 0; j < NS - 1; ++j)
+    for (int j = 1; j < NS - 1; ++j)
       if (j < nsteps) issue(j);
     for (int step = 0; step < nsteps; ++step) {
       const int k0 = k_first + 32 * step;
