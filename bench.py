@@ -51,6 +51,8 @@ def main() -> int:
     parser.add_argument("--no-decode", action="store_true", help="skip the decode measurements (for profiling prefill)")
     parser.add_argument("--prefill-prompts", type=int, default=8,
                         help="also time this many 2048-token prompts in one step (points.prefill_Nx2048); 1: skip")
+    parser.add_argument("--prefill-routing", default="both", choices=["both", "natural", "uniform"],
+                        help="profiling aid: which of the two prefill measurements to run (a reported line needs both)")
     parser.add_argument("--fake-context", action="store_true",
                         help="profiling aid, never used for reported numbers: reserve the prompts' cache pages "
                              "without computing them, so that a kernel trace holds decode steps only")
@@ -140,8 +142,9 @@ def main() -> int:
                 + batch * context * kv_token_layer * L)
 
     # ---- prefill of one 2048-token prompt
-    times = [0.0, 1.0] if args.no_prefill else []
-    for i in range(0 if args.no_prefill else 4):
+    natural = not args.no_prefill and args.prefill_routing != "uniform"
+    times = [] if natural else [0.0, 1.0]
+    for i in range(4 if natural else 0):
         sync()
         t = time.perf_counter()
         runner.step([StepEntry(f"p{i}", prompt(), [PROMPT_LEN - 1])])
@@ -152,13 +155,14 @@ def main() -> int:
     T = PROMPT_LEN
     prefill_bytes = touched = None
     uniform_s = uniform_bytes = None
-    if not args.no_prefill:     # untimed: the experts the prompt touches, layer by layer, are what it has to read
+    if natural:     # untimed: the experts the prompt touches, layer by layer, are what it has to read
         taps = {}
         runner.step([StepEntry("p_taps", prompt(), [PROMPT_LEN - 1])], taps=taps)
         runner.release("p_taps")
         touched = [int(torch.unique(i).numel()) for i, _ in taps["router"]]
         prefill_bytes = L * dense_layer + sum(touched) * expert_bytes + V * h * itemsize
         del taps
+    if not args.no_prefill and args.prefill_routing != "natural":
         # the same step with even expert load: eight distinct experts per token, drawn uniformly
         dev_gen = torch.Generator(device="cuda").manual_seed(1)
         even = [torch.rand(T, E, generator=dev_gen, device="cuda").topk(K, dim=-1).indices.to(torch.int32).contiguous()
@@ -180,7 +184,7 @@ def main() -> int:
     print(f"[bench] prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
 
     many_prompts = None
-    if args.prefill_prompts > 1 and not args.no_prefill:      # several prompts in one step: hundreds of rows per expert
+    if args.prefill_prompts > 1 and natural:      # several prompts in one step: hundreds of rows per expert
         n, best = args.prefill_prompts, float("inf")
         for i in range(3):
             ids = [f"m{i}_{j}" for j in range(n)]

@@ -158,11 +158,23 @@ def test_penalties_logprobs_and_eos(model):
     first = base[0]["token_ids"][0]
     stopped = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=6, eos_token_ids=[first]), use_tqdm=False)
     assert stopped[0]["token_ids"] == [first]
-    # a strong presence penalty forbids repeating a generated token
+    # penalties, token for token against the plain logits with the reference's rule applied by hand
+    # (layers/sampler.py:11-64: logits of prompt and generated tokens divided by the repetition
+    # penalty if positive, else multiplied; the presence penalty subtracted from generated tokens)
     pen = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True, presence_penalty=2.0,
                                                    repetition_penalty=1.5), use_tqdm=False)[0]["token_ids"]
+    tokens, generated = list(prompt), []
+    for _ in range(12):
+        logits = plain.logits(tokens)[-1].clone()
+        seen = torch.tensor(sorted(set(tokens)))
+        logits[seen] = torch.where(logits[seen] > 0, logits[seen] / 1.5, logits[seen] * 1.5)
+        if generated:
+            logits[torch.tensor(sorted(set(generated)))] -= 2.0
+        generated.append(int(logits.argmax()))
+        tokens.append(generated[-1])
+    assert pen == generated
     free = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True), use_tqdm=False)[0]["token_ids"]
-    assert len(set(pen)) >= len(set(free))
+    assert pen != free, "the penalties changed nothing: the prompt does not exercise them"
     engine.add_request(prompt, SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True, logprobs=2))
     finished = []
     while not engine.is_finished():

@@ -218,7 +218,16 @@ def test_command_line_bench_runs_every_case_on_the_gpu(tmp_path, capsys, command
     assert [(r["length"], r["batch_size"]) for r in rows] == [(40, 1), (40, 4), (130, 1), (130, 4)]
     for r in rows:
         assert r["completed"] == r["batch_size"] and r["prefill_tokens"] == r["batch_size"] * r["length"]
-        assert r["decode_tok_s"] > 0 and r["prefill_tok_s"] > 0
+        # the counts and rates of a row are those of its case: every prompt token fed once, the first
+        # generated token comes with the prompt's last portion, the five others from decode steps
+        # (a step that holds a prompt portion beside decoded tokens counts as a prompt step, as in the reference)
+        assert 5 <= r["decode_tokens"] <= 5 * r["batch_size"] and r["decode_steps"] >= 5
+        assert r["batch_size"] > 1 or r["decode_tokens"] == 5
+        assert r["prefill_steps"] >= -(-r["prefill_tokens"] // 96)          # the token budget of 96 cuts the prompts
+        assert r["decode_tok_s"] == pytest.approx(r["decode_tokens"] / r["decode_s"], rel=1e-3, abs=0.06)     # rounded to 0.1
+        assert r["prefill_tok_s"] == pytest.approx(r["prefill_tokens"] / r["prefill_s"], rel=1e-3, abs=0.06)
+        assert r["ms_per_decode_step"] == pytest.approx(r["decode_s"] / r["decode_steps"] * 1e3, rel=1e-2)
+        assert 0 < r["time_to_first_decode_s"] <= r["total_s"] and r["prefill_s"] + r["decode_s"] <= r["total_s"] * 1.001
 
 
 def test_weights_stored_in_32_bit_stay_so_under_bfloat16(tmp_path):
