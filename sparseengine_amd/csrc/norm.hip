@@ -55,7 +55,7 @@ template <typename T, typename W, int MAXV>
 __global__ void __launch_bounds__(256)
 rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* out,
                     const int32_t* __restrict__ rows, int hidden, float eps, int64_t x_stride,
-                    int64_t res_stride, int64_t out_stride, int write_residual) {
+                    int64_t res_stride, int64_t out_stride, int write_residual, int slots) {
   extern __shared__ float row_cache[];  // hidden floats, then 16 floats for the reduction
   float* scratch = row_cache + hidden;
   constexpr int VN = Vec16<T>::N;
@@ -63,20 +63,59 @@ rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* ou
   constexpr int WV = VN / WN;           // weight vectors per activation vector (1, or 2 for float weights)
   const int nvec = hidden / VN;
   const int64_t in_row = rows ? rows[blockIdx.x] : blockIdx.x;
-  const T* xr = x + in_row * x_stride;
+  const T* xr = x + in_row * slots * x_stride;
   T* rr = residual ? residual + in_row * res_stride : nullptr;
 
-  Vec16<T> xv[MAXV], rv[MAXV];
+  // x as float: the row itself, or (slots > 1) the sum of the row's `slots` consecutive rows of x,
+  // added up in float in slot order and rounded to the storage type, as a separate sum would leave it
+  float val[MAXV][VN];
+  Vec16<T> rv[MAXV];
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
     const int idx = threadIdx.x + i * 256;
-    if (idx < nvec) {
-      xv[i].v = *reinterpret_cast<const decltype(xv[i].v)*>(xr + idx * VN);
-      if (rr) rv[i].v = *reinterpret_cast<const decltype(rv[i].v)*>(rr + idx * VN);
+    if (idx < nvec && rr) rv[i].v = *reinterpret_cast<const decltype(rv[i].v)*>(rr + idx * VN);
+  }
+  if (slots == 1) {
+    Vec16<T> xv[MAXV];
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i) {
+      const int idx = threadIdx.x + i * 256;
+      if (idx < nvec) xv[i].v = *reinterpret_cast<const decltype(xv[i].v)*>(xr + idx * VN);
     }
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i)
+#pragma unroll
+      for (int j = 0; j < VN; ++j) val[i][j] = xv[i].get(j);
+  } else if constexpr (MAXV <= 4) {
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i)
+#pragma unroll
+      for (int j = 0; j < VN; ++j) val[i][j] = 0.f;
+    for (int k0 = 0; k0 < slots; k0 += 8) {
+      Vec16<T> sv[8][MAXV];
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+#pragma unroll
+        for (int i = 0; i < MAXV; ++i) {
+          const int idx = threadIdx.x + i * 256;
+          if (k0 + k < slots && idx < nvec)
+            sv[k][i].v = *reinterpret_cast<const decltype(sv[k][i].v)*>(xr + (k0 + k) * x_stride + idx * VN);
+        }
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (k0 + k < slots) {
+#pragma unroll
+          for (int i = 0; i < MAXV; ++i)
+#pragma unroll
+            for (int j = 0; j < VN; ++j) val[i][j] += sv[k][i].get(j);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i)
+#pragma unroll
+      for (int j = 0; j < VN; ++j) val[i][j] = round_to<T>(val[i][j]);
   }
   // the sums stay in registers (a thread's own vectors are all it needs after the reduction)
-  float val[MAXV][VN];
   float sq = 0.f;
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
@@ -84,7 +123,7 @@ rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* ou
     if (idx < nvec) {
 #pragma unroll
       for (int j = 0; j < VN; ++j) {
-        float v = xv[i].get(j);
+        float v = val[i][j];
         if (rr) v += rv[i].get(j);
         val[i][j] = v;
         sq += v * v;
@@ -124,7 +163,7 @@ rms_norm_vec_kernel(const T* x, T* residual, const W* __restrict__ weight, T* ou
 template <typename T, typename W>
 static int launch_rms(const void* x, void* residual, const void* weight, void* out,
                       const int32_t* rows, int n_out, int hidden, float eps, int64_t xs, int64_t rs,
-                      int64_t os, int write_residual, int vector_ok, hipStream_t stream) {
+                      int64_t os, int write_residual, int vector_ok, hipStream_t stream, int slots = 1) {
   const size_t shmem = (static_cast<size_t>(hidden) + 16) * sizeof(float);
   constexpr int VN = Vec16<T>::N;
   const T* xp = static_cast<const T*>(x);
@@ -133,9 +172,10 @@ static int launch_rms(const void* x, void* residual, const void* weight, void* o
   T* op = static_cast<T*>(out);
   if (vector_ok && hidden % VN == 0 && xs % VN == 0 && rs % VN == 0 && os % VN == 0) {
     const int per_thread = (hidden / VN + 255) / 256;
+    if (slots > 1 && per_thread > 4) return SE_ERR_SHAPE;   // rows summed on the fly: up to four vectors a thread
 #define SE_RMS(MAXV)                                                                             \
   rms_norm_vec_kernel<T, W, MAXV><<<n_out, 256, shmem, stream>>>(xp, rp, wp, op, rows, hidden, eps, \
-                                                                 xs, rs, os, write_residual)
+                                                                 xs, rs, os, write_residual, slots)
     if (per_thread <= 1) SE_RMS(1);
     else if (per_thread <= 2) SE_RMS(2);
     else if (per_thread <= 4) SE_RMS(4);
@@ -143,6 +183,7 @@ static int launch_rms(const void* x, void* residual, const void* weight, void* o
     else SE_RMS(16);
 #undef SE_RMS
   } else {
+    if (slots > 1) return SE_ERR_SHAPE;
     rms_norm_kernel<T, W><<<n_out, 256, shmem, stream>>>(xp, rp, wp, op, rows, hidden, eps, xs, rs, os,
                                                          write_residual);
   }
@@ -189,6 +230,28 @@ int se_rms_norm(const void* x, void* residual, const void* weight, void* out, co
                                      res_stride, out_stride, write_residual, vector_ok, stream);
   return launch_rms<bf16_t, bf16_t>(x, residual, weight, out, rows, n_out, hidden, eps, x_stride,
                                     res_stride, out_stride, write_residual, vector_ok, stream);
+}
+
+// The same with every input row the sum of `slots` consecutive rows of x (row r: rows r * slots ... of
+// x), added up in float in slot order and rounded to the storage type first: the sum over a token's
+// expert slots, done while the norm reads.  Sizes the wide kernel takes, up to four vectors a thread;
+// out must not be x.
+int se_rms_norm_slots(const void* x, void* residual, const void* weight, void* out, const int32_t* rows,
+                      int n_out, int hidden, float eps, int64_t x_stride, int64_t res_stride,
+                      int64_t out_stride, int write_residual, int dtype, int weight_dtype, int vector_ok,
+                      int slots, hipStream_t stream) {
+  if (n_out <= 0) return SE_OK;
+  if (hidden <= 0 || hidden > 15360 || slots < 1 || !vector_ok || x == out) return SE_ERR_SHAPE;
+  if (dtype == SE_F32) {
+    if (weight_dtype != SE_F32) return SE_ERR_SHAPE;
+    return launch_rms<float, float>(x, residual, weight, out, rows, n_out, hidden, eps, x_stride,
+                                    res_stride, out_stride, write_residual, vector_ok, stream, slots);
+  }
+  if (weight_dtype == SE_F32)
+    return launch_rms<bf16_t, float>(x, residual, weight, out, rows, n_out, hidden, eps, x_stride,
+                                     res_stride, out_stride, write_residual, vector_ok, stream, slots);
+  return launch_rms<bf16_t, bf16_t>(x, residual, weight, out, rows, n_out, hidden, eps, x_stride,
+                                    res_stride, out_stride, write_residual, vector_ok, stream, slots);
 }
 
 }  // extern "C"

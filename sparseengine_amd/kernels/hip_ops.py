@@ -65,6 +65,8 @@ _SIGNATURES = {
         "se_embedding": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "se_rms_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
                         c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p],
+        "se_rms_norm_slots": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float,
+                              c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "rope_kv": {
         "se_qk_norm_rope_store": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
@@ -195,12 +197,46 @@ class HipKernels:
         _check(_fn.get("norm", "se_embedding")(_ptr(ids), _ptr(table), _ptr(out), tokens, hidden,
                                                _code(out.dtype), _code(table.dtype), _stream()), "embedding")
 
-    def rms_norm(self, x, weight, eps: float, out, residual=None, rows=None, write_residual=True):
+    # rms_norm(slots=...) and moe_experts(sum_slots=False): the sum over a token's expert slots can be
+    # left to the norm that reads the feed-forward's result (one launch and one pass over memory fewer
+    # per layer); parts ask this flag before they hand a SlotSum on.
+    supports_slot_sums = True
+
+    def rms_norm(self, x, weight, eps: float, out, residual=None, rows=None, write_residual=True, slots: int = 1):
         """``out = norm(x (+ residual)) * weight``; with ``residual`` the rounded sum replaces it
         (unless ``write_residual`` is False).  ``rows`` (int32) selects input rows: ``out[j]`` is
-        the norm of row ``rows[j]``.  ``out`` may be ``x``."""
+        the norm of row ``rows[j]``.  ``out`` may be ``x``.  ``slots`` > 1: input row ``r`` is the
+        sum of rows ``r * slots ...`` of ``x`` (``[rows * slots, hidden]``, contiguous), added up in
+        float in slot order and rounded to the storage type first: the sum over a token's expert
+        slots done while the norm reads, bit for bit what a separate sum would give."""
         hidden = x.shape[-1]
         n_out = out.shape[0]
+        if slots > 1:
+            _require(x.dim() == 2 and x.is_contiguous() and x.shape[0] % slots == 0 and out.dim() == 2
+                     and out.data_ptr() != x.data_ptr() and out.dtype == x.dtype, "rms_norm: slot rows")
+            n_in = x.shape[0] // slots
+            if residual is not None:
+                _require(residual.shape == (n_in, hidden) and residual.dtype == x.dtype and residual.stride(1) == 1,
+                         "rms_norm: residual shape/dtype")
+            if rows is not None:
+                _i32(rows, "rows")
+                _require(rows.numel() == n_out, "rms_norm: rows/out mismatch")
+                write_residual = False
+            else:
+                _require(n_out == n_in, "rms_norm: out rows")
+            aligned = all(t is None or t.data_ptr() % 16 == 0 for t in (x, residual, weight, out))
+            status = _fn.get("norm", "se_rms_norm_slots")(
+                _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), n_out, hidden, float(eps),
+                x.stride(0), residual.stride(0) if residual is not None else 0, out.stride(0),
+                int(bool(write_residual)), _code(x.dtype), _code(weight.dtype), int(aligned), int(slots),
+                _stream()) if hidden <= 15360 else -1
+            if status == 0:
+                return
+            # sizes the fused kernel does not take: the sum first, then the norm of its result
+            summed = torch.empty(n_in, hidden, dtype=x.dtype, device=x.device)
+            _check(_fn.get("moe", "se_moe_sum")(_ptr(x), _ptr(summed), n_in, int(slots), hidden, _code(x.dtype),
+                                                _stream()), "slot sum")
+            x, slots = summed, 1
         _require(x.dim() == 2 and out.dim() == 2 and out.shape[1] == hidden, "rms_norm: x/out shapes")
         _require(x.stride(1) == 1 and out.stride(1) == 1, "rms_norm: rows must be dense")
         _require(weight.shape == (hidden,) and weight.is_contiguous(), "rms_norm: weight shape")
@@ -453,11 +489,14 @@ class HipKernels:
         return True
 
     def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, kernel=None, tile_rows=None,
-                    column_blocks=None, tiled: bool = False):
+                    column_blocks=None, tiled: bool = False, sum_slots: bool = True):
         """``out[t] = sum_k weights[t,k] * W2_e(silu(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``;
         ``w13 [E, 2I, h]`` holds gate rows then up rows, ``w2 [E, h, I]``.  ``tiled``: the tables
         have been through ``arrange_expert_weights``; row-major tables of sizes the matrix-core
         kernels take are put into tiles here, call by call (tests; the model arranges them once).
+        ``sum_slots=False``: the sum over a token's slots is left to the caller; the slots' results
+        ``[tokens * top_k, hidden]`` are returned (a view of the workspace, good until its next use) and
+        ``out`` is not written.
         ``kernel`` ("stream", "tall", "direct"), ``tile_rows`` and ``column_blocks`` override the
         choice of the matrix-core kernel and its tile (tests and measurements)."""
         tokens, hidden = x.shape
@@ -540,6 +579,8 @@ class HipKernels:
             _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                       _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
                       code, _stream()), "moe down")
+        if not sum_slots:      # the caller sums: [tokens * top_k, hidden], a token's slots one after the other
+            return ws.slot_out[:assignments]
         _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
                                             _stream()), "moe_sum")
 

@@ -42,6 +42,21 @@ class StateRequest:
     tensors: tuple[tuple[str, tuple[int, ...], torch.dtype | None], ...]
 
 
+class SlotSum:
+    """What a feed-forward hands on when the sum over a token's slots (its chosen experts) is left
+    to the reader: ``parts`` holds ``[tokens * slots, hidden]``, a token's slots one after the
+    other.  A part that says ``accepts_slot_sum`` takes it in place of ``[tokens, hidden]`` and adds
+    the slots up while it reads (a norm does: one kernel and one pass over memory fewer per layer);
+    a feed-forward is only asked for it when the part that reads its result accepts it."""
+
+    def __init__(self, parts: torch.Tensor, slots: int):
+        self.parts, self.slots = parts, int(slots)
+
+    @property
+    def shape(self):
+        return (self.parts.shape[0] // self.slots, self.parts.shape[1])
+
+
 class Part:
     """Base of mixers, feed-forwards, norms, position encodings and blocks."""
     kernel_libraries: tuple[str, ...] = ()

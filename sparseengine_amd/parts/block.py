@@ -28,16 +28,28 @@ class PreNormBlock(Part):
         request = getattr(self.mixer, "cache_request", None)
         return request() if request else None
 
-    def forward(self, fb, x, residual, cache_position: int, write_cache: bool):
-        """``x`` is consumed (normed in place); returns the new pair (x, residual)."""
+    @property
+    def accepts_slot_sum(self) -> bool:
+        """Whether ``x`` may come as a ``SlotSum`` (the first norm adds the slots up as it reads)."""
+        return bool(getattr(self.norm_mixer, "accepts_slot_sum", False))
+
+    @property
+    def can_defer_slot_sum(self) -> bool:
+        return bool(getattr(self.ffn, "can_defer_slot_sum", False))
+
+    def forward(self, fb, x, residual, cache_position: int, write_cache: bool, defer_slot_sum: bool = False):
+        """``x`` is consumed (normed in place); returns the new pair (x, residual).
+        ``defer_slot_sum``: whoever reads the returned ``x`` accepts a ``SlotSum``."""
         if residual is None:
             residual = fb.buffer("block.residual", x.shape)
             residual.copy_(x)
             self.norm_mixer.forward(fb, x)
         else:
-            self.norm_mixer.forward(fb, x, residual=residual)
+            x = self.norm_mixer.forward(fb, x, residual=residual)
         mixed = self.mixer.forward(fb, x, cache_position, write_cache)
         self.norm_ffn.forward(fb, mixed, residual=residual)
+        if defer_slot_sum and self.can_defer_slot_sum:
+            return self.ffn.forward(fb, mixed, defer_slot_sum=True), residual
         return self.ffn.forward(fb, mixed), residual
 
 

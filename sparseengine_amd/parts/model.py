@@ -63,10 +63,19 @@ class DecoderModel(Part):
         x = fb.buffer("model.hidden", (fb.num_tokens, spec.hidden_size))
         fb.kernels.embedding(fb.token_ids, self.embed.params["weight"], x)
         residual = None
+        final = len(spec.schedule) - 1
         for position, entry in enumerate(spec.schedule):
             own = entry.cache_from is None
-            x, residual = self.layers[entry.layer].forward(
-                fb, x, residual, position if own else entry.cache_from, own)
+            layer = self.layers[entry.layer]
+            # the sum over a token's expert slots may be left to whoever reads the layer's result:
+            # the next layer's first norm, or the final norm
+            reader = self.final_norm if position == final else self.layers[spec.schedule[position + 1].layer]
+            if (fb.taps is None and getattr(layer, "can_defer_slot_sum", False)
+                    and getattr(reader, "accepts_slot_sum", False)):
+                x, residual = layer.forward(fb, x, residual, position if own else entry.cache_from, own,
+                                            defer_slot_sum=True)
+            else:
+                x, residual = layer.forward(fb, x, residual, position if own else entry.cache_from, own)
             if fb.taps is not None:
                 fb.taps.setdefault("layer_out", []).append((x.float() + residual.float()))
         wanted = fb.want_index.numel()

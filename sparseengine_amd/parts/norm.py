@@ -6,7 +6,7 @@ the residual in float, stores the rounded sum as the new residual and norms the 
 from __future__ import annotations
 
 from ..config.specs import NormSpec
-from .base import NORMS, ParamDecl, Part
+from .base import NORMS, ParamDecl, Part, SlotSum
 
 
 class RMSNorm(Part):
@@ -19,14 +19,25 @@ class RMSNorm(Part):
     def param_decls(self):
         return {"weight": ParamDecl((self.hidden_size,))}
 
+    accepts_slot_sum = True     # ``x`` may be a ``SlotSum``: the slots are added up as they are read
+
     def forward(self, fb, x, out=None, residual=None):
-        """``out = norm(x (+ residual))``; the residual, if given, becomes ``x + residual``."""
+        """``out = norm(x (+ residual))``; the residual, if given, becomes ``x + residual``.
+        Returns ``out`` (``x`` itself unless ``out`` is given or ``x`` is a ``SlotSum``)."""
+        if isinstance(x, SlotSum):
+            out = fb.buffer("norm.of_slots", x.shape) if out is None else out
+            fb.kernels.rms_norm(x.parts, self.params["weight"], self.eps, out, residual=residual, slots=x.slots)
+            return out
         out = x if out is None else out
         fb.kernels.rms_norm(x, self.params["weight"], self.eps, out, residual=residual)
         return out
 
     def forward_rows(self, fb, x, residual, rows, out):
         """Norm of ``x[rows] (+ residual[rows])`` into ``out``; nothing else is written."""
+        if isinstance(x, SlotSum):
+            fb.kernels.rms_norm(x.parts, self.params["weight"], self.eps, out, residual=residual, rows=rows,
+                                slots=x.slots)
+            return out
         fb.kernels.rms_norm(x, self.params["weight"], self.eps, out, residual=residual, rows=rows)
         return out
 

@@ -73,3 +73,27 @@ def test_trace_run_program_on_the_emulated_kernels(tmp_path):
     got = traces.gather(records, logits)
     for rid, ref in expected.items():
         assert np.abs(got[rid] - ref).max() <= R.bound("float32", ref), rid
+
+
+@pytest.mark.parametrize("key,dtype", [("C_loud", "bfloat16"), ("A_loud", "float32")])
+def test_the_slot_sum_left_to_the_next_norm_changes_no_bit(tmp_path, key, dtype):
+    """Without taps the feed-forward hands its per-slot results on and the norm that reads them adds
+    them up (one launch fewer per layer); with taps the sum is a kernel of its own.  Same bits."""
+    from sparseengine_amd.engine.replay import replay_step
+    from sparseengine_amd.engine.runner import ModelRunner
+    from sparseengine_amd.parts.base import SlotSum
+    folder, requests, _, _ = model_for(tmp_path, key, [40, 3, 17])
+    records, peak = traces.mixed(requests, seed=1)
+    seen = []
+    with backends.use(backends.EmulatedBackend(guard="after")):
+        outs = []
+        for taps in (None, {}):
+            runner = ModelRunner.from_folder(folder, dtype=dtype, kv_page_size=16, num_kvcache_tokens=peak, max_num_seqs=4,
+                                             **backends.ACTIVE.runner_kwargs())
+            norm = runner.model.final_norm
+            rows = norm.forward_rows
+            norm.forward_rows = lambda fb, x, *a, _rows=rows: (seen.append(isinstance(x, SlotSum)), _rows(fb, x, *a))[1]
+            outs.append([replay_step(runner, rec, None, taps=None if taps is None else {}) for rec in records])
+    assert seen[0] is True and seen[-1] is False          # the first run deferred the sum, the second did not
+    for a, b in zip(*outs):
+        assert (a is None and b is None) or np.array_equal(a, b)

@@ -592,6 +592,42 @@ def test_skinny_linear(hip, rows, n, k):
     torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1.6e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,slots,hidden", [(1, 8, 3072), (5, 2, 256), (33, 8, 768), (7, 3, 200), (4, 11, 512), (3, 4, 20)])
+def test_norm_adds_up_slots_as_it_reads(hip, dtype, tokens, slots, hidden):
+    """``rms_norm(slots=k)`` is the slot sum followed by the norm, bit for bit: with a residual (which
+    it replaces by the sum), without one, and for chosen rows; in sizes the fused kernel takes and in
+    sizes that fall back to the two kernels."""
+    from sparseengine_amd.kernels.hip_ops import _fn, _ptr, _code, _stream
+    y = randn(tokens * slots, hidden, dtype=dtype, seed=60)
+    w = randn(hidden, dtype=dtype, seed=61)
+    res = randn(tokens, hidden, dtype=dtype, seed=62)
+    summed = torch.empty(tokens, hidden, dtype=dtype, device=DEV)
+    assert _fn.get("moe", "se_moe_sum")(_ptr(y), _ptr(summed), tokens, slots, hidden, _code(dtype), _stream()) == 0
+    ref_sum = y.view(tokens, slots, hidden).float()
+    acc = torch.zeros(tokens, hidden, device=DEV)
+    for k in range(slots):
+        acc += ref_sum[:, k]
+    assert torch.equal(summed, acc.to(dtype))
+    # with a residual
+    res_a, res_b = res.clone(), res.clone()
+    out_a = torch.empty_like(summed); out_b = torch.empty_like(summed)
+    hip.rms_norm(summed, w, 1e-5, out_a, residual=res_a)
+    hip.rms_norm(y, w, 1e-5, out_b, residual=res_b, slots=slots)
+    assert torch.equal(out_a, out_b) and torch.equal(res_a, res_b)
+    # without
+    hip.rms_norm(summed, w, 1e-5, out_a)
+    hip.rms_norm(y, w, 1e-5, out_b, slots=slots)
+    assert torch.equal(out_a, out_b)
+    # chosen rows: the residual is read, not written
+    rows = torch.tensor([tokens - 1, 0, tokens // 2], dtype=torch.int32, device=DEV)
+    pick_a = torch.empty(3, hidden, dtype=dtype, device=DEV); pick_b = torch.empty_like(pick_a)
+    res_c = res.clone()
+    hip.rms_norm(summed, w, 1e-5, pick_a, residual=res, rows=rows)
+    hip.rms_norm(y, w, 1e-5, pick_b, residual=res_c, rows=rows, slots=slots)
+    assert torch.equal(pick_a, pick_b) and torch.equal(res, res_c)
+
+
 def test_rounding_to_bfloat16_is_to_nearest_even(hip):
     """The kernels round float results to bfloat16 with the chip's conversion instruction: it has to
     give what the tensor library gives, ties (to even), overflow to infinity and infinities included.

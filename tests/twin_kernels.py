@@ -33,8 +33,16 @@ class TwinKernels:
     def embedding(self, ids, table, out):
         out.copy_(table[ids.long()])        # a float table under bfloat16 activations is rounded here
 
-    def rms_norm(self, x, weight, eps, out, residual=None, rows=None, write_residual=True):
+    supports_slot_sums = True
+
+    def rms_norm(self, x, weight, eps, out, residual=None, rows=None, write_residual=True, slots=1):
         z = x.float()
+        if slots > 1:       # a token's slots, added in float in slot order and rounded to the storage type
+            parts = z.view(-1, slots, z.shape[-1])
+            acc = torch.zeros_like(parts[:, 0])
+            for k in range(slots):
+                acc = acc + parts[:, k]
+            z = _r(acc, x.dtype)
         if residual is not None:
             z = z + residual.float()
         if rows is not None:
@@ -127,7 +135,7 @@ class TwinKernels:
         self.router_logits(x, weight, logits)
         self.router_topk(logits, bias, top_k, ids, weights, scoring=scoring, normalize=normalize, scaling=scaling)
 
-    def moe_experts(self, x, w13, w2, ids, weights, out, ws=None):
+    def moe_experts(self, x, w13, w2, ids, weights, out, ws=None, tiled=False, sum_slots=True):
         dt = x.dtype
         T, h = x.shape
         E, two_i, _ = w13.shape
@@ -144,6 +152,8 @@ class TwinKernels:
             act = _r(_r(gate * torch.sigmoid(gate), dt) * up, dt)
             y = (act @ w2[e].float().T) * weights[tok, slot, None]
             slot_out[tok, slot] = _r(y, dt)
+        if not sum_slots:       # the caller adds the slots up: [tokens * top_k, hidden] in the storage type
+            return slot_out.to(dt).view(T * K, h)
         out.copy_(slot_out.sum(1).to(dt))
 
     def silu_mul(self, x, out):
