@@ -1,6 +1,8 @@
 // Fused per-token attention input preparation for gfx950:
 //   flat QK RMSNorm (one statistic per token over all heads, optional)
-//   -> partial NeoX rotation of dims [0, R) of every q and k head (pairs (d, d + R/2))
+//   -> partial rotation of dims [0, R) of every q and k head: pairs (d, d + R/2) ("NeoX", pairing 0)
+//      or pairs (2 j, 2 j + 1) ("interleaved", pairing 1; the general kernel only); pair j turns by
+//      the angle whose cosine and sine are the table's entries j and R/2 + j
 //   -> q written back in place, k (normed, rotated) and v (raw) written to their cache page.
 //
 // Statistics, rsqrt and the rotation are float.  The flat norm rounds (x * inv_rms) to the
@@ -36,7 +38,7 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
                                           const W* __restrict__ k_weight, float eps, int heads,
                                           int kv_heads, int head_dim, int rotary_dim, T* cache,
                                           const int32_t* __restrict__ slots, int page_size,
-                                          int write_kv) {
+                                          int write_kv, int pairing) {
   // General sizes, one element at a time.  The token's whole q|k|v row is first brought into shared
   // memory (as float); everything after the barrier reads from there, so no global load waits
   // behind a store to the same row.
@@ -93,12 +95,16 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
       return round_to<T>(scaled * round_to<T>(to_float(weight[idx])));
     };
     float y;
-    if (d < half) {
-      y = normed(local) * cs[d] - normed(local + half) * cs[half + d];
-    } else if (d < rotary_dim) {
-      y = normed(local) * cs[d - half] + normed(local - half) * cs[d];
-    } else {
+    if (d >= rotary_dim) {
       y = normed(local);
+    } else if (pairing == 1) {   // neighbours: (2 j, 2 j + 1) turn by angle j
+      const int j = d >> 1;
+      y = (d & 1) ? normed(local) * cs[j] + normed(local - 1) * cs[half + j]
+                  : normed(local) * cs[j] - normed(local + 1) * cs[half + j];
+    } else if (d < half) {
+      y = normed(local) * cs[d] - normed(local + half) * cs[half + d];
+    } else {
+      y = normed(local) * cs[d - half] + normed(local - half) * cs[d];
     }
     const T stored = from_float<T>(y);
     src[c] = stored;
@@ -297,10 +303,10 @@ template <typename T, typename W>
 static int launch(void* qkv, int64_t row_stride, const int32_t* positions, const float* cos_sin,
                   const void* qw, const void* kw, float eps, int tokens, int heads, int kv_heads,
                   int head_dim, int rotary_dim, void* cache, const int32_t* slots, int page_size,
-                  int write_kv, int vector_ok, hipStream_t stream) {
+                  int write_kv, int vector_ok, int pairing, hipStream_t stream) {
   // wide path: 16-byte aligned rows, vectors that never straddle a head or a rotary boundary
   constexpr int VN = Vec16<T>::N;
-  const bool vector_path = vector_ok && head_dim % VN == 0 && (rotary_dim / 2) % VN == 0 && row_stride % VN == 0 &&
+  const bool vector_path = vector_ok && pairing == 0 && head_dim % VN == 0 && (rotary_dim / 2) % VN == 0 && row_stride % VN == 0 &&
                            (rotary_dim / 2) % 4 == 0 && (Vec16<W>::N <= VN);
   const int width = (heads + 2 * kv_heads) * head_dim;
   if (vector_path) {
@@ -324,7 +330,7 @@ static int launch(void* qkv, int64_t row_stride, const int32_t* positions, const
     qk_norm_rope_store_kernel<T, W><<<tokens, 256, shmem, stream>>>(
         static_cast<T*>(qkv), row_stride, positions, cos_sin, static_cast<const W*>(qw),
         static_cast<const W*>(kw), eps, heads, kv_heads, head_dim, rotary_dim, static_cast<T*>(cache),
-        slots, page_size, write_kv);
+        slots, page_size, write_kv, pairing);
   }
   SE_CHECK_LAUNCH();
   return SE_OK;
@@ -335,9 +341,10 @@ extern "C" int se_qk_norm_rope_store(void* qkv, int64_t row_stride, const int32_
                                      const void* k_weight, float eps, int tokens, int heads,
                                      int kv_heads, int head_dim, int rotary_dim, void* cache,
                                      const int32_t* slots, int page_size, int write_kv, int dtype,
-                                     int weight_dtype, int vector_ok, hipStream_t stream) {
+                                     int weight_dtype, int vector_ok, int pairing, hipStream_t stream) {
   if (tokens <= 0) return SE_OK;
   if (rotary_dim < 0 || rotary_dim % 2 || rotary_dim > head_dim) return SE_ERR_SHAPE;
+  if (pairing != 0 && pairing != 1) return SE_ERR_SHAPE;
   if ((q_weight == nullptr) != (k_weight == nullptr)) return SE_ERR_SHAPE;
   if (write_kv && (!cache || !slots || page_size <= 0)) return SE_ERR_SHAPE;
   if (static_cast<int64_t>(heads + 2 * kv_heads) * head_dim > 15360) return SE_ERR_SHAPE;  // row kept in LDS
@@ -345,13 +352,13 @@ extern "C" int se_qk_norm_rope_store(void* qkv, int64_t row_stride, const int32_
     if (q_weight && weight_dtype != SE_F32) return SE_ERR_SHAPE;
     return launch<float, float>(qkv, row_stride, positions, cos_sin, q_weight, k_weight, eps, tokens,
                                 heads, kv_heads, head_dim, rotary_dim, cache, slots, page_size,
-                                write_kv, vector_ok, stream);
+                                write_kv, vector_ok, pairing, stream);
   }
   if (q_weight && weight_dtype == SE_F32)
     return launch<bf16_t, float>(qkv, row_stride, positions, cos_sin, q_weight, k_weight, eps,
                                  tokens, heads, kv_heads, head_dim, rotary_dim, cache, slots,
-                                 page_size, write_kv, vector_ok, stream);
+                                 page_size, write_kv, vector_ok, pairing, stream);
   return launch<bf16_t, bf16_t>(qkv, row_stride, positions, cos_sin, q_weight, k_weight, eps, tokens,
                                 heads, kv_heads, head_dim, rotary_dim, cache, slots, page_size,
-                                write_kv, vector_ok, stream);
+                                write_kv, vector_ok, pairing, stream);
 }

@@ -71,7 +71,7 @@ _SIGNATURES = {
     "rope_kv": {
         "se_qk_norm_rope_store": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                   c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int,
-                                  c_int, c_int, c_int, c_int, c_void_p],
+                                  c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attention_generic": {
         "se_paged_attention_generic": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p,
@@ -260,10 +260,13 @@ class HipKernels:
             "rms_norm")
 
     # ------------------------------------------------------------------ attention inputs
+    ROTARY_PAIRINGS = {"neox": 0, "interleaved": 1}
+
     def qk_norm_rope_store(self, qkv, positions, cos_sin, q_weight, k_weight, eps, heads, kv_heads,
-                           head_dim, rotary_dim, cache=None, slots=None, page_size=0):
+                           head_dim, rotary_dim, cache=None, slots=None, page_size=0, pairing="neox"):
         """In place on ``qkv [T, (heads + 2 kv_heads) * head_dim]``: flat QK norm (if weights are
-        given), partial rotation by ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half), and
+        given), partial rotation by ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half; ``pairing``
+        "neox" turns dims ``(d, d + rotary_dim / 2)`` together, "interleaved" dims ``(2 j, 2 j + 1)``), and
         the write of k and v to ``cache [pages, 2, kv_heads, page_size, head_dim]`` at ``slots`` (the
         last two sizes are a page's geometry; the order of its elements is cache/layout.py's)."""
         tokens = qkv.shape[0]
@@ -278,6 +281,8 @@ class HipKernels:
         if q_weight is not None:
             _require(q_weight.shape == (heads * head_dim,) and k_weight.shape == (kv_heads * head_dim,)
                      and q_weight.dtype == k_weight.dtype, "qk norm weight shapes")
+        if pairing not in self.ROTARY_PAIRINGS:
+            raise ValueError(f"rotary pairing {pairing!r} is unknown ({', '.join(self.ROTARY_PAIRINGS)})")
         write_kv = cache is not None
         if write_kv:
             _i32(slots, "slots")
@@ -292,7 +297,7 @@ class HipKernels:
             _ptr(q_weight), _ptr(k_weight), float(eps), tokens, heads, kv_heads, head_dim, rotary_dim,
             _ptr(cache), _ptr(slots), page_size, int(write_kv), _code(qkv.dtype), wd,
             int(all(t is None or t.data_ptr() % 16 == 0 for t in (qkv, q_weight, k_weight, cache, cos_sin))),
-            _stream()), "qk_norm_rope_store")
+            self.ROTARY_PAIRINGS[pairing], _stream()), "qk_norm_rope_store")
 
     def paged_attention(self, q, cache, meta, out, scale: float, window: int = 0):
         """Causal attention of every token of the step against its request's pages.

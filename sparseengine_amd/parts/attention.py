@@ -60,7 +60,8 @@ class GQAAttention(Part):
         fb.kernels.qk_norm_rope_store(
             qkv, meta.positions, self.position.table, p.get("q_norm"), p.get("k_norm"), s.qk_norm_eps,
             s.num_heads, s.num_kv_heads, s.head_dim, self.position.rotary_dim,
-            cache if write_cache else None, meta.slots if write_cache else None, meta.page_size)
+            cache if write_cache else None, meta.slots if write_cache else None, meta.page_size,
+            pairing=getattr(self.position, "pairing", "neox"))
         attended = fb.buffer("attn.out", (T, self.q_width))
         q = qkv[:, :self.q_width].view(T, s.num_heads, s.head_dim)
         method = getattr(fb, "method", None)

@@ -81,17 +81,20 @@ def shared_table(key, build):
 
 
 class RotaryPosition(Part):
-    """Rotation of the leading ``rotary_dim`` dims of each head, NeoX pairing ``(d, d + R/2)``."""
+    """Rotation of the leading ``rotary_dim`` dims of each head; ``pairing`` "neox" turns dims
+    ``(d, d + R/2)`` together, "interleaved" dims ``(2 j, 2 j + 1)``; pair ``j`` by ``p * inv_freq[j]``."""
+    PAIRINGS = ("neox", "interleaved")
 
     def __init__(self, spec: RotarySpec, head_dim: int):
         if spec.rotary_dim % 2 or not 0 < spec.rotary_dim <= head_dim:
             raise ValueError(f"rotary_dim must be even and in (0, head_dim={head_dim}], got {spec.rotary_dim}")
-        if spec.pairing != "neox":
-            raise NotImplementedError(f"rotary pairing {spec.pairing!r} is not supported (neox)")
+        if spec.pairing not in self.PAIRINGS:
+            raise NotImplementedError(f"rotary pairing {spec.pairing!r} is not supported ({', '.join(self.PAIRINGS)})")
         if spec.max_position <= 0:
             raise ValueError("a rotary encoding needs max_position > 0")
         self.spec = spec
         self.rotary_dim = spec.rotary_dim
+        self.pairing = spec.pairing
         self.rows = spec.max_position
         self.table = None
 
@@ -112,6 +115,7 @@ class RotaryPosition(Part):
 
 class NoPosition(Part):
     rotary_dim = 0
+    pairing = "neox"
     table = None
 
     def __init__(self, spec=None, head_dim: int = 0):

@@ -55,6 +55,8 @@ def test_embedding_norm_rotation_and_cache_write(guard, twin):
             for shape in [(4, 2, 16, 8, True, 16), (6, 3, 32, 32, False, 16), (5, 5, 48, 16, True, 32),
                           (3, 1, 80, 0, False, 16), (48, 8, 128, 64, True, 64)]:
                 G.test_qk_norm_rope_store(hip, twin, dtype, *shape)
+            for shape in [(4, 2, 16, 8, True, 16), (6, 3, 32, 32, False, 16)]:
+                G.test_rotation_of_neighbouring_dims(hip, twin, dtype, *shape)
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page,window", [

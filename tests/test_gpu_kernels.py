@@ -104,7 +104,7 @@ def rope_table(max_pos, rotary_dim, theta):
 @pytest.mark.parametrize("heads,kv_heads,head_dim,rotary,norm,page", [
     (4, 2, 16, 8, True, 16), (6, 3, 32, 32, False, 16), (48, 8, 128, 64, True, 64),
     (5, 5, 48, 16, True, 32), (6, 1, 128, 64, True, 16), (3, 1, 80, 0, False, 16)])
-def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary, norm, page):
+def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary, norm, page, pairing="neox"):
     tokens, pages = 9, 7
     width = (heads + 2 * kv_heads) * head_dim
     qkv = randn(tokens, width, dtype=dtype, seed=3)
@@ -117,9 +117,18 @@ def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary,
     cache_h = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device=DEV)
     cache_t = cache_h.clone()
     a, b = qkv.clone(), qkv.clone()
-    hip.qk_norm_rope_store(a, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_h, slots, page)
-    twin.qk_norm_rope_store(b, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_t, slots, page)
+    hip.qk_norm_rope_store(a, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_h, slots, page,
+                           pairing=pairing)
+    twin.qk_norm_rope_store(b, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_t, slots, page,
+                            pairing=pairing)
     torch.testing.assert_close(a, b, **tol(dtype))
+    if pairing == "interleaved" and not norm and rotary:
+        # neighbours as complex numbers: the rotation is a multiplication by exp(i * angle) (a library routine)
+        q_in = qkv[:, :heads * head_dim].view(tokens, heads, head_dim)[..., :rotary].float()
+        angle = torch.atan2(table[positions.long(), rotary // 2:], table[positions.long(), :rotary // 2])      # [T, R/2]
+        turned = torch.view_as_real(torch.view_as_complex(q_in.reshape(tokens, heads, rotary // 2, 2).contiguous())
+                                    * torch.polar(torch.ones_like(angle), angle)[:, None, :]).reshape(tokens, heads, rotary)
+        torch.testing.assert_close(a[:, :heads * head_dim].view(tokens, heads, head_dim)[..., :rotary].float(), turned, **tol(dtype))
     torch.testing.assert_close(cache_h, cache_t, **tol(dtype))
     # v is never touched; without a norm the dims beyond the rotary part are bit-equal to the input
     assert torch.equal(a[:, (heads + kv_heads) * head_dim:], qkv[:, (heads + kv_heads) * head_dim:])
@@ -134,6 +143,14 @@ def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary,
             at = (torch.tensor([s // page]).to(DEV), torch.tensor([s % page]).to(DEV))
             assert torch.equal(layout.read_keys(cache_h, *at)[0], kq[t])
             assert torch.equal(layout.read_values(cache_h, *at)[0], a[t, (heads + kv_heads) * head_dim:].view(kv_heads, head_dim))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rotary,norm,page", [
+    (4, 2, 16, 8, True, 16), (6, 3, 32, 32, False, 16), (48, 8, 128, 64, False, 64), (5, 5, 48, 16, True, 32)])
+def test_rotation_of_neighbouring_dims(hip, twin, dtype, heads, kv_heads, head_dim, rotary, norm, page):
+    """The other pairing of a rotary encoding: dims (2 j, 2 j + 1) turn together."""
+    test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary, norm, page, pairing="interleaved")
 
 
 def make_paged(dtype, kv_heads, head_dim, page, lens, seed=0, extra_pages=3, window=0, q_lens=None):

@@ -114,6 +114,15 @@ def linear_rotary_angles(positions, rotary_dim: int, slope: float):
 POSITIONS.register("toy_linear_rotary", lambda spec, head_dim: LinearRotary(spec, head_dim))
 
 
+def neighbour_rope(x, cos, sin, rotary_dim: int):
+    """Plain rotation of dims ``(2 j, 2 j + 1)`` of each head by angle ``j``; ``x [T, heads, D]``."""
+    out = x.clone()
+    even, odd = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+    out[..., 0:rotary_dim:2] = even * cos[:, None, :] - odd * sin[:, None, :]
+    out[..., 1:rotary_dim:2] = odd * cos[:, None, :] + even * sin[:, None, :]
+    return out
+
+
 # ------------------------------------------------------------------ the architecture
 def parse(raw: dict) -> dict:
     return raw
@@ -129,7 +138,7 @@ def _layer_spec(cfg, layer) -> LayerSpec:
                                       max_position=cfg["max_position_embeddings"])
         elif layer["rotary_dim"]:
             rotary = RotarySpec(rotary_dim=layer["rotary_dim"], theta=cfg["rope_theta"],
-                                max_position=cfg["max_position_embeddings"])
+                                max_position=cfg["max_position_embeddings"], pairing=layer.get("pairing", "neox"))
         else:
             rotary = NoPositionSpec()
         mixer = AttentionSpec(num_heads=layer["heads"], num_kv_heads=layer["kv_heads"], head_dim=layer["head_dim"],
@@ -180,12 +189,14 @@ TOY_CONFIG = dict(
     architectures=["ToyForCausalLM"], model_type="toy", hidden_size=64, vocab_size=300, eps=1e-5, rope_theta=10000.0,
     max_position_embeddings=1024,
     layers=[
-        dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=16, qk_norm=True, ffn="dense", intermediate=96),
+        dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=16, pairing="interleaved", qk_norm=True,
+             ffn="dense", intermediate=96),
         dict(mixer="decay", state_size=12, decay=0.8, ffn="moe", experts=6, top_k=2, intermediate=40, scoring="softmax",
              bias=False, normalize=False, scaling=1.5),
         dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, ffn="moe", experts=4, top_k=3,
              intermediate=24),
         dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, ffn="dense", intermediate=48),
+        # (layer 0 turns neighbouring dims together, the others dims half a rotary width apart)
         dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=8, linear_rotary=0.05, ffn="sign",
              intermediate=20),
     ],
@@ -236,6 +247,9 @@ class PlainToy:
                 if layer.get("linear_rotary"):
                     angles = linear_rotary_angles(pos, R, layer["linear_rotary"])
                     q, k = P.partial_rope(q, angles.cos(), angles.sin(), R), P.partial_rope(k, angles.cos(), angles.sin(), R)
+                elif R and layer.get("pairing") == "interleaved":
+                    cos, sin = P.rope_angles(pos, R, cfg["rope_theta"])
+                    q, k = neighbour_rope(q, cos, sin, R), neighbour_rope(k, cos, sin, R)
                 elif R:
                     cos, sin = P.rope_angles(pos, R, cfg["rope_theta"])
                     q, k = P.partial_rope(q, cos, sin, R), P.partial_rope(k, cos, sin, R)

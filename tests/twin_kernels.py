@@ -54,7 +54,7 @@ class TwinKernels:
 
     # ------------------------------------------------------------------ attention inputs
     def qk_norm_rope_store(self, qkv, positions, cos_sin, q_weight, k_weight, eps, heads, kv_heads,
-                           head_dim, rotary_dim, cache=None, slots=None, page_size=0):
+                           head_dim, rotary_dim, cache=None, slots=None, page_size=0, pairing="neox"):
         T = qkv.shape[0]
         dt = qkv.dtype
         qw, kw = heads * head_dim, kv_heads * head_dim
@@ -73,6 +73,10 @@ class TwinKernels:
 
             def rot(x, n):
                 x = x.view(T, n, head_dim)
+                if pairing == "interleaved":     # neighbours (2 j, 2 j + 1) turn by angle j
+                    x1, x2 = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+                    turned = torch.stack((x1 * cos - x2 * sin, x2 * cos + x1 * sin), -1).reshape(T, n, rotary_dim)
+                    return torch.cat((turned, x[..., rotary_dim:]), -1).reshape(T, -1)
                 x1, x2 = x[..., :half], x[..., half:rotary_dim]
                 return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., rotary_dim:]), -1).reshape(T, -1)
             q, k = rot(q, heads), rot(k, kv_heads)
