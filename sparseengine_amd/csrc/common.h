@@ -171,6 +171,15 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 
 enum SeDtype { SE_F32 = 0, SE_BF16 = 1 };
 
+// What a gated feed-forward applies to its gate before the product with the up projection.
+enum SeActivation { SE_ACT_SILU = 0, SE_ACT_GELU_TANH = 1 };
+template <bool FAST_EXP>
+__device__ __forceinline__ float gate_activation(float g, int activation) {
+  if (activation == SE_ACT_GELU_TANH)     // 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))
+    return 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.f + (FAST_EXP ? __expf(-g) : expf(-g)));
+}
+
 // 16-byte vectors of storage elements
 template <typename T>
 struct Vec16;

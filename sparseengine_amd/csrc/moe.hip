@@ -327,7 +327,7 @@ __global__ void grouped_gemm_generic_kernel(const T* __restrict__ in, const T* _
                                             const int32_t* __restrict__ tile_expert,
                                             const int32_t* __restrict__ counters,
                                             const float* __restrict__ route_weight, int assignments,
-                                            int top_k, int N, int K) {
+                                            int top_k, int N, int K, int activation) {
   const int tile = blockIdx.y;
   if (tile >= counters[0]) return;  // uniform over the block
   __shared__ float xs[GG_M][GG_K + 1];
@@ -383,7 +383,7 @@ __global__ void grouped_gemm_generic_kernel(const T* __restrict__ in, const T* _
     if (MODE == 0) {
       const float gate = round_to<T>(g[j]);
       const float up = round_to<T>(u[j]);
-      const float act = round_to<T>(gate / (1.f + expf(-gate)));
+      const float act = round_to<T>(gate_activation<false>(gate, activation));
       y = act * up;
     } else {
       y = g[j] * route_weight[a];
@@ -437,14 +437,14 @@ moe_sum_vec_kernel(const T* __restrict__ y, T* __restrict__ out, int top_k, int 
   *reinterpret_cast<raw_t*>(out + t * hidden + c) = o.v;
 }
 
-// out[t, c] = silu(x[t, c]) * x[t, width + c] with the roundings of the fused expert path
+// out[t, c] = act(x[t, c]) * x[t, width + c] (act: silu or gelu) with the roundings of the fused expert path
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ out, int width) {
+__global__ void silu_mul_kernel(const T* __restrict__ x, T* __restrict__ out, int width, int activation) {
   const int64_t t = blockIdx.x;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     const float gate = to_float(x[t * 2 * width + c]);
     const float up = to_float(x[t * 2 * width + width + c]);
-    const float act = round_to<T>(gate / (1.f + expf(-gate)));
+    const float act = round_to<T>(gate_activation<false>(gate, activation));
     out[t * width + c] = from_float<T>(act * up);
   }
 }
@@ -531,14 +531,15 @@ int se_moe_align(const int32_t* ids, int assignments, int experts, int tile_rows
 int se_grouped_gemm_generic(const void* in, const void* w, void* out, const int32_t* sorted,
                             const int32_t* tile_expert, const int32_t* counters,
                             const float* route_weight, int assignments, int top_k, int N, int K,
-                            int max_tiles, int mode, int dtype, hipStream_t stream) {
+                            int max_tiles, int mode, int dtype, int activation, hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
   if (N <= 0 || K <= 0 || max_tiles <= 0 || max_tiles > 65535) return SE_ERR_SHAPE;
+  if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
   dim3 grid((N + GG_N - 1) / GG_N, max_tiles);
 #define SE_GG(T, MODE)                                                                          \
   grouped_gemm_generic_kernel<T, MODE><<<grid, 256, 0, stream>>>(                               \
       static_cast<const T*>(in), static_cast<const T*>(w), static_cast<T*>(out), sorted,        \
-      tile_expert, counters, route_weight, assignments, top_k, N, K)
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation)
   if (dtype == SE_F32) {
     if (mode == 0) SE_GG(float, 0); else SE_GG(float, 1);
   } else {
@@ -577,14 +578,15 @@ int se_moe_sum(const void* y, void* out, int tokens, int top_k, int hidden, int 
   return SE_OK;
 }
 
-int se_silu_mul(const void* x, void* out, int tokens, int width, int dtype, hipStream_t stream) {
+int se_silu_mul(const void* x, void* out, int tokens, int width, int dtype, int activation, hipStream_t stream) {
   if (tokens <= 0) return SE_OK;
+  if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
   if (dtype == SE_F32)
     silu_mul_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(x),
-                                                       static_cast<float*>(out), width);
+                                                       static_cast<float*>(out), width, activation);
   else
     silu_mul_kernel<bf16_t><<<tokens, 256, 0, stream>>>(static_cast<const bf16_t*>(x),
-                                                        static_cast<bf16_t*>(out), width);
+                                                        static_cast<bf16_t*>(out), width, activation);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

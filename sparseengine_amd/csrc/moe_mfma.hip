@@ -52,7 +52,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
                          const int32_t* __restrict__ tile_expert,
                          const int32_t* __restrict__ counters,
                          const float* __restrict__ route_weight, int assignments, int top_k, int N,
-                         int K, int max_tiles) {
+                         int K, int max_tiles, int activation) {
   constexpr int BM = 16 * MB;
   constexpr int BN = 16 * NB;
   constexpr int NBT = MODE == 0 ? 2 * NB : NB;  // weight blocks per wave: gate blocks, then up blocks
@@ -201,7 +201,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
         if (MODE == 0) {
           const float gate = round_to<bf16_t>(total[0][i]);
           const float up = round_to<bf16_t>(total[PARTS - 1][i]);
-          const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
+          const float act = round_to<bf16_t>(gate_activation<true>(gate, activation));
           v = act * up;
         } else if (MODE == 1) {
           v = total[0][i] * route_weight[a];
@@ -220,35 +220,35 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 template <int MODE, int MB, int NB, int U>
 static void launch_u(const void* in, const void* w, void* out, const int32_t* sorted,
                    const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
-                   int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
+                   int assignments, int top_k, int N, int K, int max_tiles, int activation, hipStream_t stream) {
   const int64_t items = static_cast<int64_t>(N / (16 * NB)) * max_tiles;
   const int grid = static_cast<int>((items + 7) / 8 * 8);
   grouped_gemm_mfma_kernel<MODE, MB, NB, U><<<grid, 256, 0, stream>>>(
       static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
-      tile_expert, counters, route_weight, assignments, top_k, N, K, max_tiles);
+      tile_expert, counters, route_weight, assignments, top_k, N, K, max_tiles, activation);
 }
 
 // steps of 32 per stage: as many as divide a wave's quarter of K, fewer for taller tiles (registers)
 template <int MODE, int MB, int NB>
 static void launch(const void* in, const void* w, void* out, const int32_t* sorted,
                    const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
-                   int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
+                   int assignments, int top_k, int N, int K, int max_tiles, int activation, hipStream_t stream) {
   constexpr int UMAX = MB == 1 ? 4 : (MB == 2 ? 2 : 0);
   const int quarter = K / 4;
   if (UMAX == 0) {
     launch_u<MODE, MB, NB, 0>(in, w, out, sorted, tile_expert, counters, route_weight, assignments, top_k,
-                              N, K, max_tiles, stream);
+                              N, K, max_tiles, activation, stream);
     return;
   }
   if (UMAX >= 4 && quarter % 128 == 0)
     launch_u<MODE, MB, NB, UMAX >= 4 ? 4 : 1>(in, w, out, sorted, tile_expert, counters, route_weight,
-                                              assignments, top_k, N, K, max_tiles, stream);
+                                              assignments, top_k, N, K, max_tiles, activation, stream);
   else if (UMAX >= 2 && quarter % 64 == 0)
     launch_u<MODE, MB, NB, UMAX >= 2 ? 2 : 1>(in, w, out, sorted, tile_expert, counters, route_weight,
-                                              assignments, top_k, N, K, max_tiles, stream);
+                                              assignments, top_k, N, K, max_tiles, activation, stream);
   else
     launch_u<MODE, MB, NB, 1>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                              top_k, N, K, max_tiles, stream);
+                              top_k, N, K, max_tiles, activation, stream);
 }
 
 // ---------------------------------------------------------------------------------------- //
@@ -271,7 +271,7 @@ grouped_gemm_tall_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
                          const int32_t* __restrict__ tile_expert,
                          const int32_t* __restrict__ counters,
                          const float* __restrict__ route_weight, int assignments, int top_k, int N,
-                         int K) {
+                         int K, int activation) {
   constexpr int BM = 16 * MB;
   constexpr int WROWS = 128;
   int tile, column_block;
@@ -390,7 +390,7 @@ grouped_gemm_tall_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
       for (int i = 0; i < 4; ++i) {
         const float gate = round_to<bf16_t>(acc[0][mb][i]);
         const float up = round_to<bf16_t>(acc[1][mb][i]);
-        const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
+        const float act = round_to<bf16_t>(gate_activation<true>(gate, activation));
         y[i] = float_to_bf16_bits(act * up);
       }
       uint2 packed;
@@ -416,16 +416,17 @@ grouped_gemm_tall_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, const int32_t* sorted,
                                     const int32_t* tile_expert, const int32_t* counters,
                                     const float* route_weight, int assignments, int top_k, int N,
-                                    int K, int max_tiles, int mode, int tile_rows, hipStream_t stream) {
+                                    int K, int max_tiles, int mode, int tile_rows, int activation, hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
   if (K <= 0 || K % (2 * TALL_BK) || N <= 0 || N % (mode == 0 ? 64 : 128)) return SE_ERR_SHAPE;
+  if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
   if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
   const int64_t items = static_cast<int64_t>(N / (mode == 0 ? 64 : 128)) * max_tiles;
   const int grid = static_cast<int>((items + 7) / 8 * 8);
 #define SE_TALL(MODE, MB)                                                                          \
   grouped_gemm_tall_kernel<MODE, MB><<<grid, 256, 0, stream>>>(                                    \
       static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
-      tile_expert, counters, route_weight, assignments, top_k, N, K)
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation)
   if (tile_rows == 64) { if (mode == 0) SE_TALL(0, 4); else SE_TALL(1, 4); }
   else return SE_ERR_SHAPE;
 #undef SE_TALL
@@ -465,7 +466,7 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
                          const int32_t* __restrict__ tile_expert,
                          const int32_t* __restrict__ counters,
                          const float* __restrict__ route_weight, int assignments, int top_k, int N,
-                         int K) {
+                         int K, int activation) {
   constexpr int OUT_COLS = MODE == 0 ? 128 : 256;
   constexpr int WAVES = BM / 16;                 // 4 or 8: each wavefront 64 rows x 64 weight rows
   constexpr int WCOLS = 4;                       // wave columns: the tile's 256 weight rows in 4 parts
@@ -595,7 +596,7 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
         for (int i = 0; i < 4; ++i) {
           const float gate = round_to<bf16_t>(acc[cb][mb][i]);
           const float up = round_to<bf16_t>(acc[cb + CB / 2][mb][i]);
-          const float act = round_to<bf16_t>(gate / (1.f + __expf(-gate)));
+          const float act = round_to<bf16_t>(gate_activation<true>(gate, activation));
           y[i] = float_to_bf16_bits(act * up);
         }
         uint2 packed;
@@ -623,7 +624,7 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 template <int MODE, int BM>
 static int launch_wide(const void* in, const void* w, void* out, const int32_t* sorted,
                        const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
-                       int assignments, int top_k, int N, int K, int max_tiles, hipStream_t stream) {
+                       int assignments, int top_k, int N, int K, int max_tiles, int activation, hipStream_t stream) {
   const int64_t items = static_cast<int64_t>(N / (MODE == 0 ? 128 : 256)) * max_tiles;
   const int grid = static_cast<int>((items + 7) / 8 * 8);
   constexpr size_t shared = WIDE_STAGES * (16 + BM / 16) * (WIDE_KSTEP / 32) * 1024 + BM * sizeof(int32_t);
@@ -636,29 +637,30 @@ static int launch_wide(const void* in, const void* w, void* out, const int32_t* 
   }
   grouped_gemm_wide_kernel<MODE, BM, WIDE_KSTEP><<<grid, 4 * BM, shared, stream>>>(
       static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
-      tile_expert, counters, route_weight, assignments, top_k, N, K);
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation);
   return SE_OK;
 }
 
 extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, const int32_t* sorted,
                                     const int32_t* tile_expert, const int32_t* counters,
                                     const float* route_weight, int assignments, int top_k, int N,
-                                    int K, int max_tiles, int mode, int tile_rows, hipStream_t stream) {
+                                    int K, int max_tiles, int mode, int tile_rows, int activation, hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
   if (K <= 0 || K % 64 || N <= 0 || N % (mode == 0 ? 128 : 256)) return SE_ERR_SHAPE;
+  if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
   if (tile_rows != 64 && tile_rows != 128) return SE_ERR_SHAPE;
   if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
   int status;
   if (mode == 0)
     status = tile_rows == 128 ? launch_wide<0, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                    top_k, N, K, max_tiles, stream)
+                                                    top_k, N, K, max_tiles, activation, stream)
                               : launch_wide<0, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                   top_k, N, K, max_tiles, stream);
+                                                   top_k, N, K, max_tiles, activation, stream);
   else
     status = tile_rows == 128 ? launch_wide<1, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                    top_k, N, K, max_tiles, stream)
+                                                    top_k, N, K, max_tiles, activation, stream)
                               : launch_wide<1, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                   top_k, N, K, max_tiles, stream);
+                                                   top_k, N, K, max_tiles, activation, stream);
   if (status != SE_OK) return status;
   SE_CHECK_LAUNCH();
   return SE_OK;
@@ -674,7 +676,7 @@ static void launch_dense(const void* x, const void* w, void* out, int rows, int 
   const int grid = static_cast<int>((items + 7) / 8 * 8);
   grouped_gemm_mfma_kernel<2, MB, 1, U, KW><<<grid, 64 * KW, 0, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), nullptr,
-      nullptr, nullptr, nullptr, rows, 1, N, K, tiles);
+      nullptr, nullptr, nullptr, rows, 1, N, K, tiles, 0);
 }
 
 template <int MB>
@@ -717,8 +719,9 @@ extern "C" int se_grouped_gemm_mfma(const void* in, const void* w, void* out, co
                                     const int32_t* tile_expert, const int32_t* counters,
                                     const float* route_weight, int assignments, int top_k, int N,
                                     int K, int max_tiles, int mode, int tile_rows, int col_blocks,
-                                    hipStream_t stream) {
+                                    int activation, hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
+  if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
   if (K <= 0 || K % 128 || N <= 0 || N % (16 * col_blocks)) return SE_ERR_SHAPE;
   if (max_tiles <= 0 || max_tiles > (1 << 22)) return SE_ERR_SHAPE;
   if (mode != 0 && mode != 1) return SE_ERR_SHAPE;
@@ -726,10 +729,10 @@ extern "C" int se_grouped_gemm_mfma(const void* in, const void* w, void* out, co
   if (tile_rows == 16 * MB && col_blocks == NB) {                                                   \
     if (mode == 0)                                                                                  \
       launch<0, MB, NB>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,      \
-                        top_k, N, K, max_tiles, stream);                                            \
+                        top_k, N, K, max_tiles, activation, stream);                                \
     else                                                                                            \
       launch<1, MB, NB>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,      \
-                        top_k, N, K, max_tiles, stream);                                            \
+                        top_k, N, K, max_tiles, activation, stream);                                \
     SE_CHECK_LAUNCH();                                                                              \
     return SE_OK;                                                                                   \
   }

@@ -99,19 +99,19 @@ _SIGNATURES = {
                                  c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_moe_align": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_grouped_gemm_generic": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_void_p],
         "se_moe_sum": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-        "se_silu_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "se_silu_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     },
     "moe_mfma": {
         "se_grouped_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "se_skinny_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_tall": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "sampling": {
         "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -493,9 +493,17 @@ class HipKernels:
                 w[first:first + 8].copy_(self.tile_expert_weights(w[first:first + 8]))
         return True
 
+    ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}      # what a gated feed-forward applies to its gate
+
+    def _activation(self, name: str) -> int:
+        if name not in self.ACTIVATIONS:
+            raise ValueError(f"activation {name!r} is unknown ({', '.join(self.ACTIVATIONS)})")
+        return self.ACTIVATIONS[name]
+
     def moe_experts(self, x, w13, w2, ids, weights, out, ws: MoeWorkspace, kernel=None, tile_rows=None,
-                    column_blocks=None, tiled: bool = False, sum_slots: bool = True):
-        """``out[t] = sum_k weights[t,k] * W2_e(silu(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``;
+                    column_blocks=None, tiled: bool = False, sum_slots: bool = True, activation: str = "silu"):
+        """``out[t] = sum_k weights[t,k] * W2_e(act(W1_e x_t) * W3_e x_t)``, ``e = ids[t,k]``, ``act`` silu
+        or the tanh form of gelu;
         ``w13 [E, 2I, h]`` holds gate rows then up rows, ``w2 [E, h, I]``.  ``tiled``: the tables
         have been through ``arrange_expert_weights``; row-major tables of sizes the matrix-core
         kernels take are put into tiles here, call by call (tests; the model arranges them once).
@@ -517,6 +525,7 @@ class HipKernels:
         _require(ws.fits(tokens, top_k, experts, hidden, inter, x.dtype), "moe workspace does not fit")
         assignments = tokens * top_k
         code = _code(x.dtype)
+        act = self._activation(activation)
         if self.takes_tiled_expert_weights(x.dtype, hidden, inter):
             if not tiled:
                 w13, w2 = self.tile_expert_weights(w13), self.tile_expert_weights(w2)
@@ -560,18 +569,18 @@ class HipKernels:
                     column_blocks = 2 if max_tiles * (inter // 32) >= 2048 else 1
                 _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                          column_blocks, _stream()), "moe gate-up (stream)", takes)
+                          column_blocks, act, _stream()), "moe gate-up (stream)", takes)
                 _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                          tile_rows, column_blocks, _stream()), "moe down (stream)", takes)
+                          tile_rows, column_blocks, act, _stream()), "moe down (stream)", takes)
             else:
                 gt = _fn.get("moe_mfma", "se_grouped_gemm_wide" if kernel == "direct" else "se_grouped_gemm_tall")
                 _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                          _stream()), f"moe gate-up ({kernel})", takes)
+                          act, _stream()), f"moe gate-up ({kernel})", takes)
                 _check(gt(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                          tile_rows, _stream()), f"moe down ({kernel})", takes)
+                          tile_rows, act, _stream()), f"moe down ({kernel})", takes)
         else:
             _require(not tiled, "the general expert kernel reads row-major tables")
             max_tiles = self._grouped_tiles(ids, experts, ws, 16)
@@ -580,10 +589,10 @@ class HipKernels:
             gg = _fn.get("moe", "se_grouped_gemm_generic")
             _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                       _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, code,
-                      _stream()), "moe gate-up")
+                      act, _stream()), "moe gate-up")
             _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                       _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                      code, _stream()), "moe down")
+                      code, act, _stream()), "moe down")
         if not sum_slots:      # the caller sums: [tokens * top_k, hidden], a token's slots one after the other
             return ws.slot_out[:assignments]
         _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
@@ -611,12 +620,13 @@ class HipKernels:
             return out
         return torch.mm(x, weight.t(), out=out)
 
-    def silu_mul(self, x, out):
+    def silu_mul(self, x, out, activation: str = "silu"):
+        """``out = act(x[:, :w]) * x[:, w:]``: the gated product of a dense feed-forward."""
         tokens, two_w = x.shape
         _require(x.is_contiguous() and out.is_contiguous() and out.shape == (tokens, two_w // 2)
                  and out.dtype == x.dtype, "silu_mul shapes")
         _check(_fn.get("moe", "se_silu_mul")(_ptr(x), _ptr(out), tokens, two_w // 2, _code(x.dtype),
-                                             _stream()), "silu_mul")
+                                             self._activation(activation), _stream()), "silu_mul")
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, temperature, top_k, top_p, seeds, out):

@@ -15,14 +15,17 @@ from .base import FEED_FORWARDS, ParamDecl, Part, SlotSum
 from .linear import linear
 
 
+ACTIVATIONS = ("silu", "gelu_tanh")      # what the kernels' epilogues can apply to a gate
+
+
 class RoutedExperts(Part):
     kernel_libraries = ("moe", "moe_mfma")
 
     def __init__(self, spec: MoESpec, hidden_size: int, chunk_tokens: int = 16384):
         if not 1 <= spec.top_k <= spec.num_experts:
             raise ValueError(f"top_k must be in [1, num_experts={spec.num_experts}], got {spec.top_k}")
-        if spec.activation != "silu":
-            raise NotImplementedError(f"expert activation {spec.activation!r} is not supported (silu)")
+        if spec.activation not in ACTIVATIONS:
+            raise NotImplementedError(f"expert activation {spec.activation!r} is not supported ({', '.join(ACTIVATIONS)})")
         if spec.scoring not in ("sigmoid", "softmax"):
             raise NotImplementedError(f"router scoring {spec.scoring!r} is not supported (sigmoid, softmax)")
         self.spec = spec
@@ -112,26 +115,24 @@ class RoutedExperts(Part):
         if fb.taps is not None:
             fb.taps.setdefault("router", []).append((ids.clone(), weights.clone()))
         if not sum_slots:
-            return fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws, tiled=self._tiled, sum_slots=False)
+            return fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws, tiled=self._tiled, sum_slots=False,
+                                          activation=s.activation)
         if w13.dtype == x.dtype:
-            if self._tiled:
-                fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws, tiled=True)
-            else:
-                fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws)
+            fb.kernels.moe_experts(x, w13, w2, ids, weights, out, ws, tiled=self._tiled, activation=s.activation)
         else:   # expert weights kept in float32 under a bfloat16 engine
             x32 = x.float()
             out32 = torch.empty_like(x32)
-            fb.kernels.moe_experts(x32, w13, w2, ids, weights, out32, ws)
+            fb.kernels.moe_experts(x32, w13, w2, ids, weights, out32, ws, activation=s.activation)
             out.copy_(out32)
 
 
 class DenseMLP(Part):
-    """``down(silu(gate x) * up x)``; ``gate_up`` holds the gate rows, then the up rows."""
+    """``down(act(gate x) * up x)``; ``gate_up`` holds the gate rows, then the up rows."""
     kernel_libraries = ("moe",)
 
     def __init__(self, spec: DenseMLPSpec, hidden_size: int, chunk_tokens: int = 16384):
-        if spec.activation != "silu":
-            raise NotImplementedError(f"activation {spec.activation!r} is not supported (silu)")
+        if spec.activation not in ACTIVATIONS:
+            raise NotImplementedError(f"activation {spec.activation!r} is not supported ({', '.join(ACTIVATIONS)})")
         self.spec = spec
         self.hidden_size = int(hidden_size)
 
@@ -143,7 +144,7 @@ class DenseMLP(Part):
         T, i = x.shape[0], self.spec.intermediate_size
         gate_up = linear(x, self.params["gate_up"], out=fb.buffer("mlp.gate_up", (T, 2 * i)), kernels=fb.kernels)
         act = fb.buffer("mlp.act", (T, i))
-        fb.kernels.silu_mul(gate_up, act)
+        fb.kernels.silu_mul(gate_up, act, activation=self.spec.activation)
         return linear(act, self.params["down"], out=fb.buffer("ffn.out", (T, self.hidden_size)), kernels=fb.kernels)
 
 

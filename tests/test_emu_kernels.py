@@ -111,6 +111,12 @@ def test_experts(guard, twin, tokens, hidden, inter, experts, k):
             G.test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k)
 
 
+def test_experts_with_the_other_activation(guard, twin):
+    with Emulated(guard=guard) as hip:
+        G.test_experts_with_the_other_activation(hip, twin, F32, 45, 96, 48, 16, 4)
+        G.test_experts_with_the_other_activation(hip, twin, BF16, 70, 256, 128, 4, 2)
+
+
 def test_slot_sum_dense_products_and_sampling(guard, twin):
     with Emulated(guard=guard) as hip:
         for dtype in (F32, BF16):

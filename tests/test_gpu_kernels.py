@@ -443,7 +443,7 @@ def test_moe_align_groups_every_assignment_once(hip):
     (2048, 256, 128, 64, 8),
     # hundreds of rows per expert: tiles of 128 rows x 256 weight rows
     (2048, 256, 128, 8, 8), (1000, 512, 384, 6, 3), (777, 768, 256, 3, 1)])
-def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
+def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k, activation="silu"):
     emulator_skips(tokens * k * hidden * inter, 1.2e9)
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     x = randn(tokens, hidden, dtype=dtype, seed=11)
@@ -454,19 +454,35 @@ def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k):
     weights = weights / weights.sum(-1, keepdim=True)
     ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, DEV)
     out_h = torch.empty_like(x); out_t = torch.empty_like(x)
-    hip.moe_experts(x, w13, w2, ids, weights, out_h, ws)
-    twin.moe_experts(x, w13, w2, ids, weights, out_t)
+    hip.moe_experts(x, w13, w2, ids, weights, out_h, ws, activation=activation)
+    twin.moe_experts(x, w13, w2, ids, weights, out_t, activation=activation)
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
     if dtype == torch.bfloat16 and hidden % 256 == 0 and inter % 128 == 0 and tokens <= 200:
         # every kernel and tile on a step that would not choose it (mostly padding): same result
         for kernel, rows in (("direct", 128), ("direct", 64), ("tall", 64), ("stream", 16), ("stream", 32)):
             out_w = torch.empty_like(x)
-            hip.moe_experts(x, w13, w2, ids, weights, out_w, ws, kernel=kernel, tile_rows=rows)
+            hip.moe_experts(x, w13, w2, ids, weights, out_w, ws, kernel=kernel, tile_rows=rows, activation=activation)
             torch.testing.assert_close(out_w, out_t, **tol(dtype))
-    if experts == 1:   # one expert, k = 1: a plain SwiGLU feed-forward
+    if experts == 1:   # one expert, k = 1: a plain gated feed-forward through library routines
         xf = x.float()
-        ref = (torch.nn.functional.silu(xf @ w13[0, :inter].float().T) * (xf @ w13[0, inter:].float().T)) @ w2[0].float().T
+        act = torch.nn.functional.silu if activation == "silu" else (lambda g: torch.nn.functional.gelu(g, approximate="tanh"))
+        ref = (act(xf @ w13[0, :inter].float().T) * (xf @ w13[0, inter:].float().T)) @ w2[0].float().T
         torch.testing.assert_close(out_h.float(), ref, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tokens,hidden,inter,experts,k", [(45, 96, 48, 16, 4), (9, 256, 128, 1, 1), (70, 256, 128, 4, 2),
+                                                      (300, 512, 384, 6, 3)])
+def test_experts_with_the_other_activation(hip, twin, dtype, tokens, hidden, inter, experts, k):
+    """gelu (tanh form) on the gate, in the general kernel and in every matrix-core kernel."""
+    test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k, activation="gelu_tanh")
+    x = randn(13, 2 * 72, dtype=dtype, seed=4)
+    a = torch.empty(13, 72, dtype=dtype, device=DEV); b = torch.empty_like(a)
+    hip.silu_mul(x, a, activation="gelu_tanh"); twin.silu_mul(x, b, activation="gelu_tanh")
+    torch.testing.assert_close(a, b, **tol(dtype))
+    torch.testing.assert_close(a.float(), torch.nn.functional.gelu(x[:, :72].float(), approximate="tanh") * x[:, 72:].float(), **tol(dtype))
+    with pytest.raises(ValueError, match="relu"):
+        hip.silu_mul(x, a, activation="relu")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -145,13 +145,14 @@ def _layer_spec(cfg, layer) -> LayerSpec:
                               scale=layer["head_dim"] ** -0.5, qk_norm="flat" if layer.get("qk_norm") else "none",
                               qk_norm_eps=cfg["eps"], window=layer.get("window"), position=rotary)
     if layer["ffn"] == "dense":
-        ffn = DenseMLPSpec(intermediate_size=layer["intermediate"])
+        ffn = DenseMLPSpec(intermediate_size=layer["intermediate"], activation=layer.get("activation", "silu"))
     elif layer["ffn"] == "sign":
         ffn = SignRoutedSpec(intermediate_size=layer["intermediate"])
     else:
         ffn = MoESpec(num_experts=layer["experts"], top_k=layer["top_k"], intermediate_size=layer["intermediate"],
                       scoring=layer.get("scoring", "sigmoid"), selection_bias=layer.get("bias", True),
-                      norm_topk_prob=layer.get("normalize", True), routed_scaling_factor=layer.get("scaling", 1.0))
+                      norm_topk_prob=layer.get("normalize", True), routed_scaling_factor=layer.get("scaling", 1.0),
+                      activation=layer.get("activation", "silu"))
     return LayerSpec(mixer=mixer, feed_forward=ffn, norm=NormSpec(eps=cfg["eps"]))
 
 
@@ -194,8 +195,9 @@ TOY_CONFIG = dict(
         dict(mixer="decay", state_size=12, decay=0.8, ffn="moe", experts=6, top_k=2, intermediate=40, scoring="softmax",
              bias=False, normalize=False, scaling=1.5),
         dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, ffn="moe", experts=4, top_k=3,
-             intermediate=24),
-        dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, ffn="dense", intermediate=48),
+             intermediate=24, activation="gelu_tanh"),
+        dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, ffn="dense", intermediate=48,
+             activation="gelu_tanh"),
         # (layer 0 turns neighbouring dims together, the others dims half a rotary width apart)
         dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=8, linear_rotary=0.05, ffn="sign",
              intermediate=20),
@@ -260,9 +262,11 @@ class PlainToy:
                 a = P.causal_gqa_attention(q, k, v, D ** -0.5, window=layer.get("window")).reshape(T, -1) @ w[p + "mixer.o"].T
             m, residual = P.add_rms_norm(a, residual, w[p + "norm_ffn.weight"], cfg["eps"])
             I = layer["intermediate"]
+            gelu = layer.get("activation") == "gelu_tanh"
             if layer["ffn"] == "dense":
                 gu = m @ w[p + "ffn.gate_up"].T
-                x = (torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]) @ w[p + "ffn.down"].T
+                gate = torch.nn.functional.gelu(gu[:, :I], approximate="tanh") if gelu else torch.nn.functional.silu(gu[:, :I])
+                x = (gate * gu[:, I:]) @ w[p + "ffn.down"].T
             elif layer["ffn"] == "sign":
                 choice = next(signs, None)
                 if choice is None:
@@ -280,6 +284,13 @@ class PlainToy:
                 if layer.get("normalize", True):
                     wts = wts / wts.sum(-1, keepdim=True)
                 wts = wts * layer.get("scaling", 1.0)
-                x = P.swiglu_experts(m, w[p + "ffn.w13"][:, :I], w[p + "ffn.w13"][:, I:], w[p + "ffn.w2"], ids, wts)
+                if gelu:      # the routed sum spelled out: the plain helper knows silu only
+                    x = torch.zeros_like(m)
+                    for t in range(T):
+                        for e, wt in zip(ids[t].tolist(), wts[t]):
+                            gate = torch.nn.functional.gelu(w[p + "ffn.w13"][e, :I] @ m[t], approximate="tanh")
+                            x[t] += wt * (w[p + "ffn.w2"][e] @ (gate * (w[p + "ffn.w13"][e, I:] @ m[t])))
+                else:
+                    x = P.swiglu_experts(m, w[p + "ffn.w13"][:, :I], w[p + "ffn.w13"][:, I:], w[p + "ffn.w2"], ids, wts)
         y, _ = P.add_rms_norm(x, residual, w["final_norm.weight"], cfg["eps"])
         return y @ w["head.weight"].T

@@ -139,7 +139,14 @@ class TwinKernels:
         self.router_logits(x, weight, logits)
         self.router_topk(logits, bias, top_k, ids, weights, scoring=scoring, normalize=normalize, scaling=scaling)
 
-    def moe_experts(self, x, w13, w2, ids, weights, out, ws=None, tiled=False, sum_slots=True):
+    @staticmethod
+    def _act(gate, activation):
+        if activation == "gelu_tanh":
+            return torch.nn.functional.gelu(gate, approximate="tanh")
+        assert activation == "silu"
+        return gate * torch.sigmoid(gate)
+
+    def moe_experts(self, x, w13, w2, ids, weights, out, ws=None, tiled=False, sum_slots=True, activation="silu"):
         dt = x.dtype
         T, h = x.shape
         E, two_i, _ = w13.shape
@@ -153,18 +160,18 @@ class TwinKernels:
                 continue
             gu = xf[tok] @ w13[e].float().T
             gate, up = _r(gu[:, :I], dt), _r(gu[:, I:], dt)
-            act = _r(_r(gate * torch.sigmoid(gate), dt) * up, dt)
+            act = _r(_r(self._act(gate, activation), dt) * up, dt)
             y = (act @ w2[e].float().T) * weights[tok, slot, None]
             slot_out[tok, slot] = _r(y, dt)
         if not sum_slots:       # the caller adds the slots up: [tokens * top_k, hidden] in the storage type
             return slot_out.to(dt).view(T * K, h)
         out.copy_(slot_out.sum(1).to(dt))
 
-    def silu_mul(self, x, out):
+    def silu_mul(self, x, out, activation="silu"):
         dt = x.dtype
         w = x.shape[1] // 2
         gate, up = x[:, :w].float(), x[:, w:].float()
-        out.copy_((_r(gate * torch.sigmoid(gate), dt) * up).to(dt))
+        out.copy_((_r(self._act(gate, activation), dt) * up).to(dt))
 
     # ------------------------------------------------------------------ sampling
     @staticmethod
