@@ -25,6 +25,7 @@
 // depend on its place in the tile or on what else is in the batch.
 // Requires K % 128 == 0 and N % BN == 0; other sizes take the general kernel in moe.hip.
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -486,11 +487,23 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   const int lane = tid & (SE_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / SE_WAVE);
   const int col = lane & 15, kgroup = lane >> 4;
-  const int wr = wave / WCOLS, wc = wave % WCOLS;   // the wave's 64 rows and its part of the weight rows
+  // wave (wr, wc): row blocks wr, RW + wr, 2 RW + wr, 3 RW + wr of the tile (16 rows each) and part wc of the weight rows
+  constexpr int RW = BM / 64;
+  const int wr = wave / WCOLS, wc = wave % WCOLS;
   const int expert = tile_expert[tile];
   const int n0 = column_block * OUT_COLS;
   if (tid < BM) rows[tid] = sorted[tile * BM + tid];
   __syncthreads();
+  // An expert's last tile is partly padding, which lies at its end.  Row blocks that are all padding are
+  // left out of the matrix work (with the tokens of a prompt agreeing on a few dozen experts every third
+  // tile is such a last tile); the row blocks alternate between the wave rows so that what is left is
+  // shared evenly.
+  int valid = 0;
+#pragma unroll
+  for (int r = 0; r < BM; r += SE_WAVE)
+    valid += __popcll(__ballot(rows[r + lane] < assignments));
+  const int live_blocks = __builtin_amdgcn_readfirstlane((valid + 15) / 16);
+  const int my_blocks = (live_blocks - wr + RW - 1) / RW;     // 0 .. 4, the same for the whole wave
 
   const int64_t w_rows = MODE == 0 ? 2 * static_cast<int64_t>(N) : N;
   const bf16_t* we = w + static_cast<int64_t>(expert) * w_rows * K;
@@ -548,38 +561,50 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 #pragma unroll
   for (int j = 0; j < WIDE_STAGES - 1; ++j)
     if (j < steps) issue(j);
-  for (int step = 0; step < steps; ++step) {
-    // this step's data: all but the loads of the steps after it must have come back
-    if (step + WIDE_STAGES - 2 < steps) {
-      __builtin_amdgcn_s_waitcnt(0x0F70 | ((WIDE_STAGES - 2) * HALVES * PAIRS));    // vmcnt((stages - 2) * loads per step)
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70);                               // vmcnt(0)
-    }
-    __builtin_amdgcn_s_barrier();   // everyone's part of the step is in; everyone has left step - 1
-    asm volatile("" ::: "memory");
-    if (step + WIDE_STAGES - 1 < steps) issue(step + WIDE_STAGES - 1);   // into the buffer step - 1 used
-    const uint4(*chunk)[64] = reinterpret_cast<const uint4(*)[64]>(wide_shared) + (step % WIDE_STAGES) * CHUNKS;
-#pragma unroll
-    for (int sub = 0; sub < HALVES; ++sub) {
-      uint4 bfrag[4];
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb) bfrag[mb] = chunk[HALVES * (16 + 4 * wr + mb) + sub][lane];
-#pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-        const uint4 afrag = chunk[HALVES * (CB * wc + cb) + sub][lane];
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-          acc[cb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, afrag),
-                                                               __builtin_bit_cast(bf16x8, bfrag[mb]),
-                                                               acc[cb][mb], 0, 0, 0);
+  // the loop over K for a wave with MBS live row blocks: every wave brings its chunks and meets the
+  // barriers, whatever it has to compute
+  auto run = [&](auto mbs_tag) {
+    constexpr int MBS = decltype(mbs_tag)::value;
+    for (int step = 0; step < steps; ++step) {
+      // this step's data: all but the loads of the steps after it must have come back
+      if (step + WIDE_STAGES - 2 < steps) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | ((WIDE_STAGES - 2) * HALVES * PAIRS));    // vmcnt((stages - 2) * loads per step)
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                               // vmcnt(0)
       }
+      __builtin_amdgcn_s_barrier();   // everyone's part of the step is in; everyone has left step - 1
+      asm volatile("" ::: "memory");
+      if (step + WIDE_STAGES - 1 < steps) issue(step + WIDE_STAGES - 1);   // into the buffer step - 1 used
+      const uint4(*chunk)[64] = reinterpret_cast<const uint4(*)[64]>(wide_shared) + (step % WIDE_STAGES) * CHUNKS;
+      if constexpr (MBS > 0) {
+#pragma unroll
+        for (int sub = 0; sub < HALVES; ++sub) {
+          uint4 bfrag[MBS];
+#pragma unroll
+          for (int mb = 0; mb < MBS; ++mb) bfrag[mb] = chunk[HALVES * (16 + RW * mb + wr) + sub][lane];
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) {
+            const uint4 afrag = chunk[HALVES * (CB * wc + cb) + sub][lane];
+#pragma unroll
+            for (int mb = 0; mb < MBS; ++mb)
+              acc[cb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, afrag),
+                                                                   __builtin_bit_cast(bf16x8, bfrag[mb]),
+                                                                   acc[cb][mb], 0, 0, 0);
+          }
+        }
+      }
+      asm volatile("" ::: "memory");
     }
-    asm volatile("" ::: "memory");
-  }
-  // lane (kgroup, col): acc[cb][mb][i] belongs to weight row 4 * kgroup + i of block cb, tile row 64 wr + 16 mb + col
+  };
+  if (my_blocks >= 4) run(std::integral_constant<int, 4>{});
+  else if (my_blocks == 3) run(std::integral_constant<int, 3>{});
+  else if (my_blocks == 2) run(std::integral_constant<int, 2>{});
+  else if (my_blocks == 1) run(std::integral_constant<int, 1>{});
+  else run(std::integral_constant<int, 0>{});
+  // lane (kgroup, col): acc[cb][mb][i] belongs to weight row 4 * kgroup + i of block cb, tile row 16 (RW mb + wr) + col
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
-    const int a = rows[64 * wr + 16 * mb + col];
+    const int a = rows[16 * (RW * mb + wr) + col];
     if (a >= assignments) continue;
     bf16_t* o_row = out + static_cast<int64_t>(a) * N + n0 + 4 * kgroup;
     if (MODE == 0) {
@@ -588,7 +613,7 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
       // [column % 8], like the expert tables), tile (sorted row block, column / 32): the down launch
       // then loads it as contiguous kilobytes instead of 64 bytes from each of 16 rows.  Rows of
       // padding are not written; what the down launch computes from them is not stored.
-      bf16_t* t_row = out + (static_cast<int64_t>(tile) * (BM / 16) + 4 * wr + mb) * (N / 32) * 512 + col * 8;
+      bf16_t* t_row = out + (static_cast<int64_t>(tile) * (BM / 16) + RW * mb + wr) * (N / 32) * 512 + col * 8;
 #pragma unroll
       for (int cb = 0; cb < CB / 2; ++cb) {
         uint16_t y[4];
@@ -679,25 +704,35 @@ static void launch_dense(const void* x, const void* w, void* out, int rows, int 
       nullptr, nullptr, nullptr, rows, 1, N, K, tiles, 0);
 }
 
-template <int MB>
-static void dense_by_split(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
-                           hipStream_t stream) {
-  // steps of 32 per stage of the kernel's loop; with one weight block per wave even 64 rows leave
-  // registers for two stages in flight
-  constexpr int UMAX = MB == 1 ? 4 : 2;
-  constexpr int STAGE = 32 * UMAX;
+// One choice of the stage depth U: K is split over 4, 8 or 16 wavefronts (until a few thousand are
+// in flight) if a wavefront's share of K is whole stages; false if it is not.
+template <int MB, int U>
+static bool dense_with_stage(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
+                             hipStream_t stream) {
+  constexpr int STAGE = 32 * U;
   const int64_t blocks = static_cast<int64_t>(N / 16) * tiles;
   int kw = 4;
   while (kw < 16 && blocks * kw < 3072 && K % (2 * kw * STAGE) == 0) kw *= 2;
-  if (K % (kw * STAGE) == 0) {
-    if (kw == 4) launch_dense<MB, 4, UMAX>(x, w, out, rows, N, K, tiles, stream);
-    else if (kw == 8) launch_dense<MB, 8, UMAX>(x, w, out, rows, N, K, tiles, stream);
-    else launch_dense<MB, 16, UMAX>(x, w, out, rows, N, K, tiles, stream);
-  } else if (UMAX >= 2 && K % (4 * 64) == 0) {
-    launch_dense<MB, 4, UMAX >= 2 ? 2 : 1>(x, w, out, rows, N, K, tiles, stream);
-  } else {   // K % 128 == 0 always holds here
-    launch_dense<MB, 4, 1>(x, w, out, rows, N, K, tiles, stream);
+  if (K % (kw * STAGE)) return false;
+  if (kw == 4) launch_dense<MB, 4, U>(x, w, out, rows, N, K, tiles, stream);
+  else if (kw == 8) launch_dense<MB, 8, U>(x, w, out, rows, N, K, tiles, stream);
+  else launch_dense<MB, 16, U>(x, w, out, rows, N, K, tiles, stream);
+  return true;
+}
+
+template <int MB>
+static void dense_by_split(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
+                           hipStream_t stream) {
+  // Two stages of a wavefront are in flight at a time, so the deeper the stage the more bytes it
+  // has under way: with up to 16 rows a stage of six steps (96 registers for both sets) brings a
+  // share of 384 along K (MiniMax-M2's qkv and output projections) in one round trip instead of
+  // three.  With one weight block per wavefront even 64 rows leave registers for stages of two.
+  if constexpr (MB == 1) {
+    if (dense_with_stage<MB, 6>(x, w, out, rows, N, K, tiles, stream)) return;
+    if (dense_with_stage<MB, 4>(x, w, out, rows, N, K, tiles, stream)) return;
   }
+  if (dense_with_stage<MB, 2>(x, w, out, rows, N, K, tiles, stream)) return;
+  dense_with_stage<MB, 1>(x, w, out, rows, N, K, tiles, stream);   // K % 128 == 0 always holds here
 }
 
 extern "C" int se_skinny_gemm_mfma(const void* x, const void* w, void* out, int rows, int N, int K,

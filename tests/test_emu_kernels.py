@@ -111,6 +111,12 @@ def test_experts(guard, twin, tokens, hidden, inter, experts, k):
             G.test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k)
 
 
+def test_wide_tiles_leave_out_row_blocks_of_padding(guard, twin):
+    with Emulated(guard=guard) as hip:
+        G.test_wide_tiles_leave_out_row_blocks_of_padding(hip, twin, [1, 16, 17, 47, 48, 49, 64, 65, 96, 111, 112, 113, 128, 129, 0])
+        G.test_wide_tiles_leave_out_row_blocks_of_padding(hip, twin, [128, 0, 0, 3])
+
+
 def test_experts_with_the_other_activation(guard, twin):
     with Emulated(guard=guard) as hip:
         G.test_experts_with_the_other_activation(hip, twin, F32, 45, 96, 48, 16, 4)
@@ -121,7 +127,8 @@ def test_slot_sum_dense_products_and_sampling(guard, twin):
     with Emulated(guard=guard) as hip:
         for dtype in (F32, BF16):
             G.test_silu_mul(hip, twin, dtype)
-        for shape in [(16, 256, 128), (17, 48, 256), (33, 1024, 384), (5, 50, 128), (3, 64, 96), (1, 512, 1024)]:
+        for shape in [(16, 256, 128), (17, 48, 256), (33, 1024, 384), (5, 50, 128), (3, 64, 96), (1, 512, 1024), (7, 64, 768), (16, 48, 1536),
+                      (2, 32, 3072)]:
             G.test_skinny_linear(hip, *shape)
         G.test_rounding_to_bfloat16_is_to_nearest_even(hip)
         G.test_expert_tables_arranged_in_place_are_the_tiled_copy(hip, twin)

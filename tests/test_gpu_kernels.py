@@ -470,6 +470,31 @@ def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k, activa
         torch.testing.assert_close(out_h.float(), ref, **tol(dtype))
 
 
+@pytest.mark.parametrize("counts", [[1, 16, 17, 47, 48, 49, 64, 65, 96, 111, 112, 113, 128, 129, 270, 0],
+                                    [128, 0, 0, 3], [200, 130, 80, 33, 2, 700]])
+def test_wide_tiles_leave_out_row_blocks_of_padding(hip, twin, counts):
+    """The wide expert kernel skips the row blocks of a tile that hold no row: experts with every
+    number of rows around the edges of the 16-row blocks of a 128-row tile, one slot per token so that
+    the counts are exact.  Against the twin, in both tile heights."""
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    hidden, inter, experts, tokens = 256, 128, len(counts), sum(counts)
+    emulator_skips(tokens * hidden * inter, 1.2e8)
+    dtype = torch.bfloat16
+    x = randn(tokens, hidden, dtype=dtype, seed=21)
+    w13 = randn(experts, 2 * inter, hidden, dtype=dtype, scale=hidden ** -0.5, seed=22)
+    w2 = randn(experts, hidden, inter, dtype=dtype, scale=inter ** -0.5, seed=23)
+    order = torch.randperm(tokens, generator=torch.Generator().manual_seed(24))
+    ids = torch.repeat_interleave(torch.arange(experts), torch.tensor(counts))[order].view(tokens, 1).to(torch.int32).to(DEV)
+    weights = (0.5 + torch.rand(tokens, 1, generator=torch.Generator().manual_seed(25))).to(DEV)
+    ws = MoeWorkspace(tokens, 1, experts, hidden, inter, dtype, DEV)
+    out_t = torch.empty_like(x)
+    twin.moe_experts(x, w13, w2, ids, weights, out_t)
+    for rows in (128, 64):
+        out_h = torch.full_like(x, float("nan"))
+        hip.moe_experts(x, w13, w2, ids, weights, out_h, ws, kernel="direct", tile_rows=rows)
+        torch.testing.assert_close(out_h, out_t, **tol(dtype))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("tokens,hidden,inter,experts,k", [(45, 96, 48, 16, 4), (9, 256, 128, 1, 1), (70, 256, 128, 4, 2),
                                                       (300, 512, 384, 6, 3)])
@@ -613,7 +638,8 @@ def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, p
 
 
 @pytest.mark.parametrize("rows,n,k", [(1, 8192, 3072), (8, 3072, 6144), (16, 256, 128), (17, 48, 256), (33, 1024, 384),
-                                      (64, 200064, 3072), (5, 50, 128), (3, 64, 96)])
+                                      (64, 200064, 3072), (5, 50, 128), (3, 64, 96),
+                                      (7, 64, 768), (16, 48, 1536), (2, 32, 3072), (20, 64, 768)])   # stages of six steps, K over 4, 8, 16 wavefronts
 def test_skinny_linear(hip, rows, n, k):
     """Few rows against a large matrix: the streaming kernel where its sizes fit, the library otherwise."""
     emulator_skips(rows * n * k, 4e8)
