@@ -373,7 +373,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2_rne(float lo, float hi) {   // o
   }
 
 template <int DSTEPS, int RT, int NS>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                              const bf16_t* __restrict__ cache,
                              const int32_t* __restrict__ block_table, int bt_stride,
@@ -478,18 +478,30 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     for (int ds = 0; ds < DSTEPS; ++ds)
       asm volatile("" : "+v"(qf[rt][ds].x), "+v"(qf[rt][ds].y), "+v"(qf[rt][ds].z), "+v"(qf[rt][ds].w));
 
-  // Waves 0 and 1 bring the two key blocks of a step, waves 2 and 3 one half of the value dims each:
+  // Waves 0 and 1 bring sixteen keys of a step each, waves 2 and 3 one half of the value dims each:
   // wave w fills chunks w * DSTEPS ... of a stage.  Steps are issued in order, so a lane follows its
   // key's page and place in the page by adding 32 (no division in the loop); a key past the block's
   // last one is replaced by that one (values: by its group of eight).
+  // The sixteen keys of a key chunk are consecutive ones, 256 contiguous bytes per group of eight
+  // dims (whole cache lines; the score layout wants keys 0-3, 8-11, 16-19, 24-27 in one operand and
+  // the others in the second, and chunks loaded in that order would take every line in two halves,
+  // by two waves).  The operands are gathered when they are read: row n of key block b is key
+  // 8 (n / 4) + n % 4 + 4 b.  Wave 1 brings its keys with bit 2 of their place flipped, so that the
+  // sixteen lanes of a read, half of which look into each chunk, fall on sixteen different bank groups.
   const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(&stage[0][0][0]));
   const bool loads_keys = wave < 2;
-  const int lane_key = loads_keys ? 8 * (n >> 2) + (n & 3) + 4 * wave : 8 * g;
+  const int lane_key = loads_keys ? 16 * wave + (n ^ (4 * wave)) : 8 * g;
   const int clamp_key = loads_keys ? kmax : (kmax & ~7);
   const int clamp_page = clamp_key / page_size, clamp_off = clamp_key % page_size;
   // a lane's key (values: its group of eight) wholly below `low_key` is replaced by that one's
   const int low_clamp = loads_keys ? low_key : (low_key & ~7);
   const int low_page = low_clamp / page_size, low_off = low_clamp % page_size;
+  int key_at[2];     // where the lane's vector of key block b lies among a stage's vectors, for the first 32 dims
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int key = 8 * (n >> 2) + (n & 3) + 4 * b, half = key >> 4;
+    key_at[b] = half * DSTEPS * 64 + 16 * g + ((key & 15) ^ (4 * half));
+  }
   int next_key = k_first + lane_key;                     // the lane's key of the next step to be issued
   int next_page = next_key / page_size, next_off = next_key % page_size;
   // keys lie [head_dim / 8][page_size][8], values [page_size / 8][head_dim][8]: sixteen lanes of a
@@ -534,8 +546,9 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 #pragma unroll
     for (int j = 1; j < NS - 1; ++j)
       if (j < nsteps) issue(j);
-    for (int step = 0; step < nsteps; ++step) {
-      const int k0 = k_first + 32 * step;
+    // What every wave does at the start of a step, whatever it computes then: wait for the step's data,
+    // meet the others, issue the loads of the step NS - 1 ahead.
+    auto begin_step = [&](int step) {
       // this step's data: all but the loads of the NS - 2 steps after it must have come back
       if (step + NS - 2 < nsteps) {
         __builtin_amdgcn_s_waitcnt(0x0F70 | ((NS - 2) * DSTEPS));     // vmcnt((NS - 2) * DSTEPS)
@@ -556,6 +569,10 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
         }
         issue(step + NS - 1);   // into the buffer that step - 1 has used
       }
+    };
+    // A step in full: the rows' ranges of keys, the reference maxima and the end of the cache all looked at.
+    auto whole_step = [&](int step) {
+      const int k0 = k_first + 32 * step;
       if (k0 <= wave_hi && (window <= 0 || k0 + 31 > wave_lo - window)) {
         const uint4(*buf)[64] = stage[step % NS];
         floatx4 s[RT][2];
@@ -565,7 +582,7 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
         for (int ds = 0; ds < DSTEPS; ++ds)
 #pragma unroll
           for (int b = 0; b < 2; ++b) {
-            const uint4 kf = buf[b * DSTEPS + ds][lane];
+            const uint4 kf = (&buf[0][0])[key_at[b] + 64 * ds];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
               s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
@@ -608,7 +625,84 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
           }
         }
       }
+    };
+    // Most steps of a long context lie before every row's own position, inside every row's window and
+    // before the block's last key, and raise no row's maximum beyond the slack: steps [plain_begin,
+    // plain_end) are tried without masks, without the exchange of maxima between lanes and, above all,
+    // without a path that rescales the accumulators.  (With that path inside the loop the compiler keeps
+    // the accumulators in two sets of registers and copies all 64 of them between the sets in every
+    // step; vector instructions, not matrix instructions, are what this kernel waits for.)  A step that
+    // would raise a maximum leaves the loop before it has touched anything and is done in full.
+    const int plain_limit = min(wave_lo, kmax) - 31;              // last first-key of a plain step
+    const int plain_end = plain_limit >= k_first ? min(nsteps, (plain_limit - k_first) / 32 + 1) : 0;
+    const int plain_begin =
+        window > 0 && wave_hi - window >= k_first ? (wave_hi - window - k_first) / 32 + 1 : 0;
+    int step = 0;
+    while (step < nsteps) {
+      bool begun = false;     // the step's data is in and its barrier met
+      if (step >= plain_begin && step < plain_end) {
+        for (; step < plain_end; ++step) {
+          begin_step(step);
+          const uint4(*buf)[64] = stage[step % NS];
+          floatx4 s[RT][2];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ds = 0; ds < DSTEPS; ++ds)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+              const uint4 kf = (&buf[0][0])[key_at[b] + 64 * ds];
+#pragma unroll
+              for (int rt = 0; rt < RT; ++rt)
+                s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
+                                                                   __builtin_bit_cast(bf16x8, qf[rt][ds]),
+                                                                   s[rt][b], 0, 0, 0);
+            }
+          // a lane looks at its own eight keys only: any lane of a row that sees the maximum raised says so
+          bool over = false;
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            const float m = max_bare(max3_bare(s[rt][0][0], s[rt][0][1], s[rt][0][2]),
+                                     max3_bare(max3_bare(s[rt][0][3], s[rt][1][0], s[rt][1][1]), s[rt][1][2], s[rt][1][3]));
+            over = over || !(m * scale_log2e <= run_max[rt] + SOFTMAX_SLACK);   // also with no maximum yet
+          }
+          if (__builtin_expect(__builtin_amdgcn_ballot_w64(over) != 0, 0)) {
+            begun = true;
+            break;
+          }
+          uint4 pf[RT];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            float v[8];
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              v[j] = __builtin_amdgcn_exp2f(fmaf(s[rt][j >> 2][j & 3], scale_log2e, -run_max[rt]));
+              sum += v[j];
+            }
+            run_sum[rt] += sum;
+            pf[rt].x = pack_bf16x2_rne(v[0], v[1]);
+            pf[rt].y = pack_bf16x2_rne(v[2], v[3]);
+            pf[rt].z = pack_bf16x2_rne(v[4], v[5]);
+            pf[rt].w = pack_bf16x2_rne(v[6], v[7]);
+          }
+#pragma unroll
+          for (int db = 0; db < DBLOCKS; ++db) {
+            const uint4 vf = buf[2 * DSTEPS + db][lane];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
+                                                                 __builtin_bit_cast(bf16x8, pf[rt]),
+                                                                 o[rt][db], 0, 0, 0);
+          }
+          asm volatile("" ::: "memory");
+        }
+        if (!begun) continue;     // the plain steps are done
+      }
+      if (!begun) begin_step(step);
+      whole_step(step);
       asm volatile("" ::: "memory");
+      ++step;
     }
   }
 

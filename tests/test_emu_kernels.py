@@ -88,6 +88,12 @@ def test_attention_prompt_portions(guard, twin, shape):
         G.test_paged_attention_prompt_portions(hip, twin, *shape)
 
 
+def test_prompt_attention_with_maxima_that_keep_rising(guard, twin):
+    with Emulated(guard=guard) as hip:
+        G.test_prompt_attention_with_maxima_that_keep_rising(hip, twin, 8, 2, 64, 16, 0, 700, 300)
+        G.test_prompt_attention_with_maxima_that_keep_rising(hip, twin, 8, 4, 32, 8, 500, 900, 260)
+
+
 def test_router(guard, twin):
     with Emulated(guard=guard) as hip:
         for dtype in (F32, BF16):

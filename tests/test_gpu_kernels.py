@@ -637,6 +637,44 @@ def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, p
         torch.testing.assert_close(out_h[t].float(), ref, **tol(dtype))
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page,window,ctx,q_len", [
+    (8, 2, 64, 16, 0, 700, 300), (6, 1, 128, 64, 0, 1500, 200), (8, 4, 32, 8, 500, 900, 260)])
+def test_prompt_attention_with_maxima_that_keep_rising(hip, twin, heads, kv_heads, head_dim, page, window, ctx, q_len):
+    """The shared-memory kernel runs the steps that need no mask in a loop of its own and leaves it when
+    a step would raise a row's maximum beyond its slack.  Here the maxima rise again and again deep
+    inside that range: every query has a large component along one direction, and keys every 97
+    positions lie along it, each longer than the one before (scores about 6, 12, 18, ... above the
+    rest), so a row's answer is nearly the value of the last such key it can see."""
+    emulator_skips(q_len * ctx * heads * head_dim, 2.5e9)
+    dtype = torch.bfloat16
+    cache, table = make_paged(dtype, kv_heads, head_dim, page, [ctx], seed=7, window=window, q_lens=[q_len])
+    direction = torch.ones(head_dim) / head_dim ** 0.5
+    marks = list(range(40, ctx, 97))
+    for i, pos in enumerate(marks):
+        entry = int(table[0, pos // page])
+        if entry >= 0:
+            key = (direction * (i + 1) * 6.0 * head_dim ** 0.5 / 8.0).to(dtype).to(DEV)
+            layout.write_keys(cache, torch.tensor([entry]).to(DEV), torch.tensor([pos % page]).to(DEV),
+                              key.expand(1, kv_heads, head_dim).contiguous())
+    meta = make_meta(table, [ctx], [q_len])
+    q = (randn(q_len, heads, head_dim, dtype=torch.float32, seed=9) + 8.0 * direction.to(DEV)).to(dtype)
+    scale = head_dim ** -0.5
+    out_h = torch.empty(q_len, heads * head_dim, dtype=dtype, device=DEV)
+    out_t = torch.empty_like(out_h)
+    hip.paged_attention(q, cache, meta, out_h, scale, window)
+    assert meta.work[(heads // kv_heads, window)].num_block_units > 0, "expected the shared-memory kernel"
+    twin.paged_attention(q, cache, meta, out_t, scale, window)
+    torch.testing.assert_close(out_h, out_t, **tol(dtype))
+    for t in (0, q_len // 2, q_len - 1):
+        ref = dense_attention(q[t], cache, table, 0, ctx - q_len + t, scale, window, page)
+        torch.testing.assert_close(out_h[t].float(), ref, **tol(dtype))
+        seen = [m for m in marks if m <= ctx - q_len + t]
+        weight = torch.softmax(torch.stack([(q[t, 0].float() * layout.read_keys(
+            cache, torch.tensor([int(table[0, m // page])]).to(DEV), torch.tensor([m % page]).to(DEV))[0, 0].float()).sum() * scale
+            for m in seen[-2:]]), 0)
+        assert weight[-1] > 0.9, "the last marked key must dominate, or the test shows nothing"
+
+
 @pytest.mark.parametrize("rows,n,k", [(1, 8192, 3072), (8, 3072, 6144), (16, 256, 128), (17, 48, 256), (33, 1024, 384),
                                       (64, 200064, 3072), (5, 50, 128), (3, 64, 96),
                                       (7, 64, 768), (16, 48, 1536), (2, 32, 3072), (20, 64, 768)])   # stages of six steps, K over 4, 8, 16 wavefronts
