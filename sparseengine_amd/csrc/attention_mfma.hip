@@ -510,22 +510,33 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                                        : plane + static_cast<int64_t>((wave - 2) * DSTEPS * 16 + n) * 8;
   const int off_scale = loads_keys ? 8 : D;
   const int64_t load_stride = loads_keys ? static_cast<int64_t>(32) * page_size : 128;
+  // a page's keys and values of all heads: fewer than 2^32 elements (the host checks it), so that a
+  // page's place is one multiplication of unsigned words
+  const uint32_t page_span = static_cast<uint32_t>(2 * plane);
+  const bf16_t* lane_src = cache_head + lane_base;
   auto issue = [&](int step) {
     const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS + wave * DSTEPS) * 1024u;
     const bool over = next_key > kmax;
-    const int page = page_ids[(over ? clamp_page : next_page) - window_base];
-    const bf16_t* src = cache_head + (static_cast<int64_t>(page) * 2) * plane + lane_base +
-                        static_cast<int64_t>(over ? clamp_off : next_off) * off_scale;
+    const uint32_t page = static_cast<uint32_t>(page_ids[(over ? clamp_page : next_page) - window_base]);
+    const bf16_t* src = lane_src + static_cast<uint64_t>(page) * page_span +
+                        static_cast<uint32_t>((over ? clamp_off : next_off) * off_scale);
 #pragma unroll
     for (int j = 0; j < DSTEPS; ++j) load16_to_lds(src + j * load_stride, dst + static_cast<uint32_t>(j) * 1024u);
     next_key += 32;
     next_off += 32;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)          // pages hold at least 8 keys
+    if (page_size >= 32) {               // the same for every lane: one page further at most
       if (next_off >= page_size) {
         next_off -= page_size;
         ++next_page;
       }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)        // pages hold at least 8 keys
+        if (next_off >= page_size) {
+          next_off -= page_size;
+          ++next_page;
+        }
+    }
   };
 
   const int nsteps = (key_end - k_first + 31) / 32;
@@ -863,6 +874,7 @@ extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const v
   if (q_stride % 8 || out_stride % 4 || tiles_per_block != 4 * TILED_ROW_TILES) return SE_ERR_SHAPE;
   const float scale_log2e = scale * 1.4426950408889634f;
   if (static_cast<int64_t>(num_units) * kv_heads > 0x7fffffff) return SE_ERR_SHAPE;
+  if (2 * static_cast<int64_t>(kv_heads) * page_size * head_dim > 0xffffffffLL) return SE_ERR_SHAPE;   // a page's span is a 32-bit word in the kernel
   dim3 grid(num_units * kv_heads);
 #define SE_ATT(DS)                                                                                 \
   case DS: {                                                                                       \
