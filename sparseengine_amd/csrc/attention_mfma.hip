@@ -372,7 +372,7 @@ __device__ __forceinline__ uint32_t pack_bf16x2_rne(float lo, float hi) {   // o
     pf[rt].w = pack_bf16x2_rne(v[6], v[7]);                                                        \
   }
 
-template <int DSTEPS, int RT, int NS>
+template <int DSTEPS, int RT, int NS, bool STEP_IN_PAGE>   // STEP_IN_PAGE: pages hold a multiple of 32 keys
 __global__ void __launch_bounds__(256, 2)
 paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                              const bf16_t* __restrict__ cache,
@@ -514,8 +514,40 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
   // page's place is one multiplication of unsigned words
   const uint32_t page_span = static_cast<uint32_t>(2 * plane);
   const bf16_t* lane_src = cache_head + lane_base;
+  // Pages of a multiple of 32 keys hold all keys of a step, so the step's page and the address of its
+  // first key are the same in all lanes: that arithmetic stays in scalar registers, beside the vector
+  // instructions that the loop is short of, and a lane adds only its own constant offset.  The steps at
+  // a unit's ends, where lanes are clamped to the first or the last key, take the lane-by-lane form.
+  constexpr bool page_per_step = STEP_IN_PAGE;
+  const uint32_t lane_bytes = static_cast<uint32_t>((lane_base + static_cast<int64_t>(lane_key) * off_scale) * 2);
+  int step_page = k_first / page_size, step_off = k_first % page_size;   // of the next step to be issued
   auto issue = [&](int step) {
     const uint32_t dst = stage_base + static_cast<uint32_t>((step % NS) * CHUNKS + wave * DSTEPS) * 1024u;
+    if constexpr (page_per_step) {
+      const int k = k_first + 32 * step;
+      if (k + 31 <= kmax && k >= low_key) {
+        const uint32_t page = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(page_ids[step_page - window_base]));
+        const bf16_t* base = cache_head + static_cast<uint64_t>(page) * page_span +
+                             static_cast<uint32_t>(step_off * off_scale);
+#pragma unroll
+        for (int j = 0; j < DSTEPS; ++j)
+          load16_to_lds_at(base + j * load_stride, lane_bytes, dst + static_cast<uint32_t>(j) * 1024u);
+      } else {
+        int key = k + lane_key;
+        if (key > kmax) key = clamp_key;
+        if (key < low_clamp) key = low_clamp;
+        const uint32_t page = static_cast<uint32_t>(page_ids[key / page_size - window_base]);
+        const bf16_t* src = lane_src + static_cast<uint64_t>(page) * page_span +
+                            static_cast<uint32_t>((key % page_size) * off_scale);
+#pragma unroll
+        for (int j = 0; j < DSTEPS; ++j) load16_to_lds(src + j * load_stride, dst + static_cast<uint32_t>(j) * 1024u);
+      }
+      step_off += 32;
+      if (step_off >= page_size) {
+        step_off -= page_size;
+        ++step_page;
+      }
+    } else {
     const bool over = next_key > kmax;
     const uint32_t page = static_cast<uint32_t>(page_ids[(over ? clamp_page : next_page) - window_base]);
     const bf16_t* src = lane_src + static_cast<uint64_t>(page) * page_span +
@@ -524,18 +556,12 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     for (int j = 0; j < DSTEPS; ++j) load16_to_lds(src + j * load_stride, dst + static_cast<uint32_t>(j) * 1024u);
     next_key += 32;
     next_off += 32;
-    if (page_size >= 32) {               // the same for every lane: one page further at most
+#pragma unroll
+    for (int i = 0; i < 4; ++i)          // pages hold at least 8 keys
       if (next_off >= page_size) {
         next_off -= page_size;
         ++next_page;
       }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)        // pages hold at least 8 keys
-        if (next_off >= page_size) {
-          next_off -= page_size;
-          ++next_page;
-        }
     }
   };
 
@@ -876,29 +902,33 @@ extern "C" int se_paged_attention_tiled(const void* q, int64_t q_stride, const v
   if (static_cast<int64_t>(num_units) * kv_heads > 0x7fffffff) return SE_ERR_SHAPE;
   if (2 * static_cast<int64_t>(kv_heads) * page_size * head_dim > 0xffffffffLL) return SE_ERR_SHAPE;   // a page's span is a 32-bit word in the kernel
   dim3 grid(num_units * kv_heads);
-#define SE_ATT(DS)                                                                                 \
-  case DS: {                                                                                       \
+#define SE_ATT_LAUNCH(DS, IN_PAGE)                                                                  \
+  {                                                                                                \
     constexpr size_t shared = TILED_STAGES * 4 * DS * 1024 + TILED_MAX_PAGES * sizeof(int32_t);    \
     static bool allowed = false; /* more than 64 KB of shared memory has to be asked for, once */  \
     if (!allowed) {                                                                                \
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(                                       \
-                                  &paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES>), \
+                                  &paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES, IN_PAGE>), \
                               hipFuncAttributeMaxDynamicSharedMemorySize,                          \
                               static_cast<int>(shared)) != hipSuccess)                             \
         return SE_ERR_LAUNCH;                                                                      \
       allowed = true;                                                                              \
     }                                                                                              \
-    paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES><<<grid, 256, shared, stream>>>( \
+    paged_attention_tiled_kernel<DS, TILED_ROW_TILES, TILED_STAGES, IN_PAGE><<<grid, 256, shared, stream>>>( \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(cache), block_table,  \
         bt_stride, units, static_cast<bf16_t*>(out), out_stride, part_o, part_ml, heads,          \
         kv_heads, page_size, scale_log2e, window);                                                 \
-    break;                                                                                         \
   }
+#define SE_ATT(DS)                                                                                 \
+  case DS:                                                                                         \
+    if (page_size % 32 == 0) SE_ATT_LAUNCH(DS, true) else SE_ATT_LAUNCH(DS, false)                 \
+    break;
   switch (head_dim / 32) {
     SE_ATT(1) SE_ATT(2) SE_ATT(3) SE_ATT(4)
     default: return SE_ERR_SHAPE;
   }
 #undef SE_ATT
+#undef SE_ATT_LAUNCH
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -258,5 +258,19 @@ __device__ __forceinline__ void load16_to_lds(const void* src, uint32_t lds_addr
                : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(src)   // the base is the same in all lanes
                : "memory", "m0");
 }
+// The same with the address in two parts: a base that is the same in all lanes (it stays in scalar
+// registers, and so does the arithmetic that made it) and a lane's own offset in bytes.
+__device__ __forceinline__ const void* same_in_all_lanes(const void* p) {   // tells the compiler so
+  const uint64_t bits = reinterpret_cast<uint64_t>(p);
+  const uint64_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(bits)));
+  const uint64_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(bits >> 32)));
+  return reinterpret_cast<const void*>((hi << 32) | lo);
+}
+__device__ __forceinline__ void load16_to_lds_at(const void* base, uint32_t offset, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(offset), "s"(same_in_all_lanes(base))
+               : "memory", "m0");
+}
 
 

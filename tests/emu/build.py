@@ -43,6 +43,8 @@ _ASM = [
     (r'asm volatile\("" : "\+v"\([^;]*\);', ";"),
     (r'asm volatile\("s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off"\s*:\s*:[^;]*;',
      "emu_load16_to_lds(src, lds_addr);"),
+    (r'asm volatile\("s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, %2"\s*:\s*:[^;]*;',
+     "emu_load16_to_lds(static_cast<const char*>(base) + offset, lds_addr);"),
 ]
 _DYNAMIC_SHARED = re.compile(
     r"extern\s+__shared__\s+(?:__align__\(\d+\)\s+)?((?:unsigned\s+)?\w+)\s+(\w+)\[\];")
