@@ -438,20 +438,26 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     const int pages = min(last_page - window_base + 1, TILED_MAX_PAGES);
     for (int i = tid; i < pages; i += 256) page_ids[i] = table[window_base + i];
   }
-  int token[RT], head[RT], pos[RT];
-  bool row_valid[RT];
+  // a lane's row of tile rt: whether the item has it, its token, head and position.  Worked out again
+  // where it is needed (the masked steps, the end): kept, it would cost eight registers all through
+  // a loop that has none to spare.
+  auto row_of = [&](int rt, bool& valid, int& token, int& head, int& position) {
+    const int rho = (tile0 + rt) * 16 + n;
+    valid = rho < rows_total;
+    const int rho_c = valid ? rho : rows_total - 1;   // padding rows repeat the last row
+    const int q_idx = rho_c / group;
+    head = kvh * group + rho_c % group;
+    token = q_start + q_idx;
+    position = pos0 + q_idx;
+  };
   uint4 qf[RT][DSTEPS];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int rho = (tile0 + rt) * 16 + n;
-    row_valid[rt] = rho < rows_total;
-    const int rho_c = row_valid[rt] ? rho : rows_total - 1;   // padding rows repeat the last row
-    const int q_idx = rho_c / group;
-    head[rt] = kvh * group + rho_c % group;
-    token[rt] = q_start + q_idx;
-    pos[rt] = pos0 + q_idx;
-    const bf16_t* q_row = q + static_cast<int64_t>(token[rt]) * q_stride +
-                          static_cast<int64_t>(head[rt]) * D + g * 8;
+    bool valid;
+    int token, head, position;
+    row_of(rt, valid, token, head, position);
+    const bf16_t* q_row = q + static_cast<int64_t>(token) * q_stride +
+                          static_cast<int64_t>(head) * D + g * 8;
 #pragma unroll
     for (int ds = 0; ds < DSTEPS; ++ds) qf[rt][ds] = *reinterpret_cast<const uint4*>(q_row + ds * 32);
   }
@@ -567,6 +573,12 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 
   const int nsteps = (key_end - k_first + 31) / 32;
   if (nsteps > 0) {
+    // The loop below works on two steps at a time: while the vector unit turns the scores of step t
+    // into probabilities, the matrix unit already makes the scores of step t + 1 (both from one wave's
+    // instruction stream, which is the only way the two units of a SIMD overlap reliably).  So keys
+    // are needed one step before values: the waves that bring keys run one step ahead of those that
+    // bring values, in the same ring of stages.
+    const int lead = loads_keys ? 1 : 0;
     // Only a unit's first step can begin before `low_key` (it begins less than 32 keys before it): a
     // lane whose key lies there takes `low_key`'s place for that one load and then goes on from its
     // own key.  (Done here and not inside `issue`, which is the loop's hot path.)
@@ -581,57 +593,76 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
       next_off = next_key % page_size;
     }
 #pragma unroll
-    for (int j = 1; j < NS - 1; ++j)
-      if (j < nsteps) issue(j);
-    // What every wave does at the start of a step, whatever it computes then: wait for the step's data,
-    // meet the others, issue the loads of the step NS - 1 ahead.
-    auto begin_step = [&](int step) {
-      // this step's data: all but the loads of the NS - 2 steps after it must have come back
-      if (step + NS - 2 < nsteps) {
+    for (int j = 1; j < NS; ++j)
+      if (j < NS - 1 + lead && j < nsteps) issue(j);
+    // What every wave does at the start of step t, whatever it computes then: wait for its part of the
+    // data that the step needs (the values of step t, the keys of step t + 1), meet the others, issue
+    // the loads of the step NS - 1 after that.
+    auto begin_step = [&](int t) {
+      const int mine = t + lead;
+      // all but the loads of the NS - 2 steps after `mine` must have come back
+      if (mine + NS - 2 < nsteps) {
         __builtin_amdgcn_s_waitcnt(0x0F70 | ((NS - 2) * DSTEPS));     // vmcnt((NS - 2) * DSTEPS)
       } else {
         __builtin_amdgcn_s_waitcnt(0x0F70);                           // vmcnt(0)
       }
-      __builtin_amdgcn_s_barrier();   // everyone's part of the step is in; everyone has left step - 1
+      __builtin_amdgcn_s_barrier();   // everyone's part is in; everyone has left step t - 1
       asm volatile("" ::: "memory");
-      if (step + NS - 1 < nsteps) {
-        const int k_next = k_first + 32 * (step + NS - 1);
-        if (min(k_next + 31, kmax) >= window_end) {
+      if (t + NS - 1 < nsteps) {      // values of step t + NS - 1, keys of step t + NS if there is one
+        const int k_near = k_first + 32 * (t + NS - 1);
+        const int k_far = k_first + 32 * min(t + NS, nsteps - 1);
+        if (min(k_far + 31, kmax) >= window_end) {
           // nobody reads page_ids between the barrier above and its own issue below
-          window_base = k_next / page_size;
+          window_base = k_near / page_size;
           window_end = (window_base + TILED_MAX_PAGES) * page_size;
           const int pages = min(last_page - window_base + 1, TILED_MAX_PAGES);
           for (int i = tid; i < pages; i += 256) page_ids[i] = table[window_base + i];
           __syncthreads();
         }
-        issue(step + NS - 1);   // into the buffer that step - 1 has used
+        if (mine + NS - 1 < nsteps) issue(mine + NS - 1);   // into the buffer whose last readers have met the barrier
       }
     };
-    // A step in full: the rows' ranges of keys, the reference maxima and the end of the cache all looked at.
-    auto whole_step = [&](int step) {
+    auto active = [&](int step) {      // has the wave a row that sees a key of this step?
       const int k0 = k_first + 32 * step;
-      if (k0 <= wave_hi && (window <= 0 || k0 + 31 > wave_lo - window)) {
+      return k0 <= wave_hi && (window <= 0 || k0 + 31 > wave_lo - window);
+    };
+    // lane (g, n): s[rt][b][i] becomes the score of key k0 + 8 g + 4 b + i for row n of tile rt
+    auto scores = [&](int step, floatx4 (&s)[RT][2]) {
+      const uint4* keys = &stage[step % NS][0][0];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ds = 0; ds < DSTEPS; ++ds)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const uint4 kf = keys[key_at[b] + 64 * ds];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
+                                                               __builtin_bit_cast(bf16x8, qf[rt][ds]),
+                                                               s[rt][b], 0, 0, 0);
+        }
+    };
+    // A step in full, from its scores: the rows' ranges of keys, the reference maxima and the end of the
+    // cache all looked at.
+    auto whole_step = [&](int step, floatx4 (&s)[RT][2]) {
+      const int k0 = k_first + 32 * step;
+      if (active(step)) {
         const uint4(*buf)[64] = stage[step % NS];
-        floatx4 s[RT][2];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ds = 0; ds < DSTEPS; ++ds)
-#pragma unroll
-          for (int b = 0; b < 2; ++b) {
-            const uint4 kf = (&buf[0][0])[key_at[b] + 64 * ds];
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-              s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
-                                                                 __builtin_bit_cast(bf16x8, qf[rt][ds]),
-                                                                 s[rt][b], 0, 0, 0);
-          }
-        // lane (g, n): s[rt][b][i] is the score of key k0 + 8 g + 4 b + i for row n of tile rt.
         // Most steps lie wholly inside every row's range of keys and need no mask.
         uint4 pf[RT];
         if (k0 + 31 > wave_lo || (window > 0 && k0 <= wave_hi - window)) {
+          int pos[RT];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            bool valid;
+            int token, head;
+            row_of(rt, valid, token, head, pos[rt]);
+          }
           TILED_SOFTMAX(1)
         } else {
+          const int* pos = nullptr;      // not looked at without masks
+          (void)pos;
           TILED_SOFTMAX(0)
         }
         // the block's last step may hold slots past the request's last key: whatever an earlier owner
@@ -669,77 +700,126 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     // without a path that rescales the accumulators.  (With that path inside the loop the compiler keeps
     // the accumulators in two sets of registers and copies all 64 of them between the sets in every
     // step; vector instructions, not matrix instructions, are what this kernel waits for.)  A step that
-    // would raise a maximum leaves the loop before it has touched anything and is done in full.
+    // would raise a maximum is done in full instead.
+    // a lane looks at its own eight keys only: any lane of a row that sees the maximum raised says so
+    auto raised = [&](const floatx4 (&s)[RT][2]) {
+      bool over = false;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const float m = max_bare(max3_bare(s[rt][0][0], s[rt][0][1], s[rt][0][2]),
+                                 max3_bare(max3_bare(s[rt][0][3], s[rt][1][0], s[rt][1][1]), s[rt][1][2], s[rt][1][3]));
+        over = over || !(m * scale_log2e <= run_max[rt] + SOFTMAX_SLACK);   // also with no maximum yet
+      }
+      return __builtin_amdgcn_ballot_w64(over) != 0;
+    };
+    auto plain_step = [&](int step, const floatx4 (&s)[RT][2]) {
+      const uint4(*buf)[64] = stage[step % NS];
+      uint4 pf[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        float v[8];
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          v[j] = __builtin_amdgcn_exp2f(fmaf(s[rt][j >> 2][j & 3], scale_log2e, -run_max[rt]));
+          sum += v[j];
+        }
+        run_sum[rt] += sum;
+        pf[rt].x = pack_bf16x2_rne(v[0], v[1]);
+        pf[rt].y = pack_bf16x2_rne(v[2], v[3]);
+        pf[rt].z = pack_bf16x2_rne(v[4], v[5]);
+        pf[rt].w = pack_bf16x2_rne(v[6], v[7]);
+      }
+#pragma unroll
+      for (int db = 0; db < DBLOCKS; ++db) {
+        const uint4 vf = buf[2 * DSTEPS + db][lane];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
+                                                             __builtin_bit_cast(bf16x8, pf[rt]),
+                                                             o[rt][db], 0, 0, 0);
+      }
+    };
     const int plain_limit = min(wave_lo, kmax) - 31;              // last first-key of a plain step
-    const int plain_end = plain_limit >= k_first ? min(nsteps, (plain_limit - k_first) / 32 + 1) : 0;
+    // (a plain step also makes the scores of the step after it, without asking whether there is one: the
+    // unit's last step is never among them)
+    const int plain_end = plain_limit >= k_first ? min(nsteps - 1, (plain_limit - k_first) / 32 + 1) : 0;
     const int plain_begin =
         window > 0 && wave_hi - window >= k_first ? (wave_hi - window - k_first) / 32 + 1 : 0;
-    int step = 0;
-    while (step < nsteps) {
+
+    // the keys of step 0 have to be in before the loop: of the steps issued so far (a wave that brings
+    // values has issued one fewer, and waits for nothing here) all but the first may still be under way
+    {
+      const int issued = min(NS, nsteps);
+      if (issued >= 4) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * DSTEPS));
+      } else if (issued == 3) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * DSTEPS));
+      } else if (issued == 2) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (1 * DSTEPS));
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    }
+    floatx4 sa[RT][2], sb[RT][2];     // the scores of the step at hand and of the one after it
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) sa[rt][0] = sa[rt][1] = sb[rt][0] = sb[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    if (active(0)) scores(0, sa);
+    // The row maxima are taken with bare instructions (inline assembly), which the compiler does not
+    // guard against reading a matrix instruction's result too early.  Inside the loop the scores that
+    // are looked at were issued a whole step before (sixteen more matrix instructions lie between);
+    // here the distance is made by hand.
+    asm volatile("s_nop 15\n\ts_nop 15" : "+v"(sa[0][0]), "+v"(sa[0][1]), "+v"(sa[RT - 1][0]), "+v"(sa[RT - 1][1]));
+    asm volatile("" ::: "memory");
+    int t = 0;
+    while (t < nsteps) {
       bool begun = false;     // the step's data is in and its barrier met
-      if (step >= plain_begin && step < plain_end) {
-        for (; step < plain_end; ++step) {
-          begin_step(step);
-          const uint4(*buf)[64] = stage[step % NS];
-          floatx4 s[RT][2];
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) s[rt][0] = s[rt][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int ds = 0; ds < DSTEPS; ++ds)
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-              const uint4 kf = (&buf[0][0])[key_at[b] + 64 * ds];
-#pragma unroll
-              for (int rt = 0; rt < RT; ++rt)
-                s[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
-                                                                   __builtin_bit_cast(bf16x8, qf[rt][ds]),
-                                                                   s[rt][b], 0, 0, 0);
-            }
-          // a lane looks at its own eight keys only: any lane of a row that sees the maximum raised says so
-          bool over = false;
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) {
-            const float m = max_bare(max3_bare(s[rt][0][0], s[rt][0][1], s[rt][0][2]),
-                                     max3_bare(max3_bare(s[rt][0][3], s[rt][1][0], s[rt][1][1]), s[rt][1][2], s[rt][1][3]));
-            over = over || !(m * scale_log2e <= run_max[rt] + SOFTMAX_SLACK);   // also with no maximum yet
-          }
-          if (__builtin_expect(__builtin_amdgcn_ballot_w64(over) != 0, 0)) {
+      if (t >= plain_begin && t < plain_end) {
+        bool in_b = false;    // the scores of step t are in `sb`
+        while (t < plain_end) {        // two steps a round, the two sets of scores taking turns
+          begin_step(t);
+          if (__builtin_expect(raised(sa), 0)) {
             begun = true;
             break;
           }
-          uint4 pf[RT];
+          scores(t + 1, sb);
+          plain_step(t, sa);
+          asm volatile("" ::: "memory");
+          ++t;
+          in_b = true;
+          if (t >= plain_end) break;
+          begin_step(t);
+          if (__builtin_expect(raised(sb), 0)) {
+            begun = true;
+            break;
+          }
+          scores(t + 1, sa);
+          plain_step(t, sb);
+          asm volatile("" ::: "memory");
+          ++t;
+          in_b = false;
+        }
+        if (in_b) {
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) {
-            float v[8];
-            float sum = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              v[j] = __builtin_amdgcn_exp2f(fmaf(s[rt][j >> 2][j & 3], scale_log2e, -run_max[rt]));
-              sum += v[j];
-            }
-            run_sum[rt] += sum;
-            pf[rt].x = pack_bf16x2_rne(v[0], v[1]);
-            pf[rt].y = pack_bf16x2_rne(v[2], v[3]);
-            pf[rt].z = pack_bf16x2_rne(v[4], v[5]);
-            pf[rt].w = pack_bf16x2_rne(v[6], v[7]);
+            sa[rt][0] = sb[rt][0];
+            sa[rt][1] = sb[rt][1];
           }
-#pragma unroll
-          for (int db = 0; db < DBLOCKS; ++db) {
-            const uint4 vf = buf[2 * DSTEPS + db][lane];
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-              o[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
-                                                                 __builtin_bit_cast(bf16x8, pf[rt]),
-                                                                 o[rt][db], 0, 0, 0);
-          }
-          asm volatile("" ::: "memory");
         }
         if (!begun) continue;     // the plain steps are done
       }
-      if (!begun) begin_step(step);
-      whole_step(step);
+      if (!begun) begin_step(t);
+      if (t + 1 < nsteps && active(t + 1)) scores(t + 1, sb);
+      whole_step(t, sa);
       asm volatile("" ::: "memory");
-      ++step;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        sa[rt][0] = sb[rt][0];
+        sa[rt][1] = sb[rt][1];
+      }
+      ++t;
     }
   }
 
@@ -761,10 +841,13 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
       }
       continue;
     }
-    if (!row_valid[rt] || !wave_active) continue;
+    bool valid;
+    int token, head, position;
+    row_of(rt, valid, token, head, position);
+    if (!valid || !wave_active) continue;
     const float inv = 1.f / total;
-    bf16_t* o_row = out + static_cast<int64_t>(token[rt]) * out_stride +
-                    static_cast<int64_t>(head[rt]) * D + 4 * g;
+    bf16_t* o_row = out + static_cast<int64_t>(token) * out_stride +
+                    static_cast<int64_t>(head) * D + 4 * g;
 #pragma unroll
     for (int db = 0; db < DBLOCKS; ++db) {
       uint2 packed;

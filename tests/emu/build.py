@@ -41,6 +41,8 @@ _ASM = [
     (r'asm\("v_max3_f32 %0, %1, %2, %3" : "=v"\(r\) : "v"\(a\), "v"\(b\), "v"\(c\)\);', "r = emu_max3_bare(a, b, c);"),
     # keeps values in registers before a loop: nothing to do on the host
     (r'asm volatile\("" : "\+v"\([^;]*\);', ";"),
+    # wait states after matrix instructions: nothing to do on the host
+    (r'asm volatile\("s_nop 15\\n\\ts_nop 15" : "\+v"\([^;]*\);', ";"),
     (r'asm volatile\("s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off"\s*:\s*:[^;]*;',
      "emu_load16_to_lds(src, lds_addr);"),
     (r'asm volatile\("s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, %2"\s*:\s*:[^;]*;',
