@@ -16,6 +16,14 @@ the live requests).  With random weights the tokens of a prompt agree on a few d
 the first layer, which makes a prompt cheaper than real weights would: ``prefill_uniform`` is the
 same step with every token sent to eight experts drawn evenly from all 256 (the routing is replaced
 after the router has run, so the router's own work is still in the time).
+
+    python bench.py --workload long_context | serving
+
+runs a whole workload through the engine's entry point (``LLM``: scheduler, cache manager, step
+function, sampler) instead and prints one JSON line of its own: ``long_context`` is 4 requests of
+131072 random token ids, prefilled in portions of 8192 tokens, then decode steps at batch 4 (8 layers);
+``serving`` is 32 requests with prompts of 512 to 16384 tokens in portions of 512 tokens beside the
+decoded tokens of the others, 512 output tokens each (24 layers, 217 GiB).
 """
 from __future__ import annotations
 
@@ -53,6 +61,10 @@ def main() -> int:
                         help="also time this many 2048-token prompts in one step (points.prefill_Nx2048); 1: skip")
     parser.add_argument("--prefill-routing", default="both", choices=["both", "natural", "uniform"],
                         help="profiling aid: which of the two prefill measurements to run (a reported line needs both)")
+    parser.add_argument("--workload", default="step", choices=["step", "long_context", "serving"],
+                        help="step: the decode / prefill steps described above; the others: a whole workload "
+                             "through the engine's entry point")
+    parser.add_argument("--output-len", type=int, default=None, help="decoded tokens per request of a workload")
     parser.add_argument("--fake-context", action="store_true",
                         help="profiling aid, never used for reported numbers: reserve the prompts' cache pages "
                              "without computing them, so that a kernel trace holds decode steps only")
@@ -60,6 +72,9 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
         return 2
+
+    if args.workload != "step":
+        return run_workload(args)
 
     import torch
 
@@ -242,6 +257,71 @@ def main() -> int:
         "points": points,
         "point_rooflines": point_rooflines,
     }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+def run_workload(args) -> int:
+    """A whole workload through ``LLM``: the model is MiniMax-M2's layer sizes with random weights made on
+    the device (``tiny_random``), the model folder holds nothing but its config.json."""
+    import os
+    import random
+    import tempfile
+
+    import torch
+
+    from sparseengine_amd import LLM, SamplingParams
+    from sparseengine_amd.engine.microbench import run_case
+
+    long_context = args.workload == "long_context"
+    layers = 8 if long_context else 24
+    folder = tempfile.mkdtemp(prefix="bench_model_")
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(dict(MODEL, num_hidden_layers=layers, max_position_embeddings=196608), fh)
+    sync = torch.cuda.synchronize
+    t0 = time.time()
+    if long_context:
+        length, batch, output_len = 131072, 4, args.output_len or 256
+        llm = LLM(folder, tiny_random=True, dtype=args.dtype, num_kvcache_slots=batch * (length + 4096),
+                  engine_prefill_chunk_size=8192, max_num_batched_tokens=8192, max_num_seqs_in_batch=batch)
+        print(f"[bench] engine built in {time.time() - t0:.1f} s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB "
+              f"allocated", file=sys.stderr, flush=True)
+        case = run_case(llm, length, batch, output_len, 0.0, 1.0, 0, sync=sync)
+        line = {"metric": "4 requests of 131072 tokens through the engine (MiniMax-M2 sizes, 8 layers, 1 GPU)",
+                "value": case["prefill_tok_s"], "unit": "prompt tokens/s", "n_gpus": 1, "dtype": args.dtype,
+                "data": "synthetic: random token ids, random weights",
+                "config": {"num_layers": layers, "requests": batch, "prompt_len": length, "portion": 8192,
+                           "output_len": output_len},
+                "prefill_s": case["prefill_s"], "prefill_steps": case["prefill_steps"],
+                "decode_tok_s": case["decode_tok_s"], "ms_per_decode_step": case["ms_per_decode_step"],
+                "decode_steps": case["decode_steps"], "total_s": case["total_s"]}
+    else:
+        requests, output_len = 32, args.output_len or 512
+        llm = LLM(folder, tiny_random=True, dtype=args.dtype, num_kvcache_slots=requests * 17408, max_model_len=17408,
+                  max_num_seqs_in_batch=requests, max_num_batched_tokens=512 + requests, engine_prefill_chunk_size=512,
+                  decode_reservation_tokens=1024)
+        for name, tensor in llm.runner.params.items():      # bias N(0, 0.01): routing spreads over all experts
+            if name.endswith("router_bias"):
+                tensor.mul_(0.1)
+        print(f"[bench] engine built in {time.time() - t0:.1f} s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB "
+              f"allocated", file=sys.stderr, flush=True)
+        rng = random.Random(0)
+        prompts = [[rng.randrange(MODEL["vocab_size"]) for _ in range(rng.randrange(512, 16384))] for _ in range(requests)]
+        sampling = SamplingParams(temperature=0.0, max_tokens=output_len, ignore_eos=True)
+        sync()
+        start = time.perf_counter()
+        outputs = llm.generate(prompts, sampling, use_tqdm=False)
+        sync()
+        seconds = time.perf_counter() - start
+        prompt_tokens = sum(len(p) for p in prompts)
+        output_tokens = sum(len(o["token_ids"]) for o in outputs)
+        line = {"metric": "32 requests, prompts of 512 to 16384 tokens in 512-token portions beside decodes "
+                          "(MiniMax-M2 sizes, 24 layers, 1 GPU)",
+                "value": round((prompt_tokens + output_tokens) / seconds, 1), "unit": "tokens/s (prompt + output)",
+                "n_gpus": 1, "dtype": args.dtype, "data": "synthetic: random token ids, random weights",
+                "config": {"num_layers": layers, "requests": requests, "portion": 512, "output_len": output_len},
+                "prompt_tokens": prompt_tokens, "output_tokens": output_tokens, "total_s": round(seconds, 3),
+                "preemptions": llm.scheduler.total_preemptions}
     print(json.dumps(line), flush=True)
     return 0
 
