@@ -675,6 +675,25 @@ def test_prompt_attention_with_maxima_that_keep_rising(hip, twin, heads, kv_head
         assert weight[-1] > 0.9, "the last marked key must dominate, or the test shows nothing"
 
 
+def test_prompt_attention_repeats_bit_for_bit(hip):
+    """The same step twice: the same bits (no atomics, no order that depends on timing; a wait that is too
+    weak for the loads into shared memory would show as a difference now and then)."""
+    emulator_skips(1e12)
+    heads, kv_heads, head_dim, page = 48, 8, 128, 64
+    lens, q_lens = [6000, 2500], [1500, 2500]
+    cache, table = make_paged(torch.bfloat16, kv_heads, head_dim, page, lens, seed=5)
+    meta = make_meta(table, lens, q_lens)
+    q = randn(sum(q_lens), heads, head_dim, dtype=torch.bfloat16, seed=6)
+    outs = []
+    for _ in range(6):
+        out = torch.full((sum(q_lens), heads * head_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+        hip.paged_attention(q, cache, meta, out, head_dim ** -0.5, 0)
+        outs.append(out)
+    assert not torch.isnan(outs[0].float()).any()
+    for out in outs[1:]:
+        assert torch.equal(out, outs[0])
+
+
 @pytest.mark.parametrize("rows,n,k", [(1, 8192, 3072), (8, 3072, 6144), (16, 256, 128), (17, 48, 256), (33, 1024, 384),
                                       (64, 200064, 3072), (5, 50, 128), (3, 64, 96),
                                       (7, 64, 768), (16, 48, 1536), (2, 32, 3072), (20, 64, 768)])   # stages of six steps, K over 4, 8, 16 wavefronts
