@@ -219,7 +219,8 @@ def main() -> int:
     if args.no_decode:
         return 0
     step_s, distinct, context = decode(args.batch, args.steps, args.warmup, "d")
-    print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.2f} ms/step", file=sys.stderr, flush=True)
+    print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.2f} ms/step, {sum(distinct) / len(distinct):.0f} experts touched "
+          f"per layer, {decode_bytes(args.batch, distinct, context) / step_s / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
     points, point_rooflines = {}, {}
     for b in [int(x) for x in args.points.split(",") if x]:
         s, d, c = decode(b, max(8, args.steps // 2), max(2, args.warmup // 2), f"b{b}_")
