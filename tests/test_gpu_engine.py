@@ -378,7 +378,8 @@ def run_toy_architecture(tmp_path, dtype, lengths):
     expected = {r: plain.logits(t).numpy() for r, t in requests.items()}
     records, peak = traces.mixed(requests, seed=1)
     runner = runner_for(folder, dtype, tokens=peak)
-    assert [(g.request.window, g.positions) for g in runner.cache.groups] == [(None, [0, 3, 5]), (24, [2])]
+    # three groups of cache pages: two kv heads (a layer that runs twice and the position after them), the window, one kv head
+    assert [(g.request.window, g.positions) for g in runner.cache.groups] == [(None, [0, 3, 6]), (24, [2]), (None, [5])]
     assert list(runner.cache.state_positions) == [1]
     from sparseengine_amd.engine.replay import replay_step
     out, chosen = {}, {rid: {"router": [[], []], "sign": [[]]} for rid in requests}

@@ -1,8 +1,9 @@
 """A toy architecture defined wholly in the tests, to show that parts, cache groups, state slots
 and the run order are general: layers differ in mixer (full attention, windowed attention, a
 recurrent mixer with state of its own), in feed-forward (dense, routed experts, a feed-forward
-with a routing rule of its own) and in position encoding (rotary, none, a rotation with its own
-table), the schedule runs a layer twice and lets one position read another position's cache.  Nothing in ``sparseengine_amd``
+with a routing rule of its own), in position encoding (rotary, none, a rotation with its own
+table), in norm (the engine's, one with another statistic) and in how a layer is arranged (mixer
+then feed-forward, or the two side by side), the schedule runs a layer twice and lets one position read another position's cache.  Nothing in ``sparseengine_amd``
 knows about it: it registers itself through the public registries.  It is no model of anyone's.
 """
 from __future__ import annotations
@@ -15,7 +16,8 @@ import torch
 from sparseengine_amd.config.registry import Architecture, WeightSource, register_architecture
 from sparseengine_amd.config.specs import (AttentionSpec, DenseMLPSpec, LayerSpec, ModelSpec, MoESpec, NoPositionSpec,
                                            NormSpec, RotarySpec, ScheduleEntry)
-from sparseengine_amd.parts import FEED_FORWARDS, MIXERS, POSITIONS, ParamDecl, Part, StateRequest, build_model
+from sparseengine_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, ParamDecl, Part, StateRequest,
+                                     build_model)
 from tests.plain import minimax_m2 as P
 
 
@@ -114,6 +116,88 @@ def linear_rotary_angles(positions, rotary_dim: int, slope: float):
 POSITIONS.register("toy_linear_rotary", lambda spec, head_dim: LinearRotary(spec, head_dim))
 
 
+# ------------------------------------------------------------------ a norm of another kind
+@dataclass(frozen=True)
+class MeanAbsNormSpec:
+    """``y = z / (mean |z| + eps) * w``: the statistic is the mean magnitude, not the mean square."""
+    kind: ClassVar[str] = "toy_mean_abs"
+    eps: float = 1e-5
+
+
+class MeanAbsNorm(Part):
+    """The interface of a norm: ``forward(fb, x, out, residual)`` adds ``x`` into the residual first (the
+    rounded sum becomes the residual, the unrounded sum is normed), ``forward_rows`` does it for chosen
+    rows and writes nothing but ``out``.  Statistic and sum in float, like the engine's own."""
+
+    def __init__(self, spec: MeanAbsNormSpec, hidden_size: int):
+        self.eps, self.hidden_size = float(spec.eps), int(hidden_size)
+
+    def param_decls(self):
+        return {"weight": ParamDecl((self.hidden_size,))}
+
+    def _norm(self, z):
+        return z / (z.abs().mean(-1, keepdim=True) + self.eps) * self.params["weight"].float()
+
+    def forward(self, fb, x, out=None, residual=None):
+        out = x if out is None else out
+        z = x.float()
+        if residual is not None:
+            z = z + residual.float()
+            residual.copy_(z)
+        out.copy_(self._norm(z))
+        return out
+
+    def forward_rows(self, fb, x, residual, rows, out):
+        z = x[rows.long()].float()
+        if residual is not None:
+            z = z + residual[rows.long()].float()
+        out.copy_(self._norm(z))
+        return out
+
+
+NORMS.register("toy_mean_abs", lambda spec, hidden_size: MeanAbsNorm(spec, hidden_size))
+
+
+def mean_abs_norm(z, weight, eps):
+    return z / (z.abs().mean(-1, keepdim=True) + eps) * weight
+
+
+# ------------------------------------------------------------------ another arrangement of a layer
+class SideBySideBlock(Part):
+    """Mixer and feed-forward read the same normed stream and their results are added (one norm per layer),
+    where the engine's own arrangement runs them one after the other with a norm each.  The pair
+    ``(x, residual)`` it hands on means what it means everywhere: the stream is their sum, and the next
+    norm adds them."""
+
+    def __init__(self, spec: LayerSpec, hidden_size: int, chunk_tokens: int = 16384):
+        self.norm = NORMS.build(spec.norm, hidden_size=hidden_size)
+        self.mixer = MIXERS.build(spec.mixer, hidden_size=hidden_size)
+        self.ffn = FEED_FORWARDS.build(spec.feed_forward, hidden_size=hidden_size, chunk_tokens=chunk_tokens)
+
+    def children(self):
+        return {"norm": self.norm, "mixer": self.mixer, "ffn": self.ffn}
+
+    def cache_request(self):
+        request = getattr(self.mixer, "cache_request", None)
+        return request() if request else None
+
+    def forward(self, fb, x, residual, cache_position: int, write_cache: bool):
+        if residual is None:
+            residual = fb.buffer("block.residual", x.shape)
+            residual.copy_(x)
+            u = self.norm.forward(fb, x)
+        else:
+            u = self.norm.forward(fb, x, residual=residual)
+        mixed = self.mixer.forward(fb, u, cache_position, write_cache)
+        both = fb.buffer("toy.side_by_side", mixed.shape)
+        both.copy_(mixed)
+        both += self.ffn.forward(fb, u)
+        return both, residual
+
+
+BLOCKS.register("toy_side_by_side", lambda spec, hidden_size, chunk_tokens=16384: SideBySideBlock(spec, hidden_size, chunk_tokens))
+
+
 def neighbour_rope(x, cos, sin, rotary_dim: int):
     """Plain rotation of dims ``(2 j, 2 j + 1)`` of each head by angle ``j``; ``x [T, heads, D]``."""
     out = x.clone()
@@ -153,7 +237,8 @@ def _layer_spec(cfg, layer) -> LayerSpec:
                       scoring=layer.get("scoring", "sigmoid"), selection_bias=layer.get("bias", True),
                       norm_topk_prob=layer.get("normalize", True), routed_scaling_factor=layer.get("scaling", 1.0),
                       activation=layer.get("activation", "silu"))
-    return LayerSpec(mixer=mixer, feed_forward=ffn, norm=NormSpec(eps=cfg["eps"]))
+    norm = MeanAbsNormSpec(eps=cfg["eps"]) if layer.get("norm") == "mean_abs" else NormSpec(eps=cfg["eps"])
+    return LayerSpec(mixer=mixer, feed_forward=ffn, norm=norm, block=layer.get("block", "prenorm"))
 
 
 def build_spec(cfg) -> ModelSpec:
@@ -197,13 +282,17 @@ TOY_CONFIG = dict(
         dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, ffn="moe", experts=4, top_k=3,
              intermediate=24, activation="gelu_tanh"),
         dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, ffn="dense", intermediate=48,
-             activation="gelu_tanh"),
+             activation="gelu_tanh", norm="mean_abs"),
         # (layer 0 turns neighbouring dims together, the others dims half a rotary width apart)
         dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=8, linear_rotary=0.05, ffn="sign",
              intermediate=20),
+        # mixer and feed-forward side by side behind one norm of the other kind
+        dict(mixer="attention", heads=2, kv_heads=1, head_dim=32, rotary_dim=16, ffn="dense", intermediate=32,
+             norm="mean_abs", block="toy_side_by_side"),
     ],
     # layer 0 runs twice (two caches); position 4 reads the cache of position 0 (same geometry)
-    schedule=[dict(layer=0), dict(layer=1), dict(layer=2), dict(layer=0), dict(layer=3, cache_from=0), dict(layer=4)])
+    schedule=[dict(layer=0), dict(layer=1), dict(layer=2), dict(layer=0), dict(layer=3, cache_from=0), dict(layer=5),
+              dict(layer=4)])
 
 
 # ------------------------------------------------------------------ its plain implementation
@@ -228,10 +317,12 @@ class PlainToy:
         for position, entry in enumerate(cfg["schedule"]):
             i, layer = entry["layer"], cfg["layers"][entry["layer"]]
             p = f"layers.{i}."
-            if residual is None:
-                residual, u = x, P.rms_norm(x, w[p + "norm_mixer.weight"], cfg["eps"])
-            else:
-                u, residual = P.add_rms_norm(x, residual, w[p + "norm_mixer.weight"], cfg["eps"])
+            side_by_side = layer.get("block") == "toy_side_by_side"
+            norm = (lambda z, wt: mean_abs_norm(z, wt, cfg["eps"])) if layer.get("norm") == "mean_abs" else \
+                (lambda z, wt: P.rms_norm(z, wt, cfg["eps"]))
+            first_norm = w[p + ("norm.weight" if side_by_side else "norm_mixer.weight")]
+            residual = x if residual is None else x + residual
+            u = norm(residual, first_norm)
             if layer["mixer"] == "decay":
                 s = torch.zeros(layer["state_size"])
                 a = torch.empty_like(u)
@@ -260,7 +351,11 @@ class PlainToy:
                 else:
                     kv_of[position] = (k, v)
                 a = P.causal_gqa_attention(q, k, v, D ** -0.5, window=layer.get("window")).reshape(T, -1) @ w[p + "mixer.o"].T
-            m, residual = P.add_rms_norm(a, residual, w[p + "norm_ffn.weight"], cfg["eps"])
+            if side_by_side:
+                m = u                          # the feed-forward reads what the mixer read
+            else:
+                residual = a + residual
+                m = norm(residual, w[p + "norm_ffn.weight"])
             I = layer["intermediate"]
             gelu = layer.get("activation") == "gelu_tanh"
             if layer["ffn"] == "dense":
@@ -292,5 +387,7 @@ class PlainToy:
                             x[t] += wt * (w[p + "ffn.w2"][e] @ (gate * (w[p + "ffn.w13"][e, I:] @ m[t])))
                 else:
                     x = P.swiglu_experts(m, w[p + "ffn.w13"][:, :I], w[p + "ffn.w13"][:, I:], w[p + "ffn.w2"], ids, wts)
+            if side_by_side:
+                x = a + x
         y, _ = P.add_rms_norm(x, residual, w["final_norm.weight"], cfg["eps"])
         return y @ w["head.weight"].T
