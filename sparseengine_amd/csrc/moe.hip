@@ -58,25 +58,24 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
       excluded |= 1u << i;
     }
   }
-  // k rounds of arg-max (largest value, lowest index among equals); the last value is the threshold
+  // k rounds of arg-max (largest value, lowest index among equals); the last value is the threshold.
+  // A round is two plain reductions over the wave, the maximum of the values and then the lowest index
+  // among the elements that hold it (a reduction over (value, index) pairs costs twice the instructions,
+  // and with few tokens this kernel is a lone wavefront's chain of dependent instructions).
   float threshold = 0.f;
   for (int round = 0; round < top_k; ++round) {
     float best = -INFINITY;
-    int best_idx = 0x7fffffff;
 #pragma unroll
-    for (int i = 0; i < PER_LANE; ++i) {
-      if ((taken | excluded) & (1u << i)) continue;
-      const int e = i * SE_WAVE + lane;
-      if (best_idx == 0x7fffffff || sel[i] > best) {
-        best = sel[i];
-        best_idx = e;
-      }
-    }
-    wave_reduce_pair(best, best_idx, [](float v, int i, float ov, int oi) {
-      return oi != 0x7fffffff && (i == 0x7fffffff || ov > v || (ov == v && oi < i));
-    });
-    if ((best_idx & (SE_WAVE - 1)) == lane) taken |= 1u << (best_idx / SE_WAVE);
-    threshold = best;
+    for (int i = 0; i < PER_LANE; ++i)
+      if (!((taken | excluded) & (1u << i)) && sel[i] > best) best = sel[i];
+    const float top = wave_max(best);
+    int lowest = 0x7fffffff;
+#pragma unroll
+    for (int i = PER_LANE - 1; i >= 0; --i)
+      if (!((taken | excluded) & (1u << i)) && sel[i] == top) lowest = i * SE_WAVE + lane;
+    const int winner = wave_reduce(lowest, [](int a, int b) { return a < b ? a : b; });
+    if ((winner & (SE_WAVE - 1)) == lane) taken |= 1u << (winner / SE_WAVE);
+    threshold = top;
   }
   // output order: strictly greater than the threshold by index, then the chosen ties by index
   int greater_before = 0, ties_before = 0;
