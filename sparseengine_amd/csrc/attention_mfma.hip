@@ -282,8 +282,10 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
 // rows, which binds a long prompt to the L2's bandwidth and to the latency of each step's loads.
 //
 // Such a load writes lane l's 16 bytes at (wave-uniform base) + 16 l, so shared memory holds
-// *operands*: one chunk of 1024 bytes per (key block b, 32 dims ds) and per 16 value dims db, in
-// which lane l's piece is exactly what lane l feeds the matrix core.  Reads are then conflict-free.
+// chunks of 1024 bytes in the order the loading lanes chose: per 16 value dims db one chunk in
+// which lane l's piece is exactly what lane l feeds the matrix core, and per (sixteen consecutive
+// keys, 32 dims ds) one chunk from which the lanes pick their operand's key when they read (the
+// places are chosen so that these reads are conflict-free too; see where `key_at` is set).
 // The compiler does not see these writes; the waits for them (vmcnt) are placed by hand, and the
 // barrier is a bare s_barrier: the usual fence would wait for every load in flight.
 // The request's page ids for the block's keys are copied to shared memory first (at most
