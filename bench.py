@@ -65,6 +65,9 @@ def main() -> int:
                         help="step: the decode / prefill steps described above; the others: a whole workload "
                              "through the engine's entry point")
     parser.add_argument("--output-len", type=int, default=None, help="decoded tokens per request of a workload")
+    parser.add_argument("--kv-page-size", type=int, default=None,
+                        help="tokens per cache page of a workload (default: the engine's; 16 makes block tables of 8192 "
+                             "pages for the long-context workload)")
     parser.add_argument("--fake-context", action="store_true",
                         help="profiling aid, never used for reported numbers: reserve the prompts' cache pages "
                              "without computing them, so that a kernel trace holds decode steps only")
@@ -140,9 +143,10 @@ def main() -> int:
         runner.step([StepEntry(r, [last[r]], []) for r in ids], taps=taps)       # untimed: which experts a step touches
         distinct = [int(torch.unique(i).numel()) for i, _ in taps["router"]]
         context = PROMPT_LEN + warmup + steps / 2
+        calls = time_calls(runner.kernels, lambda: runner.step([StepEntry(r, [last[r]], [0]) for r in ids]))
         for r in ids:
             runner.release(r)
-        return seconds / steps, distinct, context
+        return seconds / steps, distinct, context, calls
 
     itemsize = 2 if args.dtype == "bfloat16" else 4
     h, H, Hkv, D, E, K, I, V, L = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
@@ -156,6 +160,17 @@ def main() -> int:
         return (L * dense_layer + sum(distinct) * expert_bytes + V * h * itemsize
                 + batch * context * kv_token_layer * L)
 
+    def decode_calls(batch, distinct, context, calls):
+        """The calls a decode step's time goes to: milliseconds per step and the bytes each has to read per second."""
+        needs = {"moe_experts": sum(distinct) * expert_bytes, "paged_attention": batch * context * kv_token_layer * L,
+                 f"linear_{(H + 2 * Hkv) * D}": L * (H + 2 * Hkv) * D * h * itemsize, f"linear_{h}": L * h * H * D * itemsize,
+                 f"linear_{V}": V * h * itemsize}
+        label = {"moe_experts": "experts", "paged_attention": "attention", f"linear_{(H + 2 * Hkv) * D}": "qkv",
+                 f"linear_{h}": "o", f"linear_{V}": "head"}
+        out = {label[k]: {"ms": round(calls[k], 3), "GB/s": round(needs[k] / calls[k] / 1e6, 1)} for k in needs if calls.get(k)}
+        out["rest"] = {"ms": round(sum(v for k, v in calls.items() if k not in needs), 3)}
+        return out
+
     # ---- prefill of one 2048-token prompt
     natural = not args.no_prefill and args.prefill_routing != "uniform"
     times = [] if natural else [0.0, 1.0]
@@ -168,6 +183,7 @@ def main() -> int:
         runner.release(f"p{i}")
     prefill_s = min(times[1:])
     T = PROMPT_LEN
+    kernels = {}      # per call of the kernels object, from one step with events around each
     prefill_bytes = touched = None
     uniform_s = uniform_bytes = None
     if natural:     # untimed: the experts the prompt touches, layer by layer, are what it has to read
@@ -177,6 +193,13 @@ def main() -> int:
         touched = [int(torch.unique(i).numel()) for i, _ in taps["router"]]
         prefill_bytes = L * dense_layer + sum(touched) * expert_bytes + V * h * itemsize
         del taps
+        calls = time_calls(runner.kernels, lambda: runner.step([StepEntry("p_calls", prompt(), [PROMPT_LEN - 1])]))
+        runner.release("p_calls")
+        work = {"moe_experts": ("experts", 2 * T * K * 3 * I * h * L), "paged_attention": ("attention", 4 * H * D * T * (T + 1) / 2 * L),
+                f"linear_{(H + 2 * Hkv) * D}": ("qkv", 2 * T * h * (H + 2 * Hkv) * D * L), f"linear_{h}": ("o", 2 * T * H * D * h * L)}
+        kernels[f"prefill_{T}"] = {name: {"ms": round(calls[k], 3), "TFLOP/s": round(flops / calls[k] / 1e9, 1)}
+                                   for k, (name, flops) in work.items() if calls.get(k)}
+        kernels[f"prefill_{T}"]["rest"] = {"ms": round(sum(v for k, v in calls.items() if k not in work), 3)}
     if not args.no_prefill and args.prefill_routing != "natural":
         # the same step with even expert load: eight distinct experts per token, drawn uniformly
         dev_gen = torch.Generator(device="cuda").manual_seed(1)
@@ -218,12 +241,14 @@ def main() -> int:
     # ---- decode
     if args.no_decode:
         return 0
-    step_s, distinct, context = decode(args.batch, args.steps, args.warmup, "d")
+    step_s, distinct, context, calls = decode(args.batch, args.steps, args.warmup, "d")
+    kernels[f"decode_b{args.batch}"] = decode_calls(args.batch, distinct, context, calls)
     print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.2f} ms/step, {sum(distinct) / len(distinct):.0f} experts touched "
           f"per layer, {decode_bytes(args.batch, distinct, context) / step_s / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
     points, point_rooflines = {}, {}
     for b in [int(x) for x in args.points.split(",") if x]:
-        s, d, c = decode(b, max(8, args.steps // 2), max(2, args.warmup // 2), f"b{b}_")
+        s, d, c, calls = decode(b, max(8, args.steps // 2), max(2, args.warmup // 2), f"b{b}_")
+        kernels[f"decode_b{b}"] = decode_calls(b, d, c, calls)
         points[f"decode_b{b}"] = round(b / s, 1)
         point_rooflines[f"decode_b{b}"] = round(decode_bytes(b, d, c) / s / HBM_PEAK, 4)
         print(f"[bench] decode batch {b}: {s * 1e3:.2f} ms/step, {sum(d) / len(d):.0f} experts touched per layer, "
@@ -257,9 +282,50 @@ def main() -> int:
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
         "point_rooflines": point_rooflines,
+        # per call of the kernels object, from one step with events around each: what the step's time goes to
+        "kernels": kernels,
     }
     print(json.dumps(line), flush=True)
     return 0
+
+
+def time_calls(kernels, run) -> dict:
+    """Milliseconds per entry point of the kernels object over one call of ``run`` (an untimed step of its own):
+    a pair of events around every outermost call.  Dense products are told apart by their number of weight rows.
+    The events cost a microsecond or two each, so the figures serve for the calls that a step's time goes to."""
+    import torch
+
+    names = ("embedding", "rms_norm", "qk_norm_rope_store", "paged_attention", "route", "moe_experts", "linear")
+    spans, depth = [], [0]
+
+    def wrap(name, fn):
+        def call(*a, **k):
+            if depth[0]:
+                return fn(*a, **k)
+            label = f"linear_{a[1].shape[0]}" if name == "linear" else name
+            first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            depth[0] += 1
+            first.record()
+            try:
+                return fn(*a, **k)
+            finally:
+                last.record()
+                depth[0] -= 1
+                spans.append((label, first, last))
+        return call
+
+    for name in names:
+        setattr(kernels, name, wrap(name, getattr(kernels, name)))
+    try:
+        run()
+    finally:
+        for name in names:
+            delattr(kernels, name)       # the class's method shows again
+    torch.cuda.synchronize()
+    total = {}
+    for label, first, last in spans:
+        total[label] = total.get(label, 0.0) + first.elapsed_time(last)
+    return total
 
 
 def run_workload(args) -> int:
@@ -280,11 +346,12 @@ def run_workload(args) -> int:
     with open(os.path.join(folder, "config.json"), "w") as fh:
         json.dump(dict(MODEL, num_hidden_layers=layers, max_position_embeddings=196608), fh)
     sync = torch.cuda.synchronize
+    page = {"kv_page_size": args.kv_page_size} if args.kv_page_size else {}
     t0 = time.time()
     if long_context:
-        length, batch, output_len = 131072, 4, args.output_len or 256
+        length, batch, output_len = 131072, 4, args.output_len or 1024
         llm = LLM(folder, tiny_random=True, dtype=args.dtype, num_kvcache_slots=batch * (length + 4096),
-                  engine_prefill_chunk_size=8192, max_num_batched_tokens=8192, max_num_seqs_in_batch=batch)
+                  engine_prefill_chunk_size=8192, max_num_batched_tokens=8192, max_num_seqs_in_batch=batch, **page)
         print(f"[bench] engine built in {time.time() - t0:.1f} s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB "
               f"allocated", file=sys.stderr, flush=True)
         case = run_case(llm, length, batch, output_len, 0.0, 1.0, 0, sync=sync)
@@ -292,7 +359,7 @@ def run_workload(args) -> int:
                 "value": case["prefill_tok_s"], "unit": "prompt tokens/s", "n_gpus": 1, "dtype": args.dtype,
                 "data": "synthetic: random token ids, random weights",
                 "config": {"num_layers": layers, "requests": batch, "prompt_len": length, "portion": 8192,
-                           "output_len": output_len},
+                           "output_len": output_len, "kv_page_size": llm.config.kv_page_size},
                 "prefill_s": case["prefill_s"], "prefill_steps": case["prefill_steps"],
                 "decode_tok_s": case["decode_tok_s"], "ms_per_decode_step": case["ms_per_decode_step"],
                 "decode_steps": case["decode_steps"], "total_s": case["total_s"]}
@@ -300,7 +367,7 @@ def run_workload(args) -> int:
         requests, output_len = 32, args.output_len or 512
         llm = LLM(folder, tiny_random=True, dtype=args.dtype, num_kvcache_slots=requests * 17408, max_model_len=17408,
                   max_num_seqs_in_batch=requests, max_num_batched_tokens=512 + requests, engine_prefill_chunk_size=512,
-                  decode_reservation_tokens=1024)
+                  decode_reservation_tokens=1024, **page)
         for name, tensor in llm.runner.params.items():      # bias N(0, 0.01): routing spreads over all experts
             if name.endswith("router_bias"):
                 tensor.mul_(0.1)
@@ -309,19 +376,33 @@ def run_workload(args) -> int:
         rng = random.Random(0)
         prompts = [[rng.randrange(MODEL["vocab_size"]) for _ in range(rng.randrange(512, 16384))] for _ in range(requests)]
         sampling = SamplingParams(temperature=0.0, max_tokens=output_len, ignore_eos=True)
+        for prompt in prompts:
+            llm.add_request(prompt, sampling)
+        # a step's time by what it holds: portions of prompts beside decoded tokens, or decoded tokens alone
+        mixed_ms, decode_ms, output_tokens = [], [], 0
         sync()
         start = time.perf_counter()
-        outputs = llm.generate(prompts, sampling, use_tqdm=False)
-        sync()
+        while not llm.is_finished():
+            t1 = time.perf_counter()
+            finished, count = llm.step()
+            sync()
+            (mixed_ms if count > 0 else decode_ms).append((time.perf_counter() - t1) * 1e3)
+            output_tokens += sum(len(f[1]) for f in finished)
         seconds = time.perf_counter() - start
         prompt_tokens = sum(len(p) for p in prompts)
-        output_tokens = sum(len(o["token_ids"]) for o in outputs)
+
+        def spread(ms):
+            ms = sorted(ms)
+            at = lambda f: round(ms[min(len(ms) - 1, int(f * len(ms)))], 3)
+            return {"steps": len(ms), "mean": round(sum(ms) / len(ms), 3), "p50": at(0.5), "p90": at(0.9),
+                    "p99": at(0.99), "max": round(ms[-1], 3)} if ms else {"steps": 0}
         line = {"metric": "32 requests, prompts of 512 to 16384 tokens in 512-token portions beside decodes "
                           "(MiniMax-M2 sizes, 24 layers, 1 GPU)",
                 "value": round((prompt_tokens + output_tokens) / seconds, 1), "unit": "tokens/s (prompt + output)",
                 "n_gpus": 1, "dtype": args.dtype, "data": "synthetic: random token ids, random weights",
                 "config": {"num_layers": layers, "requests": requests, "portion": 512, "output_len": output_len},
                 "prompt_tokens": prompt_tokens, "output_tokens": output_tokens, "total_s": round(seconds, 3),
+                "step_ms_with_prompt_portions": spread(mixed_ms), "step_ms_decode_only": spread(decode_ms),
                 "preemptions": llm.scheduler.total_preemptions}
     print(json.dumps(line), flush=True)
     return 0
