@@ -15,7 +15,10 @@ step uses once - the experts it touched are counted from the step's own routing 
 the live requests).  With random weights the tokens of a prompt agree on a few dozen experts past
 the first layer, which makes a prompt cheaper than real weights would: ``prefill_uniform`` is the
 same step with every token sent to eight experts drawn evenly from all 256 (the routing is replaced
-after the router has run, so the router's own work is still in the time).
+after the router has run, so the router's own work is still in the time).  ``kernels`` holds, for the prefill
+and for every decode point, one further step with events around each call of the kernels object: the time of
+experts, attention, the dense products and the head, with the bytes (decode) or flops (prefill) each has to do
+per second.  ``--prompt-len C --no-prefill --fake-context`` gives decode steps at other context lengths.
 
     python bench.py --workload long_context | serving
 
@@ -46,6 +49,7 @@ CONTEXT_LEN = 8192
 
 
 def main() -> int:
+    global PROMPT_LEN, CONTEXT_LEN
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=64)
@@ -55,6 +59,9 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated")
     parser.add_argument("--kv-requests", type=int, default=64, help="requests of full context the cache is sized for")
+    parser.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
+                        help="tokens a request holds when its decoding starts (with --no-prefill --fake-context: decode "
+                             "steps at other context lengths; the cache is sized for --kv-requests of this plus 6144)")
     parser.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement (for profiling decode)")
     parser.add_argument("--no-decode", action="store_true", help="skip the decode measurements (for profiling prefill)")
     parser.add_argument("--prefill-prompts", type=int, default=8,
@@ -78,6 +85,7 @@ def main() -> int:
 
     if args.workload != "step":
         return run_workload(args)
+    PROMPT_LEN, CONTEXT_LEN = args.prompt_len, max(CONTEXT_LEN, args.prompt_len + 6144)
 
     import torch
 
