@@ -304,6 +304,41 @@ def test_norm_part(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("head_dim,rotary,theta,scaling", [(128, 64, 5e6, None), (48, 48, 1e4, None),
+                                                           (64, 32, 1e4, (("factor", 4.0), ("rope_type", "linear")))])
+def test_position_part(dtype, head_dim, rotary, theta, scaling):
+    """The rotary part alone: its table through the kernel that applies it (no norm, no cache write), at the
+    positions of the reference's vector (tests/test_flashinfer_rope.py:12-30).  The dims beyond the rotary ones
+    come back bit for bit, position 0 changes nothing, and positions divided by a linear scaling factor turn
+    by the angles of the plain implementation at the divided positions."""
+    from sparseengine_amd.config.specs import RotarySpec
+    from sparseengine_amd.parts import POSITIONS
+    part = POSITIONS.build(RotarySpec(rotary_dim=rotary, theta=theta, max_position=2048, scaling=scaling), head_dim=head_dim)
+    part.limit_positions(1100)
+    part.prepare(backends.ACTIVE.device)
+    assert part.table.shape == (1100, rotary) and part.table.dtype == torch.float32
+    heads, kv_heads = 3, 2
+    positions = torch.tensor([0, 1, 17, 127, 1023], dtype=torch.int32)
+    T = positions.numel()
+    qkv = torch.randn(T, (heads + 2 * kv_heads) * head_dim, generator=torch.Generator().manual_seed(5)).to(dtype)
+    given = qkv.float().clone()
+    on_device = qkv.to(backends.ACTIVE.device)
+    backends.ACTIVE.kernels().qk_norm_rope_store(on_device, positions.to(backends.ACTIVE.device), part.table, None, None, 1e-6,
+                                                 heads, kv_heads, head_dim, part.rotary_dim, None, None, 0, pairing=part.pairing)
+    got = on_device.float().cpu().clone()
+    factor = dict(scaling)["factor"] if scaling else 1.0
+    cos, sin = P.rope_angles(positions.float() / factor, rotary, theta)
+    width = (heads + kv_heads) * head_dim
+    ref = P.partial_rope(given[:, :width].reshape(T, heads + kv_heads, head_dim), cos, sin, rotary).reshape(T, width)
+    assert_part_close(dtype, got[:, :width], ref)
+    assert torch.equal(got[:, width:], given[:, width:]), "values are not rotated"
+    assert torch.equal(got[0], given[0]), "position 0 is the identity"
+    if rotary < head_dim:
+        kept = got[:, :width].reshape(T, -1, head_dim)[..., rotary:]
+        assert torch.equal(kept, given[:, :width].reshape(T, -1, head_dim)[..., rotary:]), "dims beyond the rotary ones pass through"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,head_dim,rotary,norm,window", [(6, 2, 32, 16, "flat", None), (5, 5, 48, 48, "none", 10),
                                                                         (8, 1, 64, 0, "flat", None)])
 def test_attention_part_in_two_portions(dtype, heads, kv_heads, head_dim, rotary, norm, window):
