@@ -94,6 +94,12 @@ def test_prompt_attention_with_maxima_that_keep_rising(guard, twin):
         G.test_prompt_attention_with_maxima_that_keep_rising(hip, twin, 8, 4, 32, 8, 500, 900, 260)
 
 
+def test_attention_at_the_windows_edge(guard):
+    with Emulated(guard=guard) as hip:
+        for shape in [(4, 2, 16, 16, 20, 150, 60), (6, 1, 128, 64, 100, 301, 1), (12, 4, 96, 24, 50, 400, 200)]:
+            G.test_attention_at_the_windows_edge(hip, *shape)
+
+
 def test_router(guard, twin):
     with Emulated(guard=guard) as hip:
         for dtype in (F32, BF16):

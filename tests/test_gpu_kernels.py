@@ -675,6 +675,45 @@ def test_prompt_attention_with_maxima_that_keep_rising(hip, twin, heads, kv_head
         assert weight[-1] > 0.9, "the last marked key must dominate, or the test shows nothing"
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page,window,ctx,q_len", [
+    (4, 2, 16, 16, 20, 150, 1), (4, 2, 16, 16, 20, 150, 60),           # the general kernel
+    (6, 1, 128, 64, 100, 301, 1), (12, 2, 64, 8, 33, 500, 3),          # one wavefront per tile
+    (16, 8, 64, 32, 70, 600, 300), (12, 4, 96, 24, 50, 400, 200)])     # blocks; pages that are no multiple of 32 keys
+def test_attention_at_the_windows_edge(hip, heads, kv_heads, head_dim, page, window, ctx, q_len):
+    """One key is made to dominate every query (all queries have a large component along one direction, the key
+    lies along it, its score about 30 above the rest).  For the row whose window begins with that key the answer
+    is the key's value; when the key lies one place further back, just outside that row's window, the row must
+    not see it at all.  With random keys alone one key more or less moves the answer by less than the bound."""
+    dtype = torch.bfloat16 if head_dim >= 32 else torch.float32
+    cache0, table = make_paged(dtype, kv_heads, head_dim, page, [ctx], seed=3, window=window, q_lens=[q_len])
+    direction = torch.ones(head_dim) / head_dim ** 0.5
+    meta = make_meta(table, [ctx], [q_len])
+    q = (randn(q_len, heads, head_dim, dtype=torch.float32, seed=4) + 8.0 * direction.to(DEV)).to(dtype)
+    scale = head_dim ** -0.5
+    t = q_len // 2
+    pos = ctx - q_len + t
+    for outside in (0, 1):
+        key_pos = pos - window + 1 - outside
+        entry = int(table[0, key_pos // page])
+        assert entry >= 0, "the marked key lies in a page the request still holds"
+        cache = cache0.clone()
+        where = (torch.tensor([entry]).to(DEV), torch.tensor([key_pos % page]).to(DEV))
+        layout.write_keys(cache, *where, (direction * 30.0 * head_dim ** 0.5 / 8.0).to(dtype).to(DEV).expand(1, kv_heads, head_dim).contiguous())
+        out = torch.empty(q_len, heads * head_dim, dtype=dtype, device=DEV)
+        hip.paged_attention(q, cache, meta, out, scale, window)
+        got = out[t].float().reshape(heads, head_dim)
+        value = layout.read_values(cache, *where)[0].float().repeat_interleave(heads // kv_heads, 0)
+        ref = dense_attention(q[t], cache, table, 0, pos, scale, window, page).reshape(heads, head_dim)
+        torch.testing.assert_close(got, ref, **tol(dtype))
+        if outside:
+            assert float((got - value).abs().max()) > 0.5, "a key outside the window has been seen"
+        else:
+            torch.testing.assert_close(got, value, rtol=2e-2, atol=2e-2)
+        if t + 1 < q_len:       # the next row's window has passed the key in both cases
+            after = dense_attention(q[t + 1], cache, table, 0, pos + 1, scale, window, page)
+            torch.testing.assert_close(out[t + 1].float(), after, **tol(dtype))
+
+
 def test_prompt_attention_repeats_bit_for_bit(hip):
     """The same step twice: the same bits (no atomics, no order that depends on timing; a wait that is too
     weak for the loads into shared memory would show as a difference now and then)."""
