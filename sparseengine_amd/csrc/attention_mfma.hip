@@ -732,6 +732,11 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
         pf[rt].z = pack_bf16x2_rne(v[4], v[5]);
         pf[rt].w = pack_bf16x2_rne(v[6], v[7]);
       }
+      // The wavefront asks for the instruction arbiter's favour while it feeds the matrix unit: the SIMD's
+      // other wavefront is then mostly in its exponentials, which would otherwise take turns with these
+      // instructions and leave the matrix unit waiting (a portion of 8192 tokens at context 65536: +6 %).
+      // (Reading the value operands ahead of the exponentials instead of just before their use changes nothing.)
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int db = 0; db < DBLOCKS; ++db) {
         const uint4 vf = buf[2 * DSTEPS + db][lane];
@@ -741,6 +746,7 @@ paged_attention_tiled_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
                                                              __builtin_bit_cast(bf16x8, pf[rt]),
                                                              o[rt][db], 0, 0, 0);
       }
+      __builtin_amdgcn_s_setprio(0);
     };
     const int plain_limit = min(wave_lo, kmax) - 31;              // last first-key of a plain step
     // (a plain step also makes the scores of the step after it, without asking whether there is one: the

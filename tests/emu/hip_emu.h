@@ -528,3 +528,4 @@ inline float emu_max3_bare(float a, float b, float c) { return fmaxf(fmaxf(a, b)
 #define __builtin_amdgcn_exp2f exp2f
 #define __builtin_amdgcn_s_waitcnt emu_s_waitcnt
 #define __builtin_amdgcn_s_barrier emu_s_barrier
+#define __builtin_amdgcn_s_setprio(level) ((void)(level))     // a hint to the instruction arbiter, nothing to emulate
