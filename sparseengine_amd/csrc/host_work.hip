@@ -20,7 +20,7 @@ constexpr int BLOCK_UNIT_FIELDS = 12;
 
 struct Rules {  // order of the `rules` argument
   int64_t target_waves, min_split_keys, max_splits, tiles_per_block, tiled_max_head_dim, target_blocks,
-      min_block_keys;
+      min_block_keys, prefix_per_portion;
 };
 
 // per item: in_blocks, rows (tiles or blocks), splits, chunk, first_key, base
@@ -49,9 +49,10 @@ int se_attention_work_plan(const int64_t* q_len, const int64_t* ctx_len, int ite
                            int kv_heads, int window, int head_dim, const int64_t* rules_in,
                            int64_t* plan, int64_t* counts) {
   if (items < 0 || group <= 0 || kv_heads <= 0) return -1;
-  Rules r{rules_in[0], rules_in[1], rules_in[2], rules_in[3], rules_in[4], rules_in[5], rules_in[6]};
+  Rules r{rules_in[0], rules_in[1], rules_in[2], rules_in[3], rules_in[4], rules_in[5], rules_in[6], rules_in[7]};
   const bool blocks_allowed = head_dim > 0 && head_dim % 32 == 0 && head_dim <= r.tiled_max_head_dim;
-  std::vector<int64_t> tiles(items), reach(items), nblocks(items), alone(items);
+  std::vector<int64_t> tiles(items), reach(items), nblocks(items), alone(items), cut_blocks(items);
+  int64_t whole = 0;      // blocks of items that are never cut into key ranges
   for (int i = 0; i < items; ++i) {
     if (q_len[i] < 1 || q_len[i] > ctx_len[i]) return -2;   // an item's new tokens are part of its context
     tiles[i] = (q_len[i] * group + 15) / 16;
@@ -60,13 +61,20 @@ int se_attention_work_plan(const int64_t* q_len, const int64_t* ctx_len, int ite
     plan[i * PLAN_FIELDS + 0] = in_blocks;
     nblocks[i] = in_blocks ? ceil_div(tiles[i], r.tiles_per_block) : 0;
     alone[i] = in_blocks ? 0 : tiles[i];
+    // the keys of a portion that is most of what it reads (a whole prompt) are not cut into ranges
+    const bool cut = in_blocks && reach[i] - q_len[i] >= r.prefix_per_portion * q_len[i];
+    cut_blocks[i] = cut ? nblocks[i] : 0;
+    whole += cut ? 0 : nblocks[i];
   }
-  const int64_t block_keys = keys_per_unit(nblocks, reach, kv_heads, r.target_blocks, r.min_block_keys);
+  whole *= kv_heads;
+  const int64_t block_keys = r.target_blocks > whole
+      ? keys_per_unit(cut_blocks, reach, kv_heads, r.target_blocks - whole, r.min_block_keys)
+      : int64_t(1) << 30;
   const int64_t wave_keys = keys_per_unit(alone, reach, kv_heads, r.target_waves, r.min_split_keys);
   int64_t units = 0, tasks = 0, blocks = 0, slots = 0;
   for (int i = 0; i < items; ++i) {
     const bool in_blocks = plan[i * PLAN_FIELDS + 0] != 0;
-    const int64_t keys = in_blocks ? block_keys : wave_keys;
+    const int64_t keys = in_blocks ? (cut_blocks[i] ? block_keys : int64_t(1) << 30) : wave_keys;
     const int64_t first_key = std::max<int64_t>(0, ctx_len[i] - reach[i]) / 32 * 32;
     const int64_t span = ctx_len[i] - first_key;
     int64_t splits = std::min(std::max<int64_t>(ceil_div(reach[i], keys), 1), r.max_splits);

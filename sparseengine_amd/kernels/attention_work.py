@@ -27,8 +27,17 @@ MIN_SPLIT_KEYS = 128   # keys of a range; 64 when ranges of 128 would leave most
 MAX_SPLITS = 256       # what the merge kernel's shared memory holds
 TILES_PER_BLOCK = 8    # row tiles of one block of the shared-memory kernel
 TILED_MAX_HEAD_DIM = 128
-TARGET_BLOCKS = 512    # blocks wanted in flight (two per CU); fewer: their keys are split
-MIN_BLOCK_KEYS = 512
+# Blocks, measured the same way (one request, causal flops): a portion of 512 tokens at context 16384 takes
+# 322 us in 3 ranges (576 blocks: one round of the chip's 512 places and an eighth of another) and 249 us in 8
+# ranges of 2048 keys (three rounds); at context 32768 594 against 443 us, a portion of 2048 at context 8192
+# 419 against 393 us.  Ranges under about a thousand keys lose it again to their own start-up and to the merge
+# (512 tokens at context 4096: 93 us in 3 or 4 ranges, 99 us in 8), and the rows of a whole prompt see more and
+# more keys, so equal ranges leave most of its blocks with half-empty ones (2048 tokens: 75 us whole, 105 us in
+# two ranges; 2048 at context 4096: 177 against 218 us): an item's keys are cut up only if the keys before its
+# portion are at least three times the portion.
+TARGET_BLOCKS = 1536   # blocks wanted in flight (three rounds of two per CU); fewer: their keys are split
+MIN_BLOCK_KEYS = 2048
+PREFIX_PER_PORTION = 3
 
 
 @dataclass
@@ -85,7 +94,7 @@ def build_attention_work(q_len, ctx_len, group: int, kv_heads: int, window: int 
     q = np.ascontiguousarray(q_len, dtype=np.int64)
     c = np.ascontiguousarray(ctx_len, dtype=np.int64)
     rules = np.asarray([target_waves, MIN_SPLIT_KEYS, MAX_SPLITS, TILES_PER_BLOCK, TILED_MAX_HEAD_DIM,
-                        TARGET_BLOCKS, MIN_BLOCK_KEYS], dtype=np.int64)
+                        TARGET_BLOCKS, MIN_BLOCK_KEYS, PREFIX_PER_PORTION], dtype=np.int64)
     plan = np.empty((q.size, 6), dtype=np.int64)
     counts = np.empty(4, dtype=np.int64)
     i64p, i32p = ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32)
@@ -135,8 +144,12 @@ def build_attention_work_numpy(q_len, ctx_len, group: int, kv_heads: int, window
 
     nblocks = np.where(in_blocks, -(-tiles // TILES_PER_BLOCK), 0)
     alone = np.where(in_blocks, 0, tiles)
-    keys = np.where(in_blocks, keys_per_unit(nblocks, TARGET_BLOCKS, MIN_BLOCK_KEYS),
-                    keys_per_unit(alone, target_waves, MIN_SPLIT_KEYS))
+    # blocks of an item whose portion is most of what it reads (a whole prompt) are never cut: they take
+    # their places among the blocks wanted as they are
+    cut = in_blocks & (reach - q_len >= PREFIX_PER_PORTION * q_len)
+    whole = int(np.where(cut, 0, nblocks).sum()) * kv_heads
+    block_keys = keys_per_unit(np.where(cut, nblocks, 0), TARGET_BLOCKS - whole, MIN_BLOCK_KEYS) if TARGET_BLOCKS > whole else 1 << 30
+    keys = np.where(in_blocks, np.where(cut, block_keys, 1 << 30), keys_per_unit(alone, target_waves, MIN_SPLIT_KEYS))
     # equal ranges (multiples of 32 keys) over [first_key, ctx) of every item
     first_key = np.maximum(0, ctx_len - reach) // 32 * 32
     span = ctx_len - first_key

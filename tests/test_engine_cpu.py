@@ -278,6 +278,11 @@ def test_block_work_lists_for_many_rows_cover_every_tile_once_longest_first():
     # a long single token beside a prompt gets many more ranges than its short neighbours
     work = build_attention_work([1, 2048, 1], [70000, 2048, 2048], 6, 8, 0, head_dim=128)
     assert (work.units[:, 0] == 0).sum() >= 20 * (work.units[:, 0] == 2).sum()
+    # a portion on a long prefix is cut into ranges of at least 2048 keys, about three rounds of blocks; the keys of a
+    # portion that is most of what it reads (a whole prompt, a prompt's second half) are not cut at all
+    ranges = lambda q, c: int(build_attention_work([q], [c], 6, 8, 0, head_dim=128).block_units[0, 8])
+    assert ranges(512, 16384) == 8 and ranges(512, 32768) == 8 and ranges(2048, 8192) == 2
+    assert ranges(2048, 2048) == 1 and ranges(1024, 1024) == 1 and ranges(2048, 4096) == 1 and ranges(3000, 3000) == 1
     # a head size the block kernel does not take, and a step of single tokens, keep the per-wavefront list
     assert len(build_attention_work([2048], [2048], 6, 8, 0, head_dim=160).block_units) == 0
     assert len(build_attention_work([1] * 8, [300] * 8, 6, 8, 0, head_dim=128).block_units) == 0
