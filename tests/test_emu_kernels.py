@@ -82,7 +82,9 @@ def test_attention_split_keys_and_one_far_key(guard, twin):
     (8, 8, 32, 8, 0, [420], [420]),
     (16, 8, 64, 24, 0, [300, 200], [300, 100]),         # pages that are no multiple of a step of 32 keys
     (24, 8, 96, 40, 33, [250, 100, 90], [240, 100, 1]),
-    (12, 2, 64, 16, 90, [600, 500], [30, 77])])         # few blocks and a window: their keys are split
+    (12, 2, 64, 16, 90, [600, 500], [30, 77]),          # few blocks and a window
+    (4, 2, 32, 16, 0, [2300], [40]),                    # one row block per kv head: three ranges of keys and a merge
+    (12, 2, 64, 16, 1500, [2600, 2500], [30, 77])])     # the same within a window
 def test_attention_prompt_portions(guard, twin, shape):
     with Emulated(guard=guard) as hip:
         G.test_paged_attention_prompt_portions(hip, twin, *shape)

@@ -611,7 +611,9 @@ def test_paged_attention_split_keys(hip, twin, batch, ctx, q_len):
     (48, 8, 128, 64, 0, [9000, 2100, 77], [1, 2100, 5]),          # a decoded token with a long context beside a prompt
     (48, 8, 128, 64, 0, [20000], [100]),                          # few blocks, long context: their keys are split
     (12, 2, 64, 16, 900, [6000, 5000], [300, 77]),                # the same with a window
-    (8, 8, 32, 8, 0, [17000], [4100])])                          # more pages than the kernel keeps ids of at once
+    (8, 8, 32, 8, 0, [17000], [4100]),                           # more pages than the kernel keeps ids of at once
+    (4, 2, 32, 16, 0, [2300], [40]),                             # one row block per kv head: three ranges of keys
+    (12, 2, 64, 16, 1500, [2600, 2500], [30, 77])])              # the same within a window
 def test_paged_attention_prompt_portions(hip, twin, heads, kv_heads, head_dim, page, window, lens, q_lens):
     """Steps with many rows: blocks share each step's keys and values through shared memory."""
     emulator_skips(sum(q * (min(n, window + q) if window else n) for q, n in zip(q_lens, lens)) * heads * head_dim, 2.5e9)
