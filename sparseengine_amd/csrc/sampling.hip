@@ -74,101 +74,230 @@ __device__ int block_sum_i(int v, int* scratch) {
   return total;
 }
 
-__global__ void __launch_bounds__(SAMPLE_THREADS)
-sample_kernel(const float* __restrict__ logits, int64_t stride, int vocab,
-              const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
-              const float* __restrict__ top_p, const uint64_t* __restrict__ seeds,
-              int32_t* __restrict__ out) {
-  __shared__ ArgBest arg_scratch[SAMPLE_THREADS / SE_WAVE];
-  __shared__ float f_scratch[SAMPLE_THREADS / SE_WAVE];
-  __shared__ int i_scratch[SAMPLE_THREADS / SE_WAVE];
-  const int row = blockIdx.x;
-  const float* l = logits + static_cast<int64_t>(row) * stride;
-  const float temp = temperature ? temperature[row] : 0.f;
+// ---------------------------------------------------------------------------------------- //
+// Rows with top-k or top-p.  Both filters keep a prefix of the row's tokens in descending order,
+// that is all tokens whose ordered key is at least some threshold.  A threshold is found eight
+// bits at a time: a pass over the row counts (top-k) or weighs (top-p) the tokens in the 256 bins
+// of the next eight key bits, among those that agree with the bits found so far; many blocks per
+// row share a pass and add their bins into the row's histogram, and every block of the next pass
+// reads the histograms so far and works the bits out again (a few hundred additions) rather than
+// wait for another launch to do it.  Sums are integers (a token's weight is exp(l - max) in units of
+// 2^-40), so the order in which blocks and wavefronts add them does not matter: the same row gives
+// the same token on every run and in every batch.
+//   hist [rows][2 * FILTER_PASSES][FILTER_BINS] uint64: passes 0-3 counts, 4-7 weights; zero at the start
+// ---------------------------------------------------------------------------------------- //
+#define FILTER_BINS 256
+#define FILTER_PASSES 4
+typedef unsigned long long u64;
 
-  if (!(temp > 1e-10f)) {
-    ArgBest best = {-INFINITY, -1};
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-      ArgBest c = {l[i], i};
-      if (c.value != c.value) c.value = INFINITY;  // NaN wins, as in a library arg-max
-      best = better(best, c);
-    }
-    best = block_argbest(best, arg_scratch);
-    if (threadIdx.x == 0) out[row] = best.index;
-    return;
+__device__ __forceinline__ u64 lane_value64(u64 v, int source) {
+  const uint32_t lo = __shfl(static_cast<uint32_t>(v), source);
+  const uint32_t hi = __shfl(static_cast<uint32_t>(v >> 32), source);
+  return (static_cast<u64>(hi) << 32) | lo;
+}
+
+// One wavefront, lane l holding bins 4 l ... 4 l + 3 of a pass: the largest bin d for which
+// `above` + (sum of the bins d ... 255) reaches `target` (strictly exceeds it if `strict`), and what
+// lies above that bin (`above` + sum of the bins d + 1 ... 255).  Bin 0 if none does.
+__device__ __forceinline__ int pick_bin(const u64 (&bin)[4], u64 above, u64 target, bool strict, u64& above_out) {
+  const int lane = threadIdx.x & (SE_WAVE - 1);
+  const u64 mine = bin[0] + bin[1] + bin[2] + bin[3];
+  u64 from_here = mine;      // becomes the sum over this lane and all lanes after it
+#pragma unroll
+  for (int off = 1; off < SE_WAVE; off <<= 1) {
+    const u64 other = lane_value64(from_here, (lane + off) & (SE_WAVE - 1));
+    if (lane + off < SE_WAVE) from_here += other;
   }
+  u64 tail = above + from_here - mine;      // everything above this lane's last bin
+  int found = -1;
+  u64 above_found = 0;
+#pragma unroll
+  for (int j = 3; j >= 0; --j) {
+    const u64 with = tail + bin[j];
+    if (found < 0 && (strict ? with > target : with >= target)) {
+      found = j;
+      above_found = tail;
+    }
+    tail = with;
+  }
+  const uint64_t who = __ballot(found >= 0);
+  if (who == 0) {       // cannot happen with consistent histograms; bin 0 keeps every token
+    above_out = above + lane_value64(from_here, 0);
+    return 0;
+  }
+  const int top = 63 - __builtin_clzll(who);
+  above_out = lane_value64(above_found, top);
+  return 4 * top + __shfl(found, top);
+}
 
+// The bits found by the first `passes` passes of one kind (run by one whole wavefront).
+__device__ __forceinline__ uint32_t bits_found(const u64* __restrict__ hist_kind, int passes, u64 target, bool strict) {
+  const int lane = threadIdx.x & (SE_WAVE - 1);
+  uint32_t prefix = 0;
+  u64 above = 0;
+  for (int pass = 0; pass < passes; ++pass) {
+    const u64* h = hist_kind + pass * FILTER_BINS + 4 * lane;
+    const u64 bin[4] = {h[0], h[1], h[2], h[3]};
+    prefix = (prefix << 8) | static_cast<uint32_t>(pick_bin(bin, above, target, strict, above));
+  }
+  return prefix;
+}
+
+// the largest of the row's chunk maxima (one wavefront)
+__device__ __forceinline__ float row_max(const float* __restrict__ part_max, int chunks) {
+  const int lane = threadIdx.x & (SE_WAVE - 1);
+  float m = -INFINITY;
+  for (int c = lane; c < chunks; c += SE_WAVE) m = fmaxf(m, part_max[c]);
+  return wave_max(m);
+}
+
+__device__ __forceinline__ u64 weight_of(float v, float vmax) {
+  const float w = expf(v - vmax) * 1099511627776.f;      // 2^40: the largest token weighs exactly that
+  return w == w ? static_cast<u64>(w) : 0;
+}
+
+// the weight that the tokens kept by top-p may have above them: top_p times the weight of all tokens that top-k kept
+__device__ __forceinline__ u64 nucleus_budget(const u64* __restrict__ hist_weights, float p) {
+  const int lane = threadIdx.x & (SE_WAVE - 1);
+  u64 total = hist_weights[4 * lane] + hist_weights[4 * lane + 1] + hist_weights[4 * lane + 2] + hist_weights[4 * lane + 3];
+#pragma unroll
+  for (int off = 1; off < SE_WAVE; off <<= 1) total += lane_value64(total, lane ^ off);
+  return static_cast<u64>(static_cast<double>(p) * static_cast<double>(total));
+}
+
+#define SAMPLE_CHUNK 4096
+// the chunk maxima of logit / temperature, for the weights
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_chunk_max_kernel(const float* __restrict__ logits, int64_t stride, int vocab,
+                        const float* __restrict__ temperature, const float* __restrict__ top_p,
+                        float* __restrict__ part_max, int chunks) {
+  __shared__ float scratch[SAMPLE_THREADS / SE_WAVE];
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const float temp = temperature[row];
+  if (!(temp > 1e-10f) || !(top_p[row] < 1.f)) return;     // the whole block
   const float inv_temp = 1.f / temp;
+  const float* l = logits + static_cast<int64_t>(row) * stride;
+  const int begin = chunk * SAMPLE_CHUNK;
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < SAMPLE_CHUNK / SAMPLE_THREADS; ++j) {
+    const int i = begin + threadIdx.x + j * SAMPLE_THREADS;
+    if (i < vocab) m = fmaxf(m, l[i] * inv_temp);
+  }
+  m = wave_max(m);
+  const int lane = threadIdx.x & (SE_WAVE - 1), wave = threadIdx.x / SE_WAVE;
+  if (lane == 0) scratch[wave] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < SAMPLE_THREADS / SE_WAVE; ++w) m = fmaxf(m, scratch[w]);
+    part_max[row * chunks + chunk] = m;
+  }
+}
+
+template <bool WEIGHTS>    // false: a top-k pass (counts), true: a top-p pass (weights)
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_filter_pass_kernel(const float* __restrict__ logits, int64_t stride, int vocab,
+                          const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
+                          const float* __restrict__ top_p, const float* __restrict__ part_max,
+                          u64* __restrict__ hist, int pass, int chunks) {
+  __shared__ u64 bins[SAMPLE_THREADS / SE_WAVE][FILTER_BINS];     // one set per wavefront: fewer collisions
+  __shared__ uint32_t found[2];
+  __shared__ float shared_max;
+  const int row = blockIdx.x, chunk = blockIdx.y;
+  const float temp = temperature[row];
   const int k = top_k ? top_k[row] : 0;
   const float p = top_p ? top_p[row] : 1.f;
-  // smallest ordered key that is kept
-  uint32_t keep_from = 0;
-  if (k > 0 && k < vocab) {
-    uint32_t ans = 0;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = ans | (1u << bit);
-      int cnt = 0;
-      for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS)
-        cnt += ordered_key(l[i] * inv_temp) >= cand;
-      if (block_sum_i(cnt, i_scratch) >= k) ans = cand;
+  const bool has_k = k > 0 && k < vocab, has_p = p < 1.f;
+  if (!(temp > 1e-10f) || (WEIGHTS ? !has_p : !has_k)) return;     // the whole block
+  const int lane = threadIdx.x & (SE_WAVE - 1), wave = threadIdx.x / SE_WAVE;
+  for (int i = threadIdx.x; i < (SAMPLE_THREADS / SE_WAVE) * FILTER_BINS; i += SAMPLE_THREADS) (&bins[0][0])[i] = 0;
+  u64* hist_row = hist + static_cast<int64_t>(row) * 2 * FILTER_PASSES * FILTER_BINS;
+  if (wave == 0) {
+    uint32_t k_bits = 0, p_bits = 0;
+    if (has_k) k_bits = bits_found(hist_row, WEIGHTS ? FILTER_PASSES : pass, static_cast<u64>(k), false);
+    if (WEIGHTS) {
+      const u64* weights = hist_row + FILTER_PASSES * FILTER_BINS;
+      if (pass > 0) p_bits = bits_found(weights, pass, nucleus_budget(weights, p), true);
+      const float m = row_max(part_max + row * chunks, chunks);
+      if (lane == 0) shared_max = m;
     }
-    keep_from = ans;
-  }
-  float vmax = -INFINITY;
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) vmax = fmaxf(vmax, l[i] * inv_temp);
-  {
-    ArgBest m = {vmax, 0};
-    vmax = block_argbest(m, arg_scratch).value;
-  }
-  if (p < 1.f) {
-    float z = 0.f;
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-      const float v = l[i] * inv_temp;
-      if (ordered_key(v) >= keep_from) z += expf(v - vmax);
+    if (lane == 0) {
+      found[0] = k_bits;
+      found[1] = p_bits;
     }
-    z = block_sum_f(z, f_scratch);
-    const float budget = p * z;
-    uint32_t ans = 0;  // largest key c with mass{kept key >= c} > budget, built bit by bit
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = ans | (1u << bit);
-      float mass = 0.f;
-      for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-        const float v = l[i] * inv_temp;
-        const uint32_t key = ordered_key(v);
-        if (key >= cand && key >= keep_from) mass += expf(v - vmax);
-      }
-      if (block_sum_f(mass, f_scratch) > budget) ans = cand;
-    }
-    if (ans > keep_from) keep_from = ans;
   }
-  const uint64_t seed = seeds ? seeds[row] : 0ull;
-  ArgBest best = {-INFINITY, -1};
-  for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+  __syncthreads();
+  const uint32_t k_bits = found[0], p_bits = found[1];
+  const float vmax = WEIGHTS ? shared_max : 0.f;
+  const float inv_temp = 1.f / temp;
+  const float* l = logits + static_cast<int64_t>(row) * stride;
+  const int begin = chunk * SAMPLE_CHUNK;
+  const int high = 32 - 8 * pass;       // bits above the pass's eight (32 in the first pass: no shift by that)
+#pragma unroll
+  for (int j = 0; j < SAMPLE_CHUNK / SAMPLE_THREADS; ++j) {
+    const int i = begin + threadIdx.x + j * SAMPLE_THREADS;
+    if (i >= vocab) continue;
     const float v = l[i] * inv_temp;
-    if (ordered_key(v) < keep_from) continue;
-    const float u = uniform_open(seed, static_cast<uint32_t>(i));
-    ArgBest c = {v - logf(-logf(u)), i};
-    best = better(best, c);
+    const uint32_t key = ordered_key(v);
+    const uint32_t bin = (key >> (high - 8)) & (FILTER_BINS - 1);
+    if (WEIGHTS) {
+      if (has_k && key < k_bits) continue;      // top-k has dropped it
+      if (pass > 0 && (key >> high) != p_bits) continue;
+      atomicAdd(&bins[wave][bin], weight_of(v, vmax));
+    } else {
+      if (pass > 0 && (key >> high) != k_bits) continue;
+      atomicAdd(&bins[wave][bin], static_cast<u64>(1));
+    }
   }
-  best = block_argbest(best, arg_scratch);
-  if (threadIdx.x == 0) out[row] = best.index;
+  __syncthreads();
+  if (threadIdx.x < FILTER_BINS) {
+    u64 total = 0;
+    for (int w = 0; w < SAMPLE_THREADS / SE_WAVE; ++w) total += bins[w][threadIdx.x];
+    if (total) atomicAdd(hist_row + ((WEIGHTS ? FILTER_PASSES : 0) + pass) * FILTER_BINS + threadIdx.x, total);
+  }
+}
+
+__global__ void zero_words_kernel(u64* __restrict__ words, int64_t count) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < count) words[i] = 0;
 }
 
 // Rows without top-k / top-p are one arg-max each (of the logits, or of scaled logits plus
 // noise): many blocks per row find partial maxima over stretches of the vocabulary, one
 // wavefront per row picks among them.
-#define SAMPLE_CHUNK 4096
+// With `hist` (filled by the passes above) a row's tokens below its thresholds are left out.
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_partial_kernel(const float* __restrict__ logits, int64_t stride, int vocab,
                       const float* __restrict__ temperature, const uint64_t* __restrict__ seeds,
-                      float* __restrict__ part_value, int32_t* __restrict__ part_index, int chunks) {
+                      float* __restrict__ part_value, int32_t* __restrict__ part_index, int chunks,
+                      const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
+                      const u64* __restrict__ hist) {
   __shared__ ArgBest arg_scratch[SAMPLE_THREADS / SE_WAVE];
+  __shared__ uint32_t shared_keep_from;
   const int row = blockIdx.x, chunk = blockIdx.y;
   const float* l = logits + static_cast<int64_t>(row) * stride;
   const float temp = temperature ? temperature[row] : 0.f;
   const bool greedy = !(temp > 1e-10f);
   const float inv_temp = greedy ? 1.f : 1.f / temp;
   const uint64_t seed = seeds ? seeds[row] : 0ull;
+  uint32_t keep_from = 0;      // the smallest ordered key that is kept
+  if (hist && !greedy) {       // the same for the whole block
+    if (threadIdx.x < SE_WAVE) {
+      const int k = top_k ? top_k[row] : 0;
+      const float p = top_p ? top_p[row] : 1.f;
+      const u64* hist_row = hist + static_cast<int64_t>(row) * 2 * FILTER_PASSES * FILTER_BINS;
+      uint32_t from = 0;
+      if (k > 0 && k < vocab) from = bits_found(hist_row, FILTER_PASSES, static_cast<u64>(k), false);
+      if (p < 1.f) {
+        const u64* weights = hist_row + FILTER_PASSES * FILTER_BINS;
+        const uint32_t nucleus = bits_found(weights, FILTER_PASSES, nucleus_budget(weights, p), true);
+        if (nucleus > from) from = nucleus;
+      }
+      if (threadIdx.x == 0) shared_keep_from = from;
+    }
+    __syncthreads();
+    keep_from = shared_keep_from;
+  }
   const int begin = chunk * SAMPLE_CHUNK;
   const int end = begin + SAMPLE_CHUNK < vocab ? begin + SAMPLE_CHUNK : vocab;
   ArgBest best = {-INFINITY, -1};
@@ -180,7 +309,9 @@ sample_partial_kernel(const float* __restrict__ logits, int64_t stride, int voca
       if (greedy) {
         if (v != v) v = INFINITY;
       } else {
-        v = v * inv_temp - logf(-logf(uniform_open(seed, static_cast<uint32_t>(i))));
+        v = v * inv_temp;
+        if (ordered_key(v) < keep_from) continue;
+        v -= logf(-logf(uniform_open(seed, static_cast<uint32_t>(i))));
       }
       ArgBest c = {v, i};
       best = better(best, c);
@@ -216,25 +347,47 @@ extern "C" int se_sample_unfiltered(const float* logits, int64_t stride, int row
   const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
   if (chunks > 65535) return SE_ERR_SHAPE;
   sample_partial_kernel<<<dim3(rows, chunks), SAMPLE_THREADS, 0, stream>>>(
-      logits, stride, vocab, temperature, seeds, part_value, part_index, chunks);
+      logits, stride, vocab, temperature, seeds, part_value, part_index, chunks, nullptr, nullptr, nullptr);
   SE_CHECK_LAUNCH();
   sample_final_kernel<<<rows, SE_WAVE, 0, stream>>>(part_value, part_index, chunks, out);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }
 
+// Rows with top_k and / or top_p (either may be null: off for every row); `temperature` is needed.
+// Workspace: part_value, part_index as above, part_max [rows * ceil(vocab / 4096)] floats,
+// hist [rows * 2048] 64-bit words (cleared here).
 extern "C" int se_sample(const float* logits, int64_t stride, int rows, int vocab,
                          const float* temperature, const int32_t* top_k, const float* top_p,
-                         const uint64_t* seeds, int32_t* out, hipStream_t stream) {
+                         const uint64_t* seeds, float* part_value, int32_t* part_index, float* part_max,
+                         unsigned long long* hist, int32_t* out, hipStream_t stream) {
   if (rows <= 0) return SE_OK;
-  if (vocab <= 0) return SE_ERR_SHAPE;
-  sample_kernel<<<rows, SAMPLE_THREADS, 0, stream>>>(logits, stride, vocab, temperature, top_k,
-                                                     top_p, seeds, out);
+  if (vocab <= 0 || !temperature || !part_value || !part_index || !part_max || !hist) return SE_ERR_SHAPE;
+  const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  if (chunks > 65535) return SE_ERR_SHAPE;
+  const dim3 grid(rows, chunks);
+  const int64_t words = static_cast<int64_t>(rows) * 2 * FILTER_PASSES * FILTER_BINS;
+  zero_words_kernel<<<static_cast<unsigned>((words + 255) / 256), 256, 0, stream>>>(hist, words);
+  if (top_k)
+    for (int pass = 0; pass < FILTER_PASSES; ++pass)
+      sample_filter_pass_kernel<false><<<grid, SAMPLE_THREADS, 0, stream>>>(
+          logits, stride, vocab, temperature, top_k, top_p, part_max, hist, pass, chunks);
+  if (top_p) {
+    sample_chunk_max_kernel<<<grid, SAMPLE_THREADS, 0, stream>>>(logits, stride, vocab, temperature, top_p,
+                                                                 part_max, chunks);
+    for (int pass = 0; pass < FILTER_PASSES; ++pass)
+      sample_filter_pass_kernel<true><<<grid, SAMPLE_THREADS, 0, stream>>>(
+          logits, stride, vocab, temperature, top_k, top_p, part_max, hist, pass, chunks);
+  }
+  SE_CHECK_LAUNCH();
+  sample_partial_kernel<<<grid, SAMPLE_THREADS, 0, stream>>>(
+      logits, stride, vocab, temperature, seeds, part_value, part_index, chunks, top_k, top_p, hist);
+  SE_CHECK_LAUNCH();
+  sample_final_kernel<<<rows, SE_WAVE, 0, stream>>>(part_value, part_index, chunks, out);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }
 
-// ---------------------------------------------------------------------------------------- //
 // The same arg-max sampling for callers that cannot allocate (no_alloc.h): the partial maxima go
 // to a fixed array in device memory instead of a workspace of the caller's.
 // ---------------------------------------------------------------------------------------- //
@@ -263,7 +416,7 @@ extern "C" int se_sample_unfiltered_no_alloc(const float* logits, int64_t stride
   float* part_value = reinterpret_cast<float*>(scratch_of_device[device]);
   int32_t* part_index = reinterpret_cast<int32_t*>(scratch_of_device[device] + SE_NO_ALLOC_SAMPLE_SLOTS * sizeof(float));
   sample_partial_kernel<<<dim3(rows, chunks), SAMPLE_THREADS, 0, stream>>>(
-      logits, stride, vocab, temperature, seeds, part_value, part_index, chunks);
+      logits, stride, vocab, temperature, seeds, part_value, part_index, chunks, nullptr, nullptr, nullptr);
   SE_CHECK_LAUNCH();
   sample_final_kernel<<<rows, SE_WAVE, 0, stream>>>(part_value, part_index, chunks, out);
   SE_CHECK_LAUNCH();

@@ -115,7 +115,7 @@ _SIGNATURES = {
     },
     "sampling": {
         "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                      c_void_p, c_void_p],
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_sample_unfiltered": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_void_p],
     },
@@ -641,16 +641,24 @@ class HipKernels:
                             ("top_p", top_p, torch.float32), ("seeds", seeds, torch.int64)):
             if t is not None:
                 _require(t.dtype == dt and t.numel() == rows and t.is_contiguous(), f"sample {name}")
-        if top_k is None and top_p is None:       # one arg-max per row: spread over many blocks
-            need = rows * (-(-vocab // 4096))
-            if self._sample_partials is None or self._sample_partials[0].numel() < need:
-                self._sample_partials = (torch.empty(need, dtype=torch.float32, device=logits.device),
-                                         torch.empty(need, dtype=torch.int32, device=logits.device))
+        need = rows * (-(-vocab // 4096))
+        if self._sample_partials is None or self._sample_partials[0].numel() < need:
+            self._sample_partials = (torch.empty(need, dtype=torch.float32, device=logits.device),
+                                     torch.empty(need, dtype=torch.int32, device=logits.device))
+        if top_k is None and top_p is None:       # one arg-max per row, spread over many blocks
             _check(_fn.get("sampling", "se_sample_unfiltered")(
                 _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(seeds),
                 _ptr(self._sample_partials[0]), _ptr(self._sample_partials[1]), _ptr(out), _stream()),
                 "sample")
             return
+        # top-k / top-p: passes over the row that count and weigh its tokens by eight bits of their value at a time
+        _require(temperature is not None, "sample: top_k / top_p need temperatures")
+        filters = getattr(self, "_sample_filters", None)
+        if filters is None or filters[0].numel() < need or filters[1].numel() < rows * 2048:
+            filters = (torch.empty(need, dtype=torch.float32, device=logits.device),
+                       torch.empty(rows * 2048, dtype=torch.int64, device=logits.device))
+            self._sample_filters = filters
         _check(_fn.get("sampling", "se_sample")(
             _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
-            _ptr(seeds), _ptr(out), _stream()), "sample")
+            _ptr(seeds), _ptr(self._sample_partials[0]), _ptr(self._sample_partials[1]), _ptr(filters[0]),
+            _ptr(filters[1]), _ptr(out), _stream()), "sample")

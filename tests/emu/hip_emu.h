@@ -373,6 +373,11 @@ inline int atomicAdd(int* p, int v) {
   *p = old + v;
   return old;
 }
+inline unsigned long long atomicAdd(unsigned long long* p, unsigned long long v) {
+  const unsigned long long old = *p;
+  *p = old + v;
+  return old;
+}
 
 enum { EMU_OP_SHFL = 1, EMU_OP_BALLOT, EMU_OP_DPP, EMU_OP_SWAP16, EMU_OP_SWAP32, EMU_OP_MFMA };
 

@@ -147,6 +147,8 @@ def test_slot_sum_dense_products_and_sampling(guard, twin):
         G.test_rounding_to_bfloat16_is_to_nearest_even(hip)
         G.test_expert_tables_arranged_in_place_are_the_tiled_copy(hip, twin)
         G.test_sampling(hip, twin)
+        if guard == "after":
+            G.test_sampling_keeps_exactly_the_tokens_of_the_filters(hip, 5000, 0.1, 128)
         for dtype in (F32, BF16):
             for shape in [(1, 8, 3072), (5, 2, 256), (7, 3, 200), (3, 4, 20)]:
                 G.test_norm_adds_up_slots_as_it_reads(hip, dtype, *shape)

@@ -549,11 +549,56 @@ def test_sampling(hip, twin):
     hip.sample(big, t5, None, None, s5, fast)
     hip.sample(big, t5, torch.zeros(5, dtype=torch.int32).to(DEV), None, s5, slow)
     assert torch.equal(fast, slow) and int(fast[0]) == int(big[0].argmax())
+    # filters over a vocabulary of several chunks, with many equal logits in some rows (whole groups of equal
+    # values stay or go), a top_k beyond the vocabulary and a nucleus that is one token
+    coarse = big.clone()
+    coarse[2:] = (coarse[2:] * 2).round() / 2
+    t5 = torch.tensor([0.0, 0.7, 1.0, 1.5, 0.3]).to(DEV)
+    k5 = torch.tensor([3, 40, 1000, 0, 30000], dtype=torch.int32).to(DEV)
+    p5 = torch.tensor([0.5, 0.9, 0.95, 0.3, 1e-4]).to(DEV)
+    ref5 = torch.empty_like(fast)
+    for rows_k, rows_p in ((k5, p5), (k5, None), (None, p5)):
+        hip.sample(coarse, t5, rows_k, rows_p, s5, fast)
+        twin.sample(coarse, t5, rows_k, rows_p, s5, ref5)
+        assert torch.equal(fast, ref5), (fast.tolist(), ref5.tolist())
+    assert int(fast[4]) == int(coarse[4].argmax())
     # a row's draw does not depend on the rest of the batch
     one = torch.empty(1, dtype=torch.int32, device=DEV)
     for r in range(rows):
         hip.sample(logits[r:r + 1], temp[r:r + 1], top_k[r:r + 1], top_p[r:r + 1], seeds[r:r + 1], one)
         assert int(one) == int(out[r])
+
+
+@pytest.mark.parametrize("vocab,slope,draws", [(5000, 0.1, 128), (5000, 0.06, 256), (20011, 0.01, 8192)])
+def test_sampling_keeps_exactly_the_tokens_of_the_filters(hip, vocab, slope, draws):
+    """The kept set itself, to the single token: logits fall off evenly over tokens scattered through the
+    vocabulary (several chunks), so that top_p = 0.5 keeps a few dozen of them, each likely enough to be drawn
+    several times; the tokens drawn over many seeds are then exactly the set that float64 arithmetic keeps.
+    The same for top_k."""
+    emulator_skips(draws * vocab, 2e6)
+    g = torch.Generator().manual_seed(11)
+    order = torch.randperm(vocab, generator=g)
+    ranked = 2000 if vocab > 10000 else 400
+    row = torch.full((vocab,), -50.0)
+    row[order[:ranked]] = -slope * torch.arange(ranked, dtype=torch.float32)
+    logits = row[None].repeat(draws, 1).to(DEV)
+    seeds = (torch.arange(draws, dtype=torch.int64) * 0x9E3779B1 + 99).to(DEV)
+    out = torch.empty(draws, dtype=torch.int32, device=DEV)
+    ones = torch.ones(draws).to(DEV)
+    prob = torch.softmax(row.double(), 0)[order]            # in descending order
+    before = torch.cumsum(prob, 0) - prob
+    nucleus = int((before <= 0.5).sum())
+    assert 6 <= nucleus <= 80
+    hip.sample(logits, ones, None, torch.full((draws,), 0.5).to(DEV), seeds, out)
+    assert set(out.tolist()) == set(order[:nucleus].tolist())
+    k = nucleus - 3
+    hip.sample(logits, ones, torch.full((draws,), k, dtype=torch.int32).to(DEV), None, seeds, out)
+    assert set(out.tolist()) == set(order[:k].tolist())
+    # both: the nucleus is taken among the survivors of top-k
+    inside = prob[:k] / prob[:k].sum()
+    both = int(((torch.cumsum(inside, 0) - inside) <= 0.5).sum())
+    hip.sample(logits, ones, torch.full((draws,), k, dtype=torch.int32).to(DEV), torch.full((draws,), 0.5).to(DEV), seeds, out)
+    assert set(out.tolist()) == set(order[:both].tolist()) and both < nucleus
 
 
 def test_sampling_distribution(hip):
