@@ -222,7 +222,7 @@ class LLM:
             wanting = [i.seq for i in schedule.items if i.wants_logits]
             sampled, logprobs = {}, {}
             if wanting:
-                rows = [(s.sampling_params, s.prompt_token_ids, s.completion_token_ids) for s in wanting]
+                rows = [(s.sampling_params, s.prompt_token_ids, s.completion_token_ids, s.sampler_notes) for s in wanting]
                 logits = self.sampler.apply_penalties(logits, rows)
                 tokens = self.sampler.sample(logits, rows, [(s.seed, s.num_completion_tokens) for s in wanting])
                 chosen, tops = self.sampler.logprobs(logits, tokens, [s.sampling_params.logprobs for s in wanting])

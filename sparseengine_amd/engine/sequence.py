@@ -29,6 +29,7 @@ class Sequence:
         self.num_computed_tokens = 0        # tokens whose keys and values are in the cache
         self.num_preemptions = 0
         self.seed = sampling_params.seed if sampling_params.seed is not None else self.seq_id
+        self.sampler_notes: dict = {}       # what the sampler keeps about this request between steps
 
     @property
     def num_prompt_tokens(self) -> int:

@@ -36,25 +36,36 @@ class Sampler:
         self.sampler_seed = int(sampler_seed)
 
     def apply_penalties(self, logits: torch.Tensor, rows) -> torch.Tensor:
-        """``rows``: per logits row (params, prompt ids, completion ids)."""
-        if not any(p.presence_penalty != 0.0 or p.repetition_penalty != 1.0 for p, _, _ in rows):
+        """``rows``: per logits row (params, prompt ids, completion ids[, a dict that lives as long as the
+        request]).  The distinct tokens of a prompt are worked out once per request and kept in that dict (a
+        prompt of many thousand tokens would otherwise cost milliseconds of set building in every step);
+        the completion's tokens go as they are: a token named twice is still changed once."""
+        if not any(row[0].presence_penalty != 0.0 or row[0].repetition_penalty != 1.0 for row in rows):
             return logits
         logits = logits.clone()
-        for r, (p, prompt, completion) in enumerate(rows):
+        for r, row in enumerate(rows):
+            p, prompt, completion = row[:3]
+            kept = row[3] if len(row) > 3 else None
+            generated = torch.tensor(completion, dtype=torch.long, device=logits.device) if completion else None
             if p.repetition_penalty != 1.0 and (prompt or completion):
-                seen = torch.tensor(sorted(set(prompt) | set(completion)), dtype=torch.long, device=logits.device)
+                seen = kept.get("prompt_tokens") if kept is not None else None
+                if seen is None or seen.device != logits.device:
+                    seen = torch.tensor(sorted(set(prompt)), dtype=torch.long, device=logits.device)
+                    if kept is not None:
+                        kept["prompt_tokens"] = seen
+                if generated is not None:
+                    seen = torch.cat((seen, generated))
                 values = logits[r, seen]
                 logits[r, seen] = torch.where(values > 0, values / p.repetition_penalty, values * p.repetition_penalty)
-            if p.presence_penalty != 0.0 and completion:
-                seen = torch.tensor(sorted(set(completion)), dtype=torch.long, device=logits.device)
-                logits[r, seen] -= p.presence_penalty
+            if p.presence_penalty != 0.0 and generated is not None:
+                logits[r, generated] = logits[r, generated] - p.presence_penalty
         return logits
 
     def sample(self, logits: torch.Tensor, rows, seeds_and_positions) -> list[int]:
         """``logits`` float32 ``[n, vocab]``; ``rows`` as in ``apply_penalties``;
         ``seeds_and_positions``: per row (request seed, index of the token being drawn)."""
         n = logits.shape[0]
-        params = [p for p, _, _ in rows]
+        params = [row[0] for row in rows]
         out = torch.empty(n, dtype=torch.int32, device=logits.device)
         if all(p.greedy for p in params):
             self.kernels.sample(logits, None, None, None, None, out)
