@@ -10,6 +10,7 @@ before the kernel; log-probabilities are ``log_softmax`` of the penalised float 
 """
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 _MASK = (1 << 64) - 1
@@ -70,12 +71,18 @@ class Sampler:
         if all(p.greedy for p in params):
             self.kernels.sample(logits, None, None, None, None, out)
             return out.tolist()
-        temperature = torch.tensor([0.0 if p.greedy else p.temperature for p in params], dtype=torch.float32)
-        top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32) if any(p.top_k for p in params) else None
-        top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32) if any(p.top_p < 1.0 for p in params) else None
-        seeds = torch.tensor([row_seed(self.sampler_seed, s, pos) for s, pos in seeds_and_positions], dtype=torch.int64)
-        to = lambda t: None if t is None else t.to(logits.device)
-        self.kernels.sample(logits, to(temperature), to(top_k), to(top_p), to(seeds), out)
+        # the rows' settings go to the device in one copy: seeds (64 bits each), then temperatures, top_p, top_k
+        packed = np.empty(n * 20, dtype=np.uint8)
+        packed[:8 * n].view(np.int64)[:] = [row_seed(self.sampler_seed, s, pos) for s, pos in seeds_and_positions]
+        packed[8 * n:12 * n].view(np.float32)[:] = [0.0 if p.greedy else p.temperature for p in params]
+        packed[12 * n:16 * n].view(np.float32)[:] = [p.top_p for p in params]
+        packed[16 * n:].view(np.int32)[:] = [p.top_k for p in params]
+        on_device = torch.from_numpy(packed).to(logits.device)
+        seeds = on_device[:8 * n].view(torch.int64)
+        temperature = on_device[8 * n:12 * n].view(torch.float32)
+        top_p = on_device[12 * n:16 * n].view(torch.float32) if any(p.top_p < 1.0 for p in params) else None
+        top_k = on_device[16 * n:].view(torch.int32) if any(p.top_k for p in params) else None
+        self.kernels.sample(logits, temperature, top_k, top_p, seeds, out)
         return out.tolist()
 
     @staticmethod
