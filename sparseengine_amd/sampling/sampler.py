@@ -91,12 +91,14 @@ class Sampler:
         if all(t is None for t in top):
             return [None] * len(tokens), [None] * len(tokens)
         logp = torch.log_softmax(logits, dim=-1)
-        chosen = logp.gather(1, torch.tensor(tokens, device=logits.device)[:, None])[:, 0].tolist()
+        chosen = logp.gather(1, torch.tensor(tokens, device=logits.device)[:, None])
+        most = max(k or 0 for k in top)
+        if most:        # one top-k for all rows (a row's first k entries are its own top k), one copy to the host
+            values, ids = torch.topk(logp, min(most, logp.shape[1]))
+            chosen, values, ids = torch.cat((chosen, values), 1).tolist(), None, ids.tolist()
+        else:
+            chosen, ids = chosen.tolist(), None
         tops = []
         for r, k in enumerate(top):
-            if not k:
-                tops.append(None if k is None else {})
-                continue
-            values, ids = torch.topk(logp[r], k)
-            tops.append(dict(zip(ids.tolist(), values.tolist())))
-        return [c if k is not None else None for c, k in zip(chosen, top)], tops
+            tops.append(None if k is None else dict(zip(ids[r][:k], chosen[r][1:1 + k])) if k else {})
+        return [chosen[r][0] if k is not None else None for r, k in enumerate(top)], tops
