@@ -39,27 +39,44 @@ class Sampler:
     def apply_penalties(self, logits: torch.Tensor, rows) -> torch.Tensor:
         """``rows``: per logits row (params, prompt ids, completion ids[, a dict that lives as long as the
         request]).  The distinct tokens of a prompt are worked out once per request and kept in that dict (a
-        prompt of many thousand tokens would otherwise cost milliseconds of set building in every step);
-        the completion's tokens go as they are: a token named twice is still changed once."""
+        prompt of many thousand tokens would otherwise cost milliseconds of set building in every step).
+        All rows are changed together, through flat positions ``row * vocab + token``: a dozen launches a
+        step instead of a dozen a row.  A token named twice is still changed once."""
         if not any(row[0].presence_penalty != 0.0 or row[0].repetition_penalty != 1.0 for row in rows):
             return logits
-        logits = logits.clone()
+        logits = logits.clone(memory_format=torch.contiguous_format)
+        n, vocab = logits.shape
+        flat = logits.view(-1)
+        prompts, repeated, present = [], [], []
         for r, row in enumerate(rows):
             p, prompt, completion = row[:3]
             kept = row[3] if len(row) > 3 else None
-            generated = torch.tensor(completion, dtype=torch.long, device=logits.device) if completion else None
-            if p.repetition_penalty != 1.0 and (prompt or completion):
-                seen = kept.get("prompt_tokens") if kept is not None else None
-                if seen is None or seen.device != logits.device:
-                    seen = torch.tensor(sorted(set(prompt)), dtype=torch.long, device=logits.device)
-                    if kept is not None:
-                        kept["prompt_tokens"] = seen
-                if generated is not None:
-                    seen = torch.cat((seen, generated))
-                values = logits[r, seen]
-                logits[r, seen] = torch.where(values > 0, values / p.repetition_penalty, values * p.repetition_penalty)
-            if p.presence_penalty != 0.0 and generated is not None:
-                logits[r, generated] = logits[r, generated] - p.presence_penalty
+            if p.repetition_penalty != 1.0:
+                if prompt:
+                    seen = kept.get("prompt_tokens") if kept is not None else None
+                    if seen is None or seen.device != logits.device:
+                        seen = torch.tensor(sorted(set(prompt)), dtype=torch.long, device=logits.device)
+                        if kept is not None:
+                            kept["prompt_tokens"] = seen
+                    prompts.append(seen + r * vocab)
+                repeated += [r * vocab + t for t in completion]
+            if p.presence_penalty != 0.0:
+                present += [r * vocab + t for t in completion]
+        # one copy: the rows' two penalties, then the flat positions of the completions' tokens
+        packed = np.empty(8 * n + 8 * (len(repeated) + len(present)), dtype=np.uint8)
+        packed[:4 * n].view(np.float32)[:] = [row[0].repetition_penalty for row in rows]
+        packed[4 * n:8 * n].view(np.float32)[:] = [row[0].presence_penalty for row in rows]
+        packed[8 * n:].view(np.int64)[:] = repeated + present
+        on_device = torch.from_numpy(packed).to(logits.device)
+        repetition, presence = on_device[:4 * n].view(torch.float32), on_device[4 * n:8 * n].view(torch.float32)
+        places = on_device[8 * n:].view(torch.int64)
+        where = torch.cat(prompts + [places[:len(repeated)]]) if prompts else places[:len(repeated)]
+        if where.numel():
+            values, factor = flat[where], repetition[where // vocab]
+            flat[where] = torch.where(values > 0, values / factor, values * factor)
+        if present:
+            where = places[len(repeated):]
+            flat[where] = flat[where] - presence[where // vocab]
         return logits
 
     def sample(self, logits: torch.Tensor, rows, seeds_and_positions) -> list[int]:

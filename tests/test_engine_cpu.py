@@ -186,6 +186,32 @@ def test_penalties_logprobs_and_eos(model):
     assert set(tops[0]) == set(torch.topk(ref, 2).indices.tolist())
 
 
+def test_penalties_of_several_rows_at_once():
+    """Rows with different penalties in one call, tokens named twice, a row without any: against the rule applied
+    row by row (reference layers/sampler.py:11-64); a prompt's distinct tokens are kept with the request."""
+    from sparseengine_amd.sampling.sampler import Sampler
+    torch.manual_seed(0)
+    vocab = 50
+    logits = torch.randn(4, vocab)
+    rows = [(SamplingParams(repetition_penalty=1.5), [3, 3, 7, 49], [7, 8, 8], {}),
+            (SamplingParams(presence_penalty=2.0), [1, 2], [5, 5, 0], {}),
+            (SamplingParams(), [4], [4, 4], {}),
+            (SamplingParams(repetition_penalty=0.5, presence_penalty=-1.0), [9], [], {})]
+    expect = logits.clone()
+    for r, (p, prompt, completion, _) in enumerate(rows):
+        if p.repetition_penalty != 1.0:
+            for t in set(prompt) | set(completion):
+                expect[r, t] = expect[r, t] / p.repetition_penalty if expect[r, t] > 0 else expect[r, t] * p.repetition_penalty
+        for t in set(completion):
+            expect[r, t] -= p.presence_penalty
+    sampler = Sampler(None, "cpu")
+    before = logits.clone()
+    for _ in range(2):      # the second call finds the prompts' tokens where the first left them
+        torch.testing.assert_close(sampler.apply_penalties(logits, rows), expect)
+    assert torch.equal(logits, before), "the caller's logits are not touched"
+    assert rows[0][3]["prompt_tokens"].tolist() == [3, 7, 49] and not rows[1][3]
+
+
 def test_attention_work_lists_cover_every_row_and_key_once():
     for q_len, ctx, group, kvh, window in [([1], [2049], 6, 8, 0), ([1] * 64, [2200 - i for i in range(64)], 6, 8, 0),
                                             ([37, 23, 1], [37, 150, 301], 2, 2, 0), ([2048], [2048], 6, 8, 0),
