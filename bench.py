@@ -98,7 +98,8 @@ def main() -> int:
     t0 = time.time()
     runner = ModelRunner.from_random(
         cfg, seed=0, options=dict(std=0.02, norm_std=0.1, bias_std=0.01), on_device=True, dtype=args.dtype,
-        kv_page_size=64, num_kvcache_tokens=args.kv_requests * CONTEXT_LEN, max_num_seqs=max(64, args.batch),
+        kv_page_size=64, num_kvcache_tokens=args.kv_requests * CONTEXT_LEN,
+        max_num_seqs=max([64, args.batch] + [int(x) for x in args.points.split(",") if x]),
         max_model_len=CONTEXT_LEN)
     torch.cuda.synchronize()
     print(f"[bench] model built in {time.time() - t0:.1f} s, "
