@@ -67,6 +67,8 @@ def build_parser() -> argparse.ArgumentParser:
     gen.add_argument("--prompt", action="append", default=[], help="text prompt (needs tokenizer.json); repeatable")
     gen.add_argument("--prompt-ids", action="append", default=[],
                      help="prompt as JSON list of token ids, or a file with one JSON list per line; repeatable")
+    gen.add_argument("--device", default="cuda", choices=["cuda", "cpu"],
+                     help="cpu runs only with a stand-in for the HIP kernels named in SPARSEENGINE_AMD_KERNELS (tests)")
     _add_dataclass_options(gen, Config, skip=("model",))
     _add_dataclass_options(gen, SamplingParams, prefix_if_taken="sampling_")
 
@@ -117,7 +119,13 @@ def main(argv=None) -> int:
             prompts.append(json.loads(item))
     if not prompts:
         parser.error("give at least one --prompt or --prompt-ids")
-    llm = LLM(args.model, **_collect(args, Config, skip=("model",)))
+    from .engine.runner import kernels_for_program
+    try:
+        kernels, device = kernels_for_program(args.device)
+    except ValueError as exc:
+        parser.error(str(exc))
+    seam = {} if kernels is None else {"_kernels": kernels, "_device": device}
+    llm = LLM(args.model, **_collect(args, Config, skip=("model",)), **seam)
     params = SamplingParams(**_collect(args, SamplingParams, prefix="sampling_"))
     for prompt, out in zip(prompts, llm.generate(prompts, params, use_tqdm=False)):
         print(json.dumps({"prompt": prompt, **out}))

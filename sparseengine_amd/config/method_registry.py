@@ -1,8 +1,10 @@
 """Registry of sparse-attention methods and their prefill policies.
 
 Only the dense method is registered: ``""`` (alias ``"vanilla"``) with the ``all_chunked`` prefill
-policy.  The hook is kept so that another method could bring its own cache manager and step
-hooks later (reference method_registry.py:19-36,508-525,646-665; the pass-through runtime
+policy and the paged cache manager.  A method brings three things under its name: the runtime with
+its step hooks, its prefill policy and the class of its cache manager, which the model runner builds
+in place of the paged one (reference: method_registry.py:19-36,508-525,646-665; the cache-manager
+factory by method engine/cache_manager/base.py:537-647; the pass-through runtime
 engine/sparse_methods/passthrough.py:11-32).
 """
 from __future__ import annotations
@@ -62,17 +64,27 @@ class MethodBinding:
     name: str
     runtime_factory: type
     prefill_policy: str
-    cache_manager: str = "paged"
+    cache_manager_cls: type | None = None      # None: cache.manager.CacheManager
+
+    def cache_manager(self) -> type:
+        """The class the model runner builds its cache manager from: the method's own (a subclass of
+        ``CacheManager``, or anything with its constructor and interface), else the paged one."""
+        if self.cache_manager_cls is not None:
+            return self.cache_manager_cls
+        from ..cache.manager import CacheManager
+        return CacheManager
 
 
 _METHODS: dict[str, MethodBinding] = {}
 PREFILL_POLICIES = {"all_chunked"}
 
 
-def register_method(name: str, runtime_factory, prefill_policy: str, cache_manager: str = "paged") -> None:
+def register_method(name: str, runtime_factory, prefill_policy: str, cache_manager_cls: type | None = None) -> None:
     if prefill_policy not in PREFILL_POLICIES:
         raise ValueError(f"unknown prefill policy {prefill_policy!r}; known: {sorted(PREFILL_POLICIES)}")
-    _METHODS[name] = MethodBinding(name, runtime_factory, prefill_policy, cache_manager)
+    if cache_manager_cls is not None and not callable(cache_manager_cls):
+        raise TypeError("cache_manager_cls must be a class with the constructor of cache.manager.CacheManager")
+    _METHODS[name] = MethodBinding(name, runtime_factory, prefill_policy, cache_manager_cls)
 
 
 def normalize_sparse_method(name: str | None) -> str:

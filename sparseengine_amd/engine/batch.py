@@ -34,6 +34,7 @@ class GroupMeta:
     positions: torch.Tensor        # int32 [T]
     slots: torch.Tensor            # int32 [T] page * page_size + offset of the token's own key
     page_size: int
+    block_table_host: np.ndarray = None   # block_table on the host (for checks before a launch)
     # host copies for kernels that build a work list
     item_q_start: np.ndarray = None
     item_q_len: np.ndarray = None
@@ -67,10 +68,12 @@ class ForwardBatch:
         self.item_q_len = None
         self.item_ctx_len = None
         self.item_meta = None
+        self.schedule_position = 0     # the schedule position whose layer is running
         self.method = None             # the sparse method's runtime (config/method_registry.py)
         self.want_index = None         # int32 [wanted] token indices whose logits are returned
         self.groups: dict[int, GroupMeta] = {}
         self.taps: dict | None = None
+        self.check_tables = False      # check every block-table entry a launch will read (a debug option)
 
     # views the mixers use ---------------------------------------------------------------
     def kv_view(self, position: int):
@@ -81,6 +84,9 @@ class ForwardBatch:
         """name -> [rows, ...] state tensors of the position; index them with ``item_rows``."""
         return self.cache.state[position]
 
+    def check_block_table(self, meta, window: int, num_pages: int, where: str = "") -> None:
+        check_block_table(meta, window, num_pages, where)
+
     def buffer(self, key: str, shape, dtype=None) -> torch.Tensor:
         """A reusable scratch tensor whose leading dims are cut to ``shape``."""
         shape = tuple(int(s) for s in shape)
@@ -88,6 +94,39 @@ class ForwardBatch:
         # one buffer per (purpose, row shape): only the leading dim is ever cut, so views stay dense
         full = self.scratch.get(f"{key}{shape[1:]}", shape, dtype, self.device)
         return full if full.shape[0] == shape[0] else full.narrow(0, 0, shape[0])
+
+
+class BlockTableError(RuntimeError):
+    pass
+
+
+def check_block_table(meta, window: int, num_pages: int, where: str = "") -> None:
+    """Before an attention launch: every block-table entry that the launch will read names a page of the
+    pool.  Item ``i`` holds ``ctx_len[i]`` tokens of which the last ``q_len[i]`` are this step's queries; its
+    first query sees the keys from ``max(0, position - window + 1)`` on (``window`` 0: all), so the entries
+    from that key's page to the last key's page are read and must lie in ``[0, num_pages)``; entries before
+    them may be -1 (pages a window has given back) and are not read.  A kernel that follows a bad entry
+    reads outside the cache tensor, which the device may or may not answer with a memory fault.
+    (The reference checks its slot tables the same way under a debug flag, layers/attention_backend.py:155-215.)"""
+    table = getattr(meta, "block_table_host", None)
+    if table is None:
+        table = meta.block_table.cpu().numpy()
+    q_len, ctx_len, page = np.asarray(meta.item_q_len), np.asarray(meta.item_ctx_len), int(meta.page_size)
+    first_query = ctx_len - q_len
+    low_key = np.maximum(0, first_query - window + 1) if window else np.zeros_like(ctx_len)
+    if (q_len <= 0).any() or (first_query < 0).any():
+        raise BlockTableError(f"{where}: an item with {q_len.tolist()} queries of {ctx_len.tolist()} tokens")
+    first_page, until_page = low_key // page, -(-ctx_len // page)
+    if int(until_page.max()) > table.shape[1]:
+        raise BlockTableError(f"{where}: the block table has {table.shape[1]} columns, an item needs {int(until_page.max())}")
+    column = np.arange(table.shape[1])[None, :]
+    read = (column >= first_page[:, None]) & (column < until_page[:, None])
+    bad = read & ((table < 0) | (table >= num_pages))
+    if bad.any():
+        item, col = (int(v[0]) for v in np.nonzero(bad))
+        raise BlockTableError(
+            f"{where}: item {item} (tokens {int(ctx_len[item])}, queries {int(q_len[item])}, window {window or 'none'}) "
+            f"would read block-table entry {col} = {int(table[item, col])}; the pool has pages 0..{num_pages - 1}")
 
 
 class BatchBuilder:
@@ -187,6 +226,7 @@ class BatchBuilder:
         for gi, group in enumerate(cache.groups):
             fb.groups[group.index] = GroupMeta(
                 block_table=view(6 + 2 * gi + 1, tables[group.index].shape),
+                block_table_host=tables[group.index],
                 token_row=fb.token_item, positions=fb.positions, slots=view(6 + 2 * gi),
                 page_size=cache.page_size, item_q_start=q_start, item_q_len=q_len,
                 item_ctx_len=ctx_len, item_meta=item_meta, max_ctx_len=int(ctx_len.max()),

@@ -135,11 +135,14 @@ class LLM:
         kernels = kwargs.pop("_kernels", None)           # test seam: the kernel twins on the CPU
         device = kwargs.pop("_device", "cuda")
         self.config = config = Config.from_kwargs(model, **kwargs)
-        self.method = resolve_method(config.sparse_method).runtime_factory()
+        binding = resolve_method(config.sparse_method)
+        self.method = binding.runtime_factory()
         cache_tokens = config.num_kvcache_slots
         common = dict(dtype=config.dtype, device=device, kv_page_size=config.kv_page_size,
                       max_num_seqs=config.max_num_seqs_in_gpu, max_model_len=config.max_model_len,
-                      mlp_chunk_size=config.mlp_chunk_size, kernels=kernels, method=self.method)
+                      mlp_chunk_size=config.mlp_chunk_size, kernels=kernels, method=self.method,
+                      cache_manager_cls=binding.cache_manager(),
+                      validate_runtime_invariants=config.validate_runtime_invariants)
         if config.tiny_random:
             self.runner = ModelRunner.from_random(config.raw_model_config, seed=config.tiny_random_seed,
                                                   on_device=config.tiny_random_on_device,
@@ -247,8 +250,8 @@ class LLM:
     # ------------------------------------------------------------------ the blocking call
     def generate(self, prompts, sampling_params, use_tqdm: bool = True) -> list[dict]:
         if isinstance(sampling_params, list) and len(sampling_params) != len(prompts):
-            raise ValueError("prompts and sampling_params must have the same length when sampling_params "
-                             f"is a list: prompts={len(prompts)} sampling_params={len(sampling_params)}.")
+            raise ValueError(f"{len(prompts)} prompts came with a list of {len(sampling_params)} sampling_params: "
+                             "give one for all prompts, or one per prompt")
         if not isinstance(sampling_params, list):
             sampling_params = [sampling_params] * len(prompts)
         order = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]

@@ -81,6 +81,8 @@ def build_parser() -> argparse.ArgumentParser:
                         help="max_model_len; default: longest length + output_len + 100")
     parser.add_argument("--hyper_params", default="{}", help="keyword arguments of LLM(...) as JSON or @file")
     parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--device", default="cuda", choices=["cuda", "cpu"],
+                        help="cpu runs only with a stand-in for the HIP kernels named in SPARSEENGINE_AMD_KERNELS (tests)")
     parser.add_argument("--output_jsonl", default=None, help="write one JSON row per case here as well")
     return parser
 
@@ -96,6 +98,10 @@ def main(argv=None, llm_factory=None) -> int:
     kwargs.setdefault("max_num_seqs_in_batch", max(batches))
     if llm_factory is None:
         from .llm import LLM
+        from .runner import kernels_for_program
+        kernels, device = kernels_for_program(args.device)
+        if kernels is not None:
+            kwargs.update(_kernels=kernels, _device=device)
         llm_factory = LLM
     llm = llm_factory(args.model_path, **kwargs)
     sync = None

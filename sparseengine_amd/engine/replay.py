@@ -25,7 +25,7 @@ import sys
 
 import numpy as np
 
-from .runner import ModelRunner, StepEntry
+from .runner import ModelRunner, StepEntry, kernels_for_program
 
 
 def pages_held(runner: ModelRunner, request_ids) -> dict[str, dict[str, list[int]]]:
@@ -90,6 +90,16 @@ def replay_stream(runner: ModelRunner, lines, out_dir: str, report=sys.stdout, w
     return steps
 
 
+def pool_tokens(max_tokens: int, page_size: int, max_requests: int) -> int:
+    """Tokens of cache for ``--max-tokens`` (the live requests' lengths, each rounded up to a multiple of
+    64, added up).  Pages that divide 64 hold exactly that; with other page sizes (48, 128) a request's
+    last page may reach beyond its multiple of 64, by less than a page per live request."""
+    rounded = -(-max_tokens // 64) * 64
+    if 64 % page_size == 0:
+        return rounded
+    return (-(-rounded // page_size) + max_requests) * page_size
+
+
 def main(argv=None) -> int:
     import argparse
     parser = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
@@ -98,21 +108,24 @@ def main(argv=None) -> int:
     parser.add_argument("--out", required=True, help="folder for the <step>.f32 files")
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time (each rounded up to a page multiple)")
-    parser.add_argument("--page-size", type=int, default=64, help="tokens per cache page (a divisor of 64)")
+    parser.add_argument("--page-size", type=int, default=64,
+                        help="tokens per cache page: any size the engine takes (a multiple of 8)")
     parser.add_argument("--max-requests", type=int, default=8, help="most requests live at a time")
     parser.add_argument("--taps", action="store_true", help="also write every step's intermediates")
     parser.add_argument("--device", default="cuda", choices=["cuda", "cpu"],
                         help="cpu runs only with a stand-in for the HIP kernels named in SPARSEENGINE_AMD_KERNELS (tests)")
     args = parser.parse_args(argv)
-    if args.device == "cpu" and not os.environ.get("SPARSEENGINE_AMD_KERNELS"):
-        parser.error("--device cpu needs SPARSEENGINE_AMD_KERNELS=module:factory (a test seam); the engine's "
-                     "own kernels run on the GPU only")
-    if args.page_size <= 0 or 64 % args.page_size:
-        parser.error("--page-size must divide 64")
+    try:
+        kernels, device = kernels_for_program(args.device)
+    except ValueError as exc:
+        parser.error(str(exc))
+    if args.page_size <= 0 or args.page_size % 8:
+        parser.error("--page-size must be a positive multiple of 8")
     print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
     runner = ModelRunner.from_folder(
-        args.model, dtype=args.dtype, device=args.device, kv_page_size=args.page_size,
-        num_kvcache_tokens=-(-args.max_tokens // 64) * 64, max_num_seqs=args.max_requests)
+        args.model, dtype=args.dtype, device=device, kernels=kernels, kv_page_size=args.page_size,
+        num_kvcache_tokens=pool_tokens(args.max_tokens, args.page_size, args.max_requests),
+        max_num_seqs=args.max_requests)
     print("[trace_run] ready", file=sys.stderr, flush=True)
     replay_stream(runner, sys.stdin, args.out, with_taps=args.taps)
     return 0

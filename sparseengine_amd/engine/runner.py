@@ -37,18 +37,28 @@ def require_true_float32() -> None:
     torch.set_float32_matmul_precision("highest")
 
 
-def kernels_from_environment():
-    """Test seam for the programs (``bin/trace_run``, the command line), which build their engine
-    themselves: ``SPARSEENGINE_AMD_KERNELS=module:factory`` names a stand-in for the HIP kernels that
-    works on CPU tensors (the tests' twins, or their host build of the kernel sources).  Unset,
-    as in every product run, the HIP kernels are the only path."""
+def kernels_for_program(device: str):
+    """What the programs (``bin/trace_run``, the command line) hand to the engine they build: ``(kernels,
+    device)``.  ``cuda``: ``(None, "cuda")``, the HIP kernels, the only path of the product.  ``cpu`` is a test
+    seam of the programs alone: ``SPARSEENGINE_AMD_KERNELS=module:factory`` must then name a stand-in for the
+    HIP kernels that works on CPU tensors (the tests' twins, or their host build of the kernel sources); it is
+    said so on stderr.  The variable without ``cpu`` is refused, and neither ``ModelRunner`` nor ``LLM`` looks
+    at the environment."""
     import importlib
     import os
+    import sys
     seam = os.environ.get("SPARSEENGINE_AMD_KERNELS")
+    if device != "cpu":
+        if seam:
+            raise ValueError("SPARSEENGINE_AMD_KERNELS is set, but the device asked for is not cpu: the variable "
+                             "replaces the kernels by a stand-in on the CPU (a test seam); unset it")
+        return None, device
     if not seam:
-        return None
+        raise ValueError("device cpu needs SPARSEENGINE_AMD_KERNELS=module:factory (a test seam); the engine's "
+                         "own kernels run on the GPU only")
     module, _, factory = seam.partition(":")
-    return getattr(importlib.import_module(module), factory)()
+    print(f"[sparseengine_amd] test seam: the kernels are replaced by {seam} on the CPU", file=sys.stderr, flush=True)
+    return getattr(importlib.import_module(module), factory)(), "cpu"
 
 
 @dataclass
@@ -61,15 +71,16 @@ class StepEntry:
 class ModelRunner:
     def __init__(self, arch: Architecture, cfg, params_factory, *, dtype, device="cuda", kv_page_size=64,
                  num_kvcache_tokens: int | None = None, max_num_seqs: int = 8, max_model_len: int | None = None,
-                 mlp_chunk_size: int = 16384, kernels=None, gpu_memory_utilization: float = 0.9, method=None):
+                 mlp_chunk_size: int = 16384, kernels=None, gpu_memory_utilization: float = 0.9, method=None,
+                 cache_manager_cls=None, validate_runtime_invariants: bool = False):
+        """``method`` / ``cache_manager_cls``: the sparse method's runtime and the class of its cache manager
+        (config/method_registry.py); absent: the dense method on the paged cache manager.
+        ``validate_runtime_invariants``: before every attention launch the host checks that each block-table
+        entry the launch will read names a page of the pool."""
         self.arch, self.model_config = arch, cfg
         self.dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
         require_true_float32()
-        if kernels is None:
-            kernels = kernels_from_environment()
-            if kernels is not None:
-                self.device = torch.device("cpu")
         if kernels is None:
             from ..kernels.hip_ops import HipKernels      # raises if there is no GPU or no library
             kernels = HipKernels()
@@ -93,7 +104,7 @@ class ModelRunner:
         if num_kvcache_tokens is None or int(num_kvcache_tokens) <= 0:
             num_kvcache_tokens = self.derive_cache_tokens(requests, max_num_seqs, gpu_memory_utilization)
         num_pages = max(1, -(-int(num_kvcache_tokens) // self.kv_page_size))      # a last page may be partly beyond the count
-        self.cache = CacheManager(requests, max_rows=max_num_seqs,
+        self.cache = (cache_manager_cls or CacheManager)(requests, max_rows=max_num_seqs,
                                   max_model_len=self.max_model_len, page_size=self.kv_page_size,
                                   num_pages=num_pages, dtype=self.dtype, device=self.device)
         shapes = {}
@@ -109,6 +120,7 @@ class ModelRunner:
             method = PassThroughMethod()
         self.method = method
         method.bind(self.cache)
+        self.validate_runtime_invariants = bool(validate_runtime_invariants)
 
     def derive_cache_tokens(self, requests, max_num_seqs: int, utilization: float) -> int:
         """Tokens of cache that fit the memory left after the weights: ``utilization`` of the card
@@ -203,6 +215,7 @@ class ModelRunner:
         fb.taps = taps
         fb.forced_routing = forced_routing      # measurement and test seam (parts/feed_forward.py: _force)
         fb.method = self.method
+        fb.check_tables = self.validate_runtime_invariants
         self.method.prepare_step(fb)
         logits = self.model.forward(fb)
         self.method.finish_step(fb)

@@ -66,6 +66,8 @@ class GQAAttention(Part):
         q = qkv[:, :self.q_width].view(T, s.num_heads, s.head_dim)
         method = getattr(fb, "method", None)
         visible = meta if method is None else method.select(cache_position, meta)     # what this layer may read
+        if getattr(fb, "check_tables", False):
+            fb.check_block_table(visible, s.window or 0, cache.shape[0], f"schedule position {cache_position}")
         fb.kernels.paged_attention(q, cache, visible, attended, s.scale, s.window or 0)
         if method is not None:
             method.after_attention(cache_position, fb)

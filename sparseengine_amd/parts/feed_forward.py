@@ -18,6 +18,20 @@ from .linear import linear
 ACTIVATIONS = ("silu", "gelu_tanh")      # what the kernels' epilogues can apply to a gate
 
 
+def forced_experts(fb):
+    """Measurement and test seam, kept in this one place: ``fb.forced_routing`` holds, by schedule position
+    (a list, or a dict that names some positions), the experts ``[T, top_k]`` that every token of the step
+    is to take at that position's routed feed-forward; ``fb.schedule_position`` is the position that runs.
+    Nothing in the product sets it."""
+    given = getattr(fb, "forced_routing", None)
+    if given is None:
+        return None
+    position = getattr(fb, "schedule_position", 0)
+    if isinstance(given, dict):
+        return given.get(position)
+    return given[position] if position < len(given) else None
+
+
 class RoutedExperts(Part):
     kernel_libraries = ("moe", "moe_mfma")
 
@@ -51,35 +65,27 @@ class RoutedExperts(Part):
             self._tiled = bool(arrange(self.params["w13"], self.params["w2"]))
 
     def _workspace_for(self, fb, tokens: int, dtype):
+        """The scratch tensors of the expert pipeline: the kernels object makes them (their shape is its
+        kernels' business); they are kept with the step's other scratch and made anew when they do not fit."""
         s = self.spec
         ws = fb.scratch.tensors.get("moe.workspace")
         if ws is None or not ws.fits(tokens, s.top_k, s.num_experts, self.hidden_size, s.intermediate_size, dtype):
-            from ..kernels.hip_ops import MoeWorkspace
-            factory = getattr(fb.kernels, "make_moe_workspace", None) or MoeWorkspace
-            ws = factory(max(tokens, 1), s.top_k, s.num_experts, self.hidden_size, s.intermediate_size,
-                         dtype, fb.device)
+            ws = fb.kernels.make_moe_workspace(max(tokens, 1), s.top_k, s.num_experts, self.hidden_size,
+                                               s.intermediate_size, dtype, fb.device)
             fb.scratch.tensors["moe.workspace"] = ws
         return ws
 
     can_defer_slot_sum = True
-    DEFER_SLOT_SUM_TOKENS = 64
 
     def forward(self, fb, x, defer_slot_sum: bool = False):
         """``defer_slot_sum``: the reader accepts a ``SlotSum``; it gets one when the step is a single
-        chunk, the kernels leave the sum to their caller and nobody taps the routing."""
+        chunk of no more tokens than the kernels object says the hand-over pays for
+        (``slot_sum_deferral_tokens``: 0 or absent, never)."""
         s, p, T = self.spec, self.params, x.shape[0]
         out = fb.buffer("ffn.out", (T, self.hidden_size))
-        forced = None
-        given = getattr(fb, "forced_routing", None)
-        if given is not None:       # measurement and test seam, see ``_force``
-            call = getattr(fb, "_routed_calls", 0)
-            fb._routed_calls = call + 1
-            forced = given[call] if call < len(given) else None
-        # Measured on MI355X at MiniMax-M2 sizes: the norm that adds the slots up saves a launch in a decode
-        # step (batch 8: 5.96 -> 5.93 ms) and loses against the two kernels from a few hundred tokens on
-        # (a 2048-token step: 17.6 -> 18.2 ms): so only steps of few tokens hand the slots on.
-        if (defer_slot_sum and T <= self.DEFER_SLOT_SUM_TOKENS and p["w13"].dtype == x.dtype
-                and getattr(fb.kernels, "supports_slot_sums", False)):
+        forced = forced_experts(fb)
+        if (defer_slot_sum and T <= int(getattr(fb.kernels, "slot_sum_deferral_tokens", 0))
+                and p["w13"].dtype == x.dtype):
             return SlotSum(self._forward_chunk(fb, x, out, forced, sum_slots=False), s.top_k)
         for start in range(0, T, self.chunk_tokens):
             stop = min(T, start + self.chunk_tokens)
@@ -87,8 +93,7 @@ class RoutedExperts(Part):
         return out
 
     def _force(self, logits, forced, ids, weights):
-        """Measurement and test seam (``fb.forced_routing``: per routed layer of the step the experts
-        ``[T, top_k]`` every token is to take, or None): the router's choice is replaced, the weights
+        """Measurement and test seam (``forced_experts``): the router's choice is replaced, the weights
         are the chosen experts' own scores as the router would have weighted them.  A run in reduced
         precision can so be compared with one in float32 expert for expert, and a benchmark can
         spread its tokens evenly over the experts; nothing in the product sets it."""

@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import ModelSpec
-from .base import BLOCKS, NORMS, ParamDecl, Part
+from .base import BLOCKS, NORMS, ParamDecl, Part, SlotSum
 from .linear import linear
 
 
@@ -67,17 +67,17 @@ class DecoderModel(Part):
         for position, entry in enumerate(spec.schedule):
             own = entry.cache_from is None
             layer = self.layers[entry.layer]
+            fb.schedule_position = position
             # the sum over a token's expert slots may be left to whoever reads the layer's result:
             # the next layer's first norm, or the final norm
             reader = self.final_norm if position == final else self.layers[spec.schedule[position + 1].layer]
-            if (fb.taps is None and getattr(layer, "can_defer_slot_sum", False)
-                    and getattr(reader, "accepts_slot_sum", False)):
+            if getattr(layer, "can_defer_slot_sum", False) and getattr(reader, "accepts_slot_sum", False):
                 x, residual = layer.forward(fb, x, residual, position if own else entry.cache_from, own,
                                             defer_slot_sum=True)
             else:
                 x, residual = layer.forward(fb, x, residual, position if own else entry.cache_from, own)
             if fb.taps is not None:
-                fb.taps.setdefault("layer_out", []).append((x.float() + residual.float()))
+                fb.taps.setdefault("layer_out", []).append(_stream_value(x, residual))
         wanted = fb.want_index.numel()
         if wanted == 0:
             return torch.empty(0, spec.vocab_size, dtype=torch.float32, device=fb.device)
@@ -86,6 +86,16 @@ class DecoderModel(Part):
         weight = (self.head or self.embed).params["weight"]
         logits = linear(last, weight, out=fb.buffer("model.logits", (wanted, spec.vocab_size)), kernels=fb.kernels)
         return logits.to(torch.float32, copy=True)      # the caller's own tensor, not the scratch buffer
+
+
+def _stream_value(x, residual) -> torch.Tensor:
+    """The residual stream after a layer, in float, for a tap: ``x + residual``, where ``x`` may still be
+    a token's slots waiting to be added up by the next norm (rounded to the storage type first, as that
+    norm does)."""
+    if isinstance(x, SlotSum):
+        tokens, hidden = x.shape
+        x = x.parts.view(tokens, x.slots, hidden).float().sum(1).to(x.parts.dtype)
+    return x.float() + residual.float()
 
 
 def build_model(spec: ModelSpec, chunk_tokens: int = 16384) -> DecoderModel:

@@ -77,8 +77,8 @@ def test_trace_run_program_on_the_emulated_kernels(tmp_path):
 
 @pytest.mark.parametrize("key,dtype", [("C_loud", "bfloat16"), ("A_loud", "float32")])
 def test_the_slot_sum_left_to_the_next_norm_changes_no_bit(tmp_path, key, dtype):
-    """Without taps the feed-forward hands its per-slot results on and the norm that reads them adds
-    them up (one launch fewer per layer); with taps the sum is a kernel of its own.  Same bits."""
+    """In steps of few tokens the feed-forward hands its per-slot results on and the norm that reads them
+    adds them up (one launch fewer per layer); otherwise the sum is a kernel of its own.  Same bits."""
     from sparseengine_amd.engine.replay import replay_step
     from sparseengine_amd.engine.runner import ModelRunner
     from sparseengine_amd.parts.base import SlotSum
@@ -87,13 +87,15 @@ def test_the_slot_sum_left_to_the_next_norm_changes_no_bit(tmp_path, key, dtype)
     seen = []
     with backends.use(backends.EmulatedBackend(guard="after")):
         outs = []
-        for taps in (None, {}):
+        for deferral_tokens in (64, 0):
+            options = backends.ACTIVE.runner_kwargs()
+            options["kernels"].slot_sum_deferral_tokens = deferral_tokens
             runner = ModelRunner.from_folder(folder, dtype=dtype, kv_page_size=16, num_kvcache_tokens=peak, max_num_seqs=4,
-                                             **backends.ACTIVE.runner_kwargs())
+                                             **options)
             norm = runner.model.final_norm
             rows = norm.forward_rows
             norm.forward_rows = lambda fb, x, *a, _rows=rows: (seen.append(isinstance(x, SlotSum)), _rows(fb, x, *a))[1]
-            outs.append([replay_step(runner, rec, None, taps=None if taps is None else {}) for rec in records])
+            outs.append([replay_step(runner, rec, None, taps={}) for rec in records])
     assert seen[0] is True and seen[-1] is False          # the first run deferred the sum, the second did not
     for a, b in zip(*outs):
         assert (a is None and b is None) or np.array_equal(a, b)

@@ -490,9 +490,23 @@ def test_a_second_sparse_method_gets_every_hook(model):
             calls.append(("extra", new_tokens))
             return {0: 0}
 
-    method_registry.register_method("counting", Counting, "all_chunked")
+    from sparseengine_amd.cache.manager import CacheManager
+
+    class CountingCache(CacheManager):
+        """The method's own cache manager: the paged one, counting what it is asked."""
+        appended = 0
+
+        def append(self, items):
+            CountingCache.appended += sum(n for _, n in items)
+            return super().append(items)
+
+    method_registry.register_method("counting", Counting, "all_chunked", cache_manager_cls=CountingCache)
     try:
+        assert method_registry.resolve_method("counting").cache_manager() is CountingCache
+        assert method_registry.resolve_method("vanilla").cache_manager() is CacheManager
         engine = llm(folder, sparse_method="counting")
+        assert type(engine.runner.cache) is CountingCache and engine.oracle.cache is engine.runner.cache
+        assert type(llm(folder).runner.cache) is CacheManager
         prompt = list(requests.values())[1][:17]
         out = engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True), use_tqdm=False)
         assert out[0]["token_ids"] == plain.greedy(prompt, 3)
@@ -503,10 +517,44 @@ def test_a_second_sparse_method_gets_every_hook(model):
         assert [c[1] for c in calls if c[0] == "select"] == list(range(layers)) * 3
         assert [c[1] for c in calls if c[0] == "after"] == list(range(layers)) * 3
         assert any(c[0] == "extra" for c in calls)
+        assert CountingCache.appended == len(prompt) + 2          # the prompt, then two fed-back tokens
         with pytest.raises(ValueError, match="counting"):
             llm(folder, sparse_method="counting", prefill_schedule_policy="something_else")
     finally:
         method_registry._METHODS.pop("counting", None)
+
+
+def test_block_table_entries_are_checked_before_a_launch(model):
+    """``validate_runtime_invariants``: before attention launches, every block-table entry the launch will
+    read must name a page of the pool.  Entries a window has given back (-1) lie before what is read and
+    pass; an entry inside the read range that is -1 or beyond the pool stops the step on the host, with
+    the item and the entry named."""
+    from types import SimpleNamespace
+    from sparseengine_amd.engine.batch import BlockTableError, check_block_table
+    table = np.array([[3, 5, 9, -1], [-1, -1, 2, 7]], dtype=np.int32)
+    meta = SimpleNamespace(block_table_host=table, page_size=16, item_q_len=np.array([4, 1]), item_ctx_len=np.array([40, 60]))
+    with pytest.raises(BlockTableError, match=r"item 1 .* entry 0 = -1"):
+        check_block_table(meta, 0, 10)                             # no window: item 1 reads its pages 0..3
+    check_block_table(meta, 24, 10)                                # window 24: item 1 reads keys 36..59, pages 2..3
+    with pytest.raises(BlockTableError, match=r"item 0 .* entry 2 = 9"):
+        check_block_table(meta, 0, 9)                              # page 9 of a pool of 9
+    meta.item_ctx_len = np.array([50, 60])
+    with pytest.raises(BlockTableError, match=r"item 0 .* entry 3 = -1"):
+        check_block_table(meta, 24, 10)                            # item 0 now reaches into its fourth page
+    meta.item_ctx_len = np.array([40, 70])
+    with pytest.raises(BlockTableError, match="4 columns"):
+        check_block_table(meta, 24, 10)
+    # in the engine: on for a whole generation, and a table corrupted behind the cache manager's back is caught
+    folder, requests, _, _ = model
+    engine = llm(folder, validate_runtime_invariants=True)
+    prompt = list(requests.values())[3][:40]
+    engine.generate([prompt], SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True), use_tqdm=False)
+    runner = engine.runner
+    assert runner.validate_runtime_invariants
+    runner.step([StepEntry("x", prompt[:20], [])])
+    runner.cache.groups[0].table[runner.cache.row_of("x"), 0] = -1
+    with pytest.raises(BlockTableError, match="entry 0 = -1"):
+        runner.step([StepEntry("x", prompt[20:22], [1])])
 
 
 def test_replay_writes_the_pages_each_request_held(model, tmp_path):
@@ -562,3 +610,17 @@ def test_trace_run_program_on_the_cpu(model, tmp_path):
     for rid in got:
         assert np.abs(got[rid] - expected[rid]).max() < 2e-5 * max(1.0, np.abs(expected[rid]).max())
     assert len(open(tmp_path / "out" / "pages.jsonl").readlines()) == len(records)
+    # the variable without --device cpu is refused: it never replaces the GPU's kernels quietly
+    on_gpu = [a for a in cmd if a not in ("--device", "cpu")]
+    refused = subprocess.run(on_gpu, input="", capture_output=True, text=True, env=env)
+    assert refused.returncode != 0 and "SPARSEENGINE_AMD_KERNELS is set" in refused.stderr
+    # every page size the engine takes, also one that does not divide 64 and one above it
+    for page_size in (48, 128):
+        out = tmp_path / f"out{page_size}"
+        other = [str(out) if a == str(tmp_path / "out") else a for a in cmd]
+        other[other.index("--page-size") + 1] = str(page_size)
+        proc = subprocess.run(other, input="".join(json.dumps(r) + "\n" for r in records), capture_output=True,
+                              text=True, env=env, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        for r in records:
+            assert np.abs(np.fromfile(out / f"{r['step']}.f32", dtype="<f4").reshape(-1, vocab) - logits[r["step"]]).max() < 2e-5

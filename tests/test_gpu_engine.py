@@ -17,9 +17,7 @@ from tests.plain.minimax_m2 import PlainMiniMaxM2
 pytestmark = pytest.mark.gpu
 
 
-def bound(dtype, ref):
-    scale = float(np.abs(ref).max())
-    return 2e-5 * max(scale, 1.0) if dtype == "float32" else 0.04 * scale
+from tests.test_gpu_replay import assert_close_to_plain, bound      # noqa: E402  (float32 bound; bfloat16: rounding noise only)
 
 
 def runner_for(folder, dtype, tokens=1024, page_size=16, rows=4):
@@ -62,8 +60,7 @@ def test_long_decoding_token_by_token(tmp_path, key, dtype):
     got, routing = replay_with_routing(runner, records)
     plain = PlainMiniMaxM2(folder)
     ref = plain.logits(tokens, forced_routing=routing["long"] if dtype == "bfloat16" else None).numpy()
-    err = np.abs(got["long"] - ref).max(-1)
-    assert err.max() <= bound(dtype, ref), f"first position over the bound: {int(np.argmax(err > bound(dtype, ref)))}"
+    assert_close_to_plain(dtype, got["long"], ref, f"{key}, {n} tokens one by one")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -79,7 +76,7 @@ def test_first_tokens_of_a_sequence(tmp_path, dtype):
     for i, (r, t) in enumerate(seqs.items()):
         forced = [ids[i:i + 1].cpu().long() for ids, _ in taps["router"]] if dtype == "bfloat16" else None
         ref = plain.logits(t[:1], forced_routing=forced).numpy()
-        assert np.abs(logits[i] - ref[0]).max() <= bound(dtype, ref)
+        assert_close_to_plain(dtype, logits[i:i + 1], ref, f"first token of {r}")
     taps = {}
     logits = runner.step([StepEntry(r, t[1:3], [0, 1]) for r, t in seqs.items()], taps=taps).cpu().numpy()
     if dtype == "float32":
@@ -183,6 +180,8 @@ def command_line_backend(monkeypatch):
     named through the environment, as for any other program."""
     if backends.ACTIVE.name == "emu":
         monkeypatch.setenv("SPARSEENGINE_AMD_KERNELS", "tests.emu.kernels:EmuKernels")
+        return ["--device", "cpu"]
+    return []
 
 
 def test_command_line_generates_what_the_entry_point_generates(tmp_path, capsys, command_line_backend):
@@ -200,7 +199,7 @@ def test_command_line_generates_what_the_entry_point_generates(tmp_path, capsys,
     capsys.readouterr()
     assert main(["generate", "--model", folder, "--prompt-ids", json.dumps(prompts[0]), "--prompt-ids", str(ids_file),
                  "--dtype", "float32", "--num-kvcache-slots", "512", "--kv-page-size", "16", "--temperature", "0.7",
-                 "--top-k", "20", "--max-tokens", "9", "--ignore-eos", "--seed", "5"]) == 0
+                 "--top-k", "20", "--max-tokens", "9", "--ignore-eos", "--seed", "5", *command_line_backend]) == 0
     lines = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
     assert [line["prompt"] for line in lines] == prompts
     assert [line["token_ids"] for line in lines] == [e["token_ids"] for e in expected]
@@ -213,7 +212,7 @@ def test_command_line_bench_runs_every_case_on_the_gpu(tmp_path, capsys, command
     capsys.readouterr()
     assert main(["bench", "--model_path", folder, "--lengths", "40,130", "--batch_sizes", "1,4", "--output_len", "6",
                  "--hyper_params", json.dumps({"kv_page_size": 16, "num_kvcache_slots": 2048,
-                                               "max_num_batched_tokens": 96})]) == 0
+                                               "max_num_batched_tokens": 96}), *command_line_backend]) == 0
     rows = [json.loads(line) for line in capsys.readouterr().out.splitlines() if line.startswith("{")]
     assert [(r["length"], r["batch_size"]) for r in rows] == [(40, 1), (40, 4), (130, 1), (130, 4)]
     for r in rows:
@@ -241,7 +240,7 @@ def test_weights_stored_in_32_bit_stay_so_under_bfloat16(tmp_path):
     records = traces.changing_portions({"r": tokens}, seed=3)
     got, routing = replay_with_routing(runner, records)
     ref = PlainMiniMaxM2(folder).logits(tokens, forced_routing=routing["r"]).numpy()
-    assert np.abs(got["r"] - ref).max() <= bound("bfloat16", ref)
+    assert_close_to_plain("bfloat16", got["r"], ref, "weights kept in float32")
 
 
 # ------------------------------------------------------------------ each part alone
@@ -436,8 +435,7 @@ def run_toy_architecture(tmp_path, dtype, lengths):
         if dtype == "bfloat16":   # a near-tie of a routed layer may tip in bfloat16: the plain run takes the engine's choices
             forced = {kind: [torch.cat(chunks) for chunks in layers] for kind, layers in chosen[rid].items()}
             ref = plain.logits(requests[rid], forced=forced).numpy()
-        err = np.abs(got[rid] - ref).max(-1)
-        assert err.max() <= bound(dtype, ref), f"{rid}: first position over the bound {int(np.argmax(err > bound(dtype, ref)))}"
+        assert_close_to_plain(dtype, got[rid], ref, f"toy architecture, request {rid}")
     assert all(g.pool.free_count == g.pool.num_pages for g in runner.cache.groups)
     windowed = runner.cache.groups[1]
     assert windowed.pool.num_pages >= 4      # and a window of 24 never held more than 4 pages of 16 per request

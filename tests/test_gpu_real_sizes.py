@@ -34,7 +34,7 @@ from tests.plain.minimax_m2 import PlainMiniMaxM2
 pytestmark = pytest.mark.gpu
 
 REAL = dict(
-    architectures=["MiniMaxM2ForCausalLM"], model_type="minimax_m2", num_hidden_layers=1, hidden_size=3072,
+    architectures=["MiniMaxM2ForCausalLM"], model_type="minimax_m2", num_hidden_layers=2, hidden_size=3072,
     num_attention_heads=48, num_key_value_heads=8, head_dim=128, rotary_dim=64, rope_theta=5000000.0,
     num_local_experts=256, num_experts_per_tok=8, intermediate_size=1536, vocab_size=2048, rms_norm_eps=1e-6,
     use_qk_norm=True, max_position_embeddings=1024, tie_word_embeddings=False)
@@ -84,53 +84,71 @@ def replay(runner, records, forced=None):
     return out, chosen
 
 
+def choices_by_request(records, chosen, requests):
+    """Per request and layer the experts chosen for each of its positions, from the per-step records."""
+    layers = len(next(iter(chosen.values())))
+    out = {rid: [[] for _ in range(layers)] for rid in requests}
+    for rec in records:
+        cursor = 0
+        for e in rec["entries"]:
+            n = len(e["tokens"])
+            for layer in range(layers):
+                out[e["id"]][layer].append(chosen[rec["step"]][layer][cursor:cursor + n])
+            cursor += n
+    return {rid: [torch.cat(parts).long() for parts in layers] for rid, layers in out.items()}
+
+
+def plain_with_choices(plain, tokens, choices, slack, what):
+    """The plain logits with the given experts, after checking that every choice is a top-k of the plain
+    selection scores up to ``slack`` (rounding may tip a near-tie among 256 experts; nothing else may)."""
+    log = {}
+    ref = plain.logits(tokens, forced_routing=choices, routing_log=log).cpu().numpy()
+    for layer, ids in enumerate(choices):
+        scores = log[layer]
+        kth = torch.topk(scores, ids.shape[1], dim=-1).values[:, -1:]
+        assert (scores.gather(1, ids) >= kth - slack).all(), f"{what}, layer {layer}: an expert below the top-{ids.shape[1]} was chosen"
+    return ref
+
+
+def assert_float32_meets_plain(got, ref, what):
+    err = np.abs(got - ref).max(-1)
+    bound = 2e-5 * max(1.0, float(np.abs(ref).max()))
+    assert err.max() <= bound, f"float32 engine against plain, {what}: error {err.max():.3g} at position {int(err.argmax())}, bound {bound:.3g}"
+
+
 def test_bfloat16_against_float32_at_real_layer_sizes():
     if backends.ACTIVE.name != "hip":
         pytest.skip("sizes of the full model: GPU only")
     torch.manual_seed(0)
     requests = {"a": random_tokens(5, 2048, 1), "b": random_tokens(130, 2048, 2), "c": random_tokens(700, 2048, 3)}
     full = engine("float32", 1024)
-    # float32 engine against the plain implementation (its own routing: both are float32)
     plain = plain_model()
+    # the float32 engine against the plain implementation, every request whole, with its own routing:
+    # both are float32, so a choice may differ from the plain one only where two scores agree to rounding
     whole = traces.whole(requests)
-    logits32, _ = replay(full, whole)
+    logits32, chosen32 = replay(full, whole)
     got32 = traces.gather(whole, logits32)
-    spread = {}
-    for rid in ("a", "b"):
-        ref = plain.logits(requests[rid]).cpu().numpy()
-        spread[rid] = float(ref.std())
-        err = np.abs(got32[rid] - ref).max()
-        assert err <= 2e-5 * max(1.0, float(np.abs(ref).max())), f"float32 engine against plain, request {rid}: {err}"
-    scores_of = {}
-    for rid in requests:       # the plain selection scores, to check the bfloat16 engine's choices against
-        log = {}
-        plain.logits(requests[rid], routing_log=log)
-        scores_of[rid] = log[0].cpu()
-    del plain
-    torch.cuda.empty_cache()
+    own = choices_by_request(whole, chosen32, requests)
+    for rid, tokens in requests.items():
+        assert_float32_meets_plain(got32[rid], plain_with_choices(plain, tokens, own[rid], 2e-5, f"float32, request {rid}"),
+                                   f"request {rid} whole")
 
     half = engine("bfloat16", 1024)
-    assert half.model.layers[0].ffn._tiled is True
+    assert all(layer.ffn._tiled is True for layer in half.model.layers)
     mixed, _ = traces.mixed(requests, seed=4)
     modes = {"whole": whole, "tail": traces.prefill_then_decode(requests, tail=32),
              "portions": traces.changing_portions(requests, seed=5), "mixed": mixed}
     for mode, records in modes.items():
         logits16, chosen = replay(half, records)
-        # every choice of the bfloat16 engine is a top-8 of the plain scores up to the slack
-        fed = {rid: 0 for rid in requests}
-        for rec in records:
-            cursor = 0
-            for e in rec["entries"]:
-                n = len(e["tokens"])
-                ids = chosen[rec["step"]][0][cursor:cursor + n].cpu().long()
-                scores = scores_of[e["id"]][fed[e["id"]]:fed[e["id"]] + n]
-                kth = torch.topk(scores, 8, dim=-1).values[:, -1:]
-                assert (scores.gather(1, ids) >= kth - ROUTING_SLACK).all(), f"{mode}: an expert far below the top-8 was chosen"
-                fed[e["id"]] += n
-                cursor += n
         reference, _ = replay(full, records, forced=chosen)
         got, ref = traces.gather(records, logits16), traces.gather(records, reference)
+        theirs = choices_by_request(records, chosen, requests)
         for rid in requests:
+            # the float32 engine, cut and batched this way and with the bfloat16 engine's choices, against the
+            # plain implementation with the same choices (each a top-8 of the plain scores up to the slack)
+            assert_float32_meets_plain(
+                ref[rid], plain_with_choices(plain, requests[rid], theirs[rid], ROUTING_SLACK, f"{mode}, request {rid}"),
+                f"{mode}, request {rid}")
             scale = float(ref[rid].std())
             err = np.abs(got[rid] - ref[rid])
             per_position = np.sqrt((err ** 2).mean(-1)) / scale

@@ -24,11 +24,50 @@ SHORT_LENGTHS = {"A": [5, 17, 64, 1, 100], "B": [1, 9, 65, 16, 130], "C": [3, 40
 
 
 def bound(dtype, ref):
-    """Largest allowed |engine - plain|.  float32: a few units of float rounding of the largest
-    logit.  bfloat16: activations are rounded to 8 bits of mantissa about thirty times on the way
-    to a logit; 4 % of the largest logit covers that and no more."""
-    scale = float(np.abs(ref).max())
-    return 2e-5 * max(scale, 1.0) if dtype == "float32" else 0.04 * scale
+    """Largest allowed |engine - plain| in float32: a few units of float rounding of the largest logit."""
+    assert dtype == "float32"
+    return 2e-5 * max(float(np.abs(ref).max()), 1.0)
+
+
+def assert_close_to_plain(dtype, got, ref, what):
+    """``got`` and ``ref``: ``[positions, vocab]`` of one request.  float32: within ``bound``; bfloat16: rounding
+    noise and nothing else (below)."""
+    assert got.shape == ref.shape, what
+    if dtype == "bfloat16":
+        return assert_bfloat16_rounding_only(got, ref, what)
+    err = np.abs(got - ref).max(axis=-1)
+    worst = int(err.argmax())
+    assert err[worst] <= bound(dtype, ref), (
+        f"{what}: first position over the bound {int(np.argmax(err > bound(dtype, ref)))}, worst position {worst}, "
+        f"error {err[worst]:.3g}, bound {bound(dtype, ref):.3g}")
+
+
+# bfloat16 against the plain implementation (float32, the engine's expert choices): what rounding looks like.
+# A bfloat16 rounding is off by 2^-9 / sqrt(3) = 0.11 % of the value (rms); about fifteen roundings per layer
+# lie between the embedding and a logit, so a logit is off by about 0.11 % * sqrt(15 * layers + 1) of the logits'
+# spread, the same at every position of a request (a little more where attention averages many rounded keys
+# and values), Gaussian over the vocabulary.  A wrong key, page or expert is neither: it moves the logits of
+# some positions by their whole spread.  So: (1) at every single position the rms error is at most RMS_BOUND of
+# the spread of that request's logits; (2) no single logit is further off than 6.5 times the request's rms
+# error (a Gaussian tail over the few hundred thousand logits of a request ends near 5) plus 1 % of its own size.
+RMS_BOUND = 0.015
+MEASURED = []      # (request length, largest per-position rms error / spread, largest error / rms): printed with -s
+
+
+def assert_bfloat16_rounding_only(got, ref, what):
+    scale = float(ref.std())
+    err = np.abs(got - ref)
+    per_position = np.sqrt((err ** 2).mean(-1)) / scale
+    rms = float(np.sqrt((err ** 2).mean()))
+    MEASURED.append((len(ref), float(per_position.max()), float(err.max() / max(rms, 1e-30))))
+    assert per_position.max() <= RMS_BOUND, (
+        f"{what}: rms error {per_position.max():.4f} of the spread at position {int(per_position.argmax())} "
+        f"(median over positions {float(np.median(per_position)):.4f})")
+    allowed = 6.5 * rms + 1e-2 * np.abs(ref)
+    worst = np.unravel_index(int((err - allowed).argmax()), err.shape)
+    assert (err <= allowed).all(), (
+        f"{what}: position {worst[0]}, token {worst[1]}: bfloat16 {got[worst]:.4f}, plain {ref[worst]:.4f}, "
+        f"rms error of the request {rms:.4f}, spread of the logits {scale:.3f}")
 
 
 @pytest.fixture(scope="module", params=["A_loud", "B_loud", "A", "B", "C_loud"])
@@ -54,13 +93,16 @@ def run_records(folder, dtype, records, max_tokens, page_size):
     from sparseengine_amd.engine.runner import ModelRunner
     runner = ModelRunner.from_folder(folder, dtype=dtype, kv_page_size=page_size,
                                      num_kvcache_tokens=-(-max_tokens // 64) * 64, max_num_seqs=4,
-                                     **backends.ACTIVE.runner_kwargs())
+                                     validate_runtime_invariants=True, **backends.ACTIVE.runner_kwargs())
     out, routing = {}, {}
     for rec in records:
-        taps = {}
+        taps = {} if dtype == "bfloat16" else None      # the experts chosen: only bfloat16 is compared through them
         logits = replay_step(runner, rec, None, taps=taps)
         if logits is not None:
             out[rec["step"]] = logits
+        if taps is None:
+            runner.cache.check_invariants()
+            continue
         cursor = 0
         for e in rec["entries"]:
             n = len(e["tokens"])
@@ -95,13 +137,10 @@ def compare(dtype, got, model, routing):
                 picked = scores.gather(1, chosen.long())
                 assert (picked >= kth - ROUTING_SLACK).all(), f"{rid} layer {layer}: an expert far below the top-{k} was chosen"
                 assert sorted(set(map(int, chosen[0]))) == sorted(map(int, chosen[0])) and chosen.shape[0] == len(toks)
-        assert got[rid].shape == ref.shape, rid
-        err = np.abs(got[rid] - ref).max(axis=-1)
-        worst = int(err.argmax())
-        assert err[worst] <= bound(dtype, ref), (
-            f"request {rid} (length {len(ref)}): first position over the bound "
-            f"{int(np.argmax(err > bound(dtype, ref)))}, worst position {worst}, error {err[worst]:.3g}, "
-            f"bound {bound(dtype, ref):.3g}")
+        assert_close_to_plain(dtype, got[rid], ref, f"request {rid} (length {len(ref)})")
+    if dtype == "bfloat16" and MEASURED:
+        print(f"[bfloat16 against plain] {len(MEASURED)} requests so far: largest per-position rms error "
+              f"{max(m[1] for m in MEASURED):.4f} of the spread, largest single error {max(m[2] for m in MEASURED):.2f} rms")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -150,12 +189,13 @@ def test_trace_run_program(model, dtype, tmp_path):
     folder, requests, expected, plain = model
     records, peak = traces.mixed(requests, seed=3)
     out_dir = tmp_path / "out"
-    env = dict(os.environ)
+    env, on_cpu = dict(os.environ), []
     if backends.ACTIVE.name == "emu":      # the program builds its engine itself: name the kernels' stand-in
         env.update(SPARSEENGINE_AMD_KERNELS="tests.emu.kernels:EmulatedProgramKernels", PYTHONPATH=ROOT)
+        on_cpu = ["--device", "cpu"]
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-         "--out", str(out_dir), "--max-tokens", str(peak), "--page-size", "16"],
+         "--out", str(out_dir), "--max-tokens", str(peak), "--page-size", "16", *on_cpu],
         input="".join(json.dumps(r) + "\n" for r in records), capture_output=True, text=True, timeout=1800, env=env)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {r['step']}" for r in records]
@@ -169,7 +209,7 @@ def test_trace_run_program(model, dtype, tmp_path):
         other = tmp_path / "out_module"
         proc = subprocess.run(
             [sys.executable, "-m", "sparseengine_amd", "replay", "--model", folder, "--dtype", dtype, "--out", str(other),
-             "--max-tokens", str(peak), "--page-size", "16"], cwd=ROOT,
+             "--max-tokens", str(peak), "--page-size", "16", *on_cpu], cwd=ROOT,
             input="".join(json.dumps(r) + "\n" for r in records[:6]), capture_output=True, text=True, timeout=1800,
             env=env)
         assert proc.returncode == 0, proc.stderr[-2000:]

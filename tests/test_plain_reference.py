@@ -167,3 +167,97 @@ def test_float64_agrees(model_a, tmp_path):
     m64 = plain.PlainMiniMaxM2(make_folder(tmp_path, "A_loud"), dtype=torch.float64)
     toks = random_tokens(25, 512, 5)
     assert (m64.logits(toks).float() - model_a.logits(toks)).abs().max() < 5e-5
+
+
+def one_layer_model(tmp_path, zero=()):
+    """Configuration A cut to one layer, loud weights; tensors whose names end in one of ``zero`` are zeroed."""
+    from sparseengine_amd.weights.random_weights import write_model_folder
+    raw, options, seed = CONFIGS["A_loud"]
+    folder = write_model_folder(str(tmp_path / "one_layer"), dict(raw, num_hidden_layers=1), seed, options)
+    m = plain.PlainMiniMaxM2(folder)
+    for name in m.w:
+        if name.endswith(tuple(zero)):
+            m.w[name] = torch.zeros_like(m.w[name])
+    return m
+
+
+def test_qk_norm_comes_before_the_rotation(tmp_path):
+    """The reference's own statement of the order (tests/test_minimax_m2_model.py:357-417): the rotated
+    dims of what attention receives are the rotation of the *normed* row, the other dims are the
+    normed row bit for bit.  With a norm weight that differs from dim to dim the other order
+    (rotate, then norm) gives other numbers; the test says by how much."""
+    m = one_layer_model(tmp_path)
+    c, p = m.cfg, "model.layers.0.self_attn."
+    H, Hkv, D, R = c.num_attention_heads, c.num_key_value_heads, c.head_dim, c.rotary_dim
+    assert H * D == c.hidden_size          # so that an identity projection makes q the input row itself
+    eye = torch.eye(c.hidden_size)
+    m.w[p + "q_proj.weight"], m.w[p + "k_proj.weight"], m.w[p + "v_proj.weight"] = eye, eye[:Hkv * D], eye[Hkv * D:2 * Hkv * D]
+    torch.manual_seed(3)
+    m.w[p + "q_norm.weight"] = torch.linspace(0.2, 3.0, H * D)[torch.randperm(H * D)]      # strongly non-uniform
+    m.w[p + "k_norm.weight"] = torch.linspace(3.0, 0.2, Hkv * D)
+    u = torch.randn(3, c.hidden_size)
+    u[:, :D] *= 0.1
+    u[:, D:2 * D] *= 10.0
+    positions = torch.tensor([0, 1, 17])
+    q, k, v = m.attention_inputs(0, u, positions)
+    normed_q = F.rms_norm(u, (H * D,), m.w[p + "q_norm.weight"], c.rms_norm_eps).view(3, H, D)
+    normed_k = F.rms_norm(u[:, :Hkv * D], (Hkv * D,), m.w[p + "k_norm.weight"], c.rms_norm_eps).view(3, Hkv, D)
+    assert torch.equal(v, u[:, Hkv * D:2 * Hkv * D].view(3, Hkv, D))                      # values: neither normed nor turned
+    # the angle written out: p * theta^(-2d/R), pairs (d, d + R/2)
+    d = torch.arange(R // 2, dtype=torch.float64)
+    angle = positions.double()[:, None] * c.rope_theta ** (-2 * d / R)
+    cos, sin = angle.cos().float()[:, None, :], angle.sin().float()[:, None, :]
+    for got, normed in ((q, normed_q), (k, normed_k)):
+        assert torch.equal(got[..., R:], normed[..., R:])                                 # pass-through dims: the normed row itself
+        lo, hi = normed[..., :R // 2], normed[..., R // 2:R]
+        torch.testing.assert_close(got[..., :R // 2], lo * cos - hi * sin, atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(got[..., R // 2:R], hi * cos + lo * sin, atol=1e-5, rtol=1e-5)
+    # the other order: rotate the raw row, then norm it
+    raw_cos, raw_sin = plain.rope_angles(positions, R, c.rope_theta)
+    swapped = plain.flat_qk_norm(plain.partial_rope(u.view(3, H, D), raw_cos, raw_sin, R).reshape(3, -1),
+                                 m.w[p + "q_norm.weight"], c.rms_norm_eps).view(3, H, D)
+    assert torch.equal(swapped[0], q[0])                                                   # position 0 turns nothing
+    assert (swapped[1:, :, :R] - q[1:, :, :R]).abs().max() > 0.1
+
+
+def hand_written_layer(m, toks, attention=True, experts=True):
+    """One pre-norm layer and the head with library norms, written out: ``r = e (+ a)``;
+    ``y = norm_f(r (+ moe(norm_post(r))))`` (models/minimax_m2.py:381-397, models/qwen3.py:291-325)."""
+    c, w = m.cfg, m.w
+    n = lambda z, name: F.rms_norm(z, (c.hidden_size,), w[name], c.rms_norm_eps)
+    e = w["model.embed_tokens.weight"][toks]
+    positions = torch.arange(len(toks))
+    r = e
+    if attention:
+        r = e + m.attention(0, n(e, "model.layers.0.input_layernorm.weight"), positions)
+    out = r
+    if experts:
+        out = r + m.moe(0, n(r, "model.layers.0.post_attention_layernorm.weight"))
+    return n(out, "model.norm.weight") @ w["lm_head.weight"].T
+
+
+def test_the_residual_inside_a_layer(tmp_path):
+    """What only one of the two zeroed projections shows: the mixer's result is added to the residual
+    before the second norm, that norm reads the sum (not the mixer's result alone: with the output
+    projection zeroed that would norm a zero row and the experts would add nothing), and the final norm
+    reads the experts' result plus that same sum."""
+    toks = random_tokens(9, 512, 6)
+    only_attention = one_layer_model(tmp_path, zero=(".w2.weight",))
+    torch.testing.assert_close(only_attention.logits(toks), hand_written_layer(only_attention, toks, experts=False))
+    only_experts = one_layer_model(tmp_path, zero=("o_proj.weight",))
+    expect = hand_written_layer(only_experts, toks, attention=False)
+    torch.testing.assert_close(only_experts.logits(toks), expect)
+    bare = one_layer_model(tmp_path, zero=("o_proj.weight", ".w2.weight"))
+    assert (expect - bare.logits(toks)).abs().max() > 1e-2          # the experts did add something
+    both = one_layer_model(tmp_path)
+    full = hand_written_layer(both, toks)
+    torch.testing.assert_close(both.logits(toks), full)
+    # the second norm reading the mixer's result alone would give other logits
+    c, w = both.cfg, both.w
+    e = w["model.embed_tokens.weight"][toks]
+    a = both.attention(0, F.rms_norm(e, (c.hidden_size,), w["model.layers.0.input_layernorm.weight"], c.rms_norm_eps),
+                       torch.arange(len(toks)))
+    wrong = F.rms_norm(e + a + both.moe(0, F.rms_norm(a, (c.hidden_size,), w["model.layers.0.post_attention_layernorm.weight"],
+                                                       c.rms_norm_eps)),
+                       (c.hidden_size,), w["model.norm.weight"], c.rms_norm_eps) @ w["lm_head.weight"].T
+    assert (wrong - full).abs().max() > 1e-2

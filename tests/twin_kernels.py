@@ -33,7 +33,7 @@ class TwinKernels:
     def embedding(self, ids, table, out):
         out.copy_(table[ids.long()])        # a float table under bfloat16 activations is rounded here
 
-    supports_slot_sums = True
+    slot_sum_deferral_tokens = 64
 
     def rms_norm(self, x, weight, eps, out, residual=None, rows=None, write_residual=True, slots=1):
         z = x.float()
