@@ -12,7 +12,9 @@ the mean number of experts per layer that its tokens chose); ``points`` holds de
 64 and the prefill of eight 2048-token prompts in one step; ``roofline`` prices the batch-8 decode
 step against 8 TB/s and ``point_rooflines`` the other decode points the same way (every weight the
 step uses once - the experts it touched are counted from the step's own routing - and the cache of
-the live requests).  With random weights the tokens of a prompt agree on a few dozen experts past
+the live requests).  ``roofline.measured_peak`` is what a kernel of this engine that does nothing but read 8 GiB
+reaches on this box at the start of the run (``memory`` holds that and the rate of a copy), and ``measured_frac`` /
+``point_rooflines_measured`` price the same steps against it.  With random weights the tokens of a prompt agree on a few dozen experts past
 the first layer, which makes a prompt cheaper than real weights would: ``prefill_uniform`` is the
 same step with every token sent to eight experts drawn evenly from all 256 (the routing is replaced
 after the router has run, so the router's own work is still in the time).  ``kernels`` holds, for the prefill
@@ -95,6 +97,12 @@ def main() -> int:
     from sparseengine_amd.sampling.sampler import Sampler
 
     cfg = dict(MODEL, num_hidden_layers=args.layers)
+    from sparseengine_amd.kernels.hip_ops import HipKernels
+    memory = HipKernels().measure_memory(gib=8.0)       # before the model is there: what this box's memory delivers
+    torch.cuda.empty_cache()
+    measured_peak = memory["read_GBps"] * 1e9
+    print(f"[bench] memory: a kernel that only reads 8 GiB {memory['read_GBps']:.0f} GB/s, a copy "
+          f"{memory['copy_GBps']:.0f} GB/s (read + written)", file=sys.stderr, flush=True)
     t0 = time.time()
     runner = ModelRunner.from_random(
         cfg, seed=0, options=dict(std=0.02, norm_std=0.1, bias_std=0.01), on_device=True, dtype=args.dtype,
@@ -254,12 +262,13 @@ def main() -> int:
     kernels[f"decode_b{args.batch}"] = decode_calls(args.batch, distinct, context, calls)
     print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.2f} ms/step, {sum(distinct) / len(distinct):.0f} experts touched "
           f"per layer, {decode_bytes(args.batch, distinct, context) / step_s / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
-    points, point_rooflines = {}, {}
+    points, point_rooflines, point_rooflines_measured = {}, {}, {}
     for b in [int(x) for x in args.points.split(",") if x]:
         s, d, c, calls = decode(b, max(8, args.steps // 2), max(2, args.warmup // 2), f"b{b}_")
         kernels[f"decode_b{b}"] = decode_calls(b, d, c, calls)
         points[f"decode_b{b}"] = round(b / s, 1)
         point_rooflines[f"decode_b{b}"] = round(decode_bytes(b, d, c) / s / HBM_PEAK, 4)
+        point_rooflines_measured[f"decode_b{b}"] = round(decode_bytes(b, d, c) / s / measured_peak, 4)
         print(f"[bench] decode batch {b}: {s * 1e3:.2f} ms/step, {sum(d) / len(d):.0f} experts touched per layer, "
               f"{decode_bytes(b, d, c) / s / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
 
@@ -281,16 +290,22 @@ def main() -> int:
                     "frac": round(prefill_flops / prefill_s / peak, 5),
                     # a 2048-token step reads every expert it touches for a few dozen rows each: memory bound too
                     "hbm_frac": None if prefill_bytes is None else round(prefill_bytes / prefill_s / HBM_PEAK, 4),
+                    "hbm_measured_frac": None if prefill_bytes is None else round(prefill_bytes / prefill_s / measured_peak, 4),
                     "flops": prefill_flops, "bytes": prefill_bytes,
                     "experts_touched": None if touched is None else round(sum(touched) / len(touched), 1)},
         "prefill_uniform": None if uniform_s is None else {
             "value": round(T / uniform_s, 1), "tokens": T, "ms": round(uniform_s * 1e3, 3),
             "frac": round(prefill_flops / uniform_s / peak, 5), "hbm_frac": round(uniform_bytes / uniform_s / HBM_PEAK, 4),
+            "hbm_measured_frac": round(uniform_bytes / uniform_s / measured_peak, 4),
             "bytes": uniform_bytes, "experts_touched": min(E, T * K)},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4)},
+                     "frac": round(achieved / HBM_PEAK, 4), "measured_peak": round(measured_peak / 1e9, 1),
+                     "measured_frac": round(achieved / measured_peak, 4)},
+        # a kernel that only reads / a kernel that copies 8 GiB, timed at the start of this run
+        "memory": memory,
         "points": points,
         "point_rooflines": point_rooflines,
+        "point_rooflines_measured": point_rooflines_measured,
         # per call of the kernels object, from one step with events around each: what the step's time goes to
         "kernels": kernels,
     }

@@ -113,6 +113,10 @@ _SIGNATURES = {
         "se_grouped_gemm_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
+    "memory_probe": {
+        "se_stream_read": [c_void_p, c_int64, c_void_p, c_int, c_void_p],
+        "se_stream_copy": [c_void_p, c_void_p, c_int64, c_int, c_void_p],
+    },
     "sampling": {
         "se_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
@@ -178,7 +182,7 @@ class HipKernels:
     """The kernel interface of the engine, served by the gfx950 libraries."""
 
     libraries = ("norm", "rope_kv", "attention_generic", "attention_mfma", "moe", "moe_mfma", "sampling",
-                 "host_work")
+                 "host_work", "memory_probe")
 
     def __init__(self):
         if not torch.cuda.is_available():
@@ -669,3 +673,54 @@ class HipKernels:
             _ptr(logits), logits.stride(0), rows, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
             _ptr(seeds), _ptr(self._sample_partials[0]), _ptr(self._sample_partials[1]), _ptr(filters[0]),
             _ptr(filters[1]), _ptr(out), _stream()), "sample")
+
+    # ------------------------------------------------------------------ what the memory delivers
+    PROBE_BLOCKS = 4096     # 16 blocks of 256 threads per CU, each thread with eight 16-byte loads in flight
+
+    def stream_read(self, src: torch.Tensor, sink: torch.Tensor | None = None) -> torch.Tensor:
+        """Read every byte of ``src`` once and nothing else: the kernel the weight-streaming kernels are
+        priced against.  ``sink`` (int32, one word per block) takes the exclusive-or of what each block read."""
+        _require(src.is_contiguous() and src.data_ptr() % 16 == 0 and (src.numel() * src.element_size()) % 16 == 0,
+                 "stream_read: a contiguous tensor of a multiple of 16 bytes")
+        if sink is None:
+            sink = torch.empty(self.PROBE_BLOCKS, dtype=torch.int32, device=src.device)
+        _i32(sink, "sink")
+        _check(_fn.get("memory_probe", "se_stream_read")(_ptr(src), src.numel() * src.element_size(), _ptr(sink),
+                                                         sink.numel(), _stream()), "stream_read")
+        return sink
+
+    def stream_copy(self, src: torch.Tensor, dst: torch.Tensor) -> torch.Tensor:
+        _require(src.is_contiguous() and dst.is_contiguous() and src.dtype == dst.dtype and src.shape == dst.shape
+                 and src.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0
+                 and (src.numel() * src.element_size()) % 16 == 0, "stream_copy: two contiguous tensors of one shape, 16-byte multiples")
+        _check(_fn.get("memory_probe", "se_stream_copy")(_ptr(src), _ptr(dst), src.numel() * src.element_size(),
+                                                         self.PROBE_BLOCKS, _stream()), "stream_copy")
+        return dst
+
+    def measure_memory(self, gib: float = 8.0, repeats: int = 5, device="cuda") -> dict:
+        """Bytes per second of a kernel that only reads ``gib`` GiB (far beyond the caches) and of one that copies
+        them (bytes read plus bytes written): the best of ``repeats`` runs each, after one untimed run."""
+        words = int(gib * 2 ** 30) // 16
+        src = torch.empty(words * 4, dtype=torch.int32, device=device).random_()
+        sink = torch.empty(self.PROBE_BLOCKS, dtype=torch.int32, device=device)
+        size = src.numel() * 4
+
+        def best(run):
+            run()
+            rates = []
+            for _ in range(repeats):
+                first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                first.record()
+                run()
+                last.record()
+                last.synchronize()
+                rates.append(first.elapsed_time(last) * 1e-3)
+            return min(rates)
+
+        read_s = best(lambda: self.stream_read(src, sink))
+        dst = torch.empty_like(src)
+        copy_s = best(lambda: self.stream_copy(src, dst))
+        library_copy_s = best(lambda: dst.copy_(src))
+        del src, dst
+        return {"bytes": size, "read_GBps": round(size / read_s / 1e9, 1), "copy_GBps": round(2 * size / copy_s / 1e9, 1),
+                "library_copy_GBps": round(2 * size / library_copy_s / 1e9, 1)}

@@ -1029,3 +1029,23 @@ def test_experts_on_random_shapes_and_lumpy_routing(hip, twin):
             hip.moe_experts(x, a13, a2, ids, weights, out, ws, kernel=kernel, tile_rows=rows, tiled=True)
             torch.testing.assert_close(out, ref, **tol(dtype), msg=lambda m: (
                 f"case {case}: {tokens} tokens, {experts} experts, top {k}, hidden {hidden}, width {inter}, kernel {kernel}: {m}"))
+
+
+def test_memory_probe_reads_and_copies_every_byte(hip):
+    """The kernels the benchmarks price memory with: the read kernel's per-block words fold to the exclusive-or
+    of the whole buffer (so every 16 bytes were read exactly once), also with a tail that does not fill a
+    block's share; the copy kernel copies every byte."""
+    if backends.ACTIVE.name != "hip":
+        pytest.skip("a timing aid of the benchmarks: GPU only")
+    for words in (1, 256 * 8 * 3 + 5, 1 << 20):
+        src = torch.randint(-2 ** 31, 2 ** 31 - 1, (words * 4,), dtype=torch.int64).to(torch.int32).to(DEV)
+        sink = torch.zeros(7 if words < 100 else 333, dtype=torch.int32, device=DEV)
+        hip.stream_read(src, sink)
+        import numpy as np
+        assert (int(np.bitwise_xor.reduce(sink.cpu().numpy().view("uint32")))
+                == int(np.bitwise_xor.reduce(src.cpu().numpy().view("uint32"))))
+        dst = torch.zeros_like(src)
+        hip.stream_copy(src, dst)
+        assert torch.equal(src, dst)
+    with pytest.raises(ValueError):
+        hip.stream_read(torch.zeros(3, dtype=torch.int32, device=DEV))

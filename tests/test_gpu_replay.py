@@ -29,12 +29,12 @@ def bound(dtype, ref):
     return 2e-5 * max(float(np.abs(ref).max()), 1.0)
 
 
-def assert_close_to_plain(dtype, got, ref, what):
+def assert_close_to_plain(dtype, got, ref, what, independent=None):
     """``got`` and ``ref``: ``[positions, vocab]`` of one request.  float32: within ``bound``; bfloat16: rounding
     noise and nothing else (below)."""
     assert got.shape == ref.shape, what
     if dtype == "bfloat16":
-        return assert_bfloat16_rounding_only(got, ref, what)
+        return assert_bfloat16_rounding_only(got, ref, what, independent)
     err = np.abs(got - ref).max(axis=-1)
     worst = int(err.argmax())
     assert err[worst] <= bound(dtype, ref), (
@@ -48,26 +48,50 @@ def assert_close_to_plain(dtype, got, ref, what):
 # spread, the same at every position of a request (a little more where attention averages many rounded keys
 # and values), Gaussian over the vocabulary.  A wrong key, page or expert is neither: it moves the logits of
 # some positions by their whole spread.  So: (1) at every single position the rms error is at most RMS_BOUND of
-# the spread of that request's logits; (2) no single logit is further off than 6.5 times the request's rms
-# error (a Gaussian tail over the few hundred thousand logits of a request ends near 5) plus 1 % of its own size.
+# the spread of that request's logits; (2) no single logit is further off than 6.5 times its position's rms
+# error (a Gaussian tail over a vocabulary of a thousand ends near 4) plus 1 % of its own size.
+# Measured on MI355X over the five configurations and all ways of cutting: 0.5 to 1.2 % at all but one of about
+# 7000 positions.  The one (configuration A_loud, request r5, position 72: 4.1 %) is a place where this tiny
+# model with its loud weights amplifies rounding: an independent bfloat16 implementation (the tensor-library
+# twins of the kernels, on the CPU) is off by 4.3 % at that same position and by 0.6 to 0.9 % around it.  A
+# position above RMS_BOUND is therefore allowed only where that independent implementation is off by at least
+# half as much (``independent``).
 RMS_BOUND = 0.015
-MEASURED = []      # (request length, largest per-position rms error / spread, largest error / rms): printed with -s
+MEASURED = []      # (request length, largest per-position rms error / spread, largest error / position rms): printed with -s
 
 
-def assert_bfloat16_rounding_only(got, ref, what):
+def assert_bfloat16_rounding_only(got, ref, what, independent=None):
+    """``independent()``: the per-position rms error (in units of the spread) of another bfloat16
+    implementation on the same request, asked for only if a position is above ``RMS_BOUND``."""
     scale = float(ref.std())
     err = np.abs(got - ref)
-    per_position = np.sqrt((err ** 2).mean(-1)) / scale
-    rms = float(np.sqrt((err ** 2).mean()))
-    MEASURED.append((len(ref), float(per_position.max()), float(err.max() / max(rms, 1e-30))))
-    assert per_position.max() <= RMS_BOUND, (
-        f"{what}: rms error {per_position.max():.4f} of the spread at position {int(per_position.argmax())} "
-        f"(median over positions {float(np.median(per_position)):.4f})")
-    allowed = 6.5 * rms + 1e-2 * np.abs(ref)
+    position_rms = np.sqrt((err ** 2).mean(-1))
+    per_position = position_rms / scale
+    MEASURED.append((len(ref), float(per_position.max()), float((err / np.maximum(position_rms[:, None], 1e-30)).max())))
+    allowed_rms = np.full_like(per_position, RMS_BOUND)
+    if per_position.max() > RMS_BOUND and independent is not None:
+        allowed_rms = np.maximum(allowed_rms, 2.0 * independent())
+    over = per_position > allowed_rms
+    assert not over.any(), (
+        f"{what}: rms error {per_position[over].max():.4f} of the spread at position {int(np.argmax(over))} "
+        f"(allowed there {allowed_rms[int(np.argmax(over))]:.4f}, median over positions {float(np.median(per_position)):.4f})")
+    allowed = 6.5 * position_rms[:, None] + 1e-2 * np.abs(ref)
     worst = np.unravel_index(int((err - allowed).argmax()), err.shape)
     assert (err <= allowed).all(), (
         f"{what}: position {worst[0]}, token {worst[1]}: bfloat16 {got[worst]:.4f}, plain {ref[worst]:.4f}, "
-        f"rms error of the request {rms:.4f}, spread of the logits {scale:.3f}")
+        f"rms error of the position {position_rms[worst[0]]:.4f}, spread of the logits {scale:.3f}")
+
+
+def twin_bfloat16_error(folder, tokens, routing, ref):
+    """Per-position rms error (in units of the spread) of the kernels' tensor-library twins in bfloat16 on the
+    CPU, the request whole, with the same expert choices: an implementation that shares no kernel with the GPU's."""
+    from sparseengine_amd.engine.runner import ModelRunner, StepEntry
+    from tests.twin_kernels import TwinKernels
+    runner = ModelRunner.from_folder(folder, dtype="bfloat16", device="cpu", kernels=TwinKernels(), kv_page_size=16,
+                                     num_kvcache_tokens=-(-len(tokens) // 64) * 64, max_num_seqs=1)
+    logits = runner.step([StepEntry("twin", list(tokens), list(range(len(tokens))))],
+                         forced_routing=[r.to(torch.int32) for r in routing]).numpy()
+    return np.sqrt(((logits - ref) ** 2).mean(-1)) / float(ref.std())
 
 
 @pytest.fixture(scope="module", params=["A_loud", "B_loud", "A", "B", "C_loud"])
@@ -137,7 +161,8 @@ def compare(dtype, got, model, routing):
                 picked = scores.gather(1, chosen.long())
                 assert (picked >= kth - ROUTING_SLACK).all(), f"{rid} layer {layer}: an expert far below the top-{k} was chosen"
                 assert sorted(set(map(int, chosen[0]))) == sorted(map(int, chosen[0])) and chosen.shape[0] == len(toks)
-        assert_close_to_plain(dtype, got[rid], ref, f"request {rid} (length {len(ref)})")
+        assert_close_to_plain(dtype, got[rid], ref, f"request {rid} (length {len(ref)})",
+                              independent=lambda: twin_bfloat16_error(folder, toks, routing[rid], ref))
     if dtype == "bfloat16" and MEASURED:
         print(f"[bfloat16 against plain] {len(MEASURED)} requests so far: largest per-position rms error "
               f"{max(m[1] for m in MEASURED):.4f} of the spread, largest single error {max(m[2] for m in MEASURED):.2f} rms")

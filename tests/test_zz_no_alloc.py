@@ -31,12 +31,23 @@ def test_sampling_without_allocation_matches_the_entry_point_with_a_workspace():
         hip.sample(logits, temperature, None, None, seeds, expected)
         got = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
         torch.cuda.synchronize()
-        before = torch.cuda.memory_stats()["allocation.all.allocated"]
         status = fn(logits.data_ptr(), logits.stride(0), rows, vocab, temperature.data_ptr(), seeds.data_ptr(),
                     got.data_ptr(), stream)
         assert status == 0
         torch.cuda.synchronize()
-        assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+        assert torch.equal(got, expected)
+        # "allocates nothing": the device's own count of free bytes (which sees every hipMalloc, not only the
+        # tensor library's) and the tensor library's count are the same before and after a further call; the
+        # call above has asked for the array's address already, so this one is a call like every later one
+        got.fill_(-1)
+        torch.cuda.synchronize()
+        free_before, allocations_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_stats()["allocation.all.allocated"]
+        status = fn(logits.data_ptr(), logits.stride(0), rows, vocab, temperature.data_ptr(), seeds.data_ptr(),
+                    got.data_ptr(), stream)
+        assert status == 0
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == allocations_before
         assert torch.equal(got, expected)
         assert int(got[0]) == int(logits[0].argmax())
         # greedy, no temperature and no seeds
