@@ -35,6 +35,15 @@ class Architecture:
     random_tensor: Callable                              # (config, name, shape, generator, options) -> float32 tensor
     stored_dtype: Callable[[str], str]                   # tensor name -> "bfloat16" | "float32" as a checkpoint stores it
     config_to_dict: Callable[[Any], dict]
+    # (ModelSpec, chunk_tokens) -> the model: None builds ``parts.DecoderModel``; an architecture whose two
+    # ends differ from it (an embedding multiplier, a scale or cap on the logits) names a subclass here
+    model_factory: Callable | None = None
+
+    def make_model(self, spec: ModelSpec, chunk_tokens: int = 16384):
+        if self.model_factory is not None:
+            return self.model_factory(spec, chunk_tokens=chunk_tokens)
+        from ..parts import build_model
+        return build_model(spec, chunk_tokens=chunk_tokens)
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}

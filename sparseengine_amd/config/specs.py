@@ -98,6 +98,9 @@ class ModelSpec:
     final_norm: NormSpec
     max_position: int
     tie_word_embeddings: bool = False
+    # (name, value) pairs for an architecture's own model class (``Architecture.model_factory``): constants of
+    # the model's two ends that the generic decoder does not have (an embedding multiplier, a logit scale)
+    constants: tuple[tuple[str, float], ...] = ()
 
     def __post_init__(self):
         for pos, entry in enumerate(self.schedule):

@@ -149,7 +149,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
       const bf16_t* k_row = cache + (static_cast<int64_t>(PK) * 2) * plane + kvh * head_span +    \
                             (static_cast<int64_t>(g) * page_size + key % page_size) * 8;          \
       _Pragma("unroll") for (int ds = 0; ds < DSTEPS; ++ds)                                       \
-          KF[b][ds] = *reinterpret_cast<const uint4*>(k_row + static_cast<int64_t>(ds) * 32 * page_size); \
+          KF[b][ds] = load16_once(k_row + static_cast<int64_t>(ds) * 32 * page_size);             \
     }                                                                                             \
     int vkey = (K0) + 8 * g;                                                                      \
     if (vkey > last_key) vkey = last_key & ~7;                                                    \
@@ -158,7 +158,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* v_col = cache + (static_cast<int64_t>(PV) * 2 + 1) * plane + kvh * head_span +  \
                           static_cast<int64_t>(vkey % page_size) * D + n * 8;                     \
     _Pragma("unroll") for (int db = 0; db < DBLOCKS; ++db)                                        \
-        VF[db] = *reinterpret_cast<const uint4*>(v_col + db * 128);                               \
+        VF[db] = load16_once(v_col + db * 128);                                                   \
   }
 
 #define ATT_COMPUTE(KF, VF, K0)                                                                   \

@@ -14,12 +14,17 @@
 //   MODE 1 (down): in row = act[a]; w = w2[e], [N, K]; out[a, n] = (in . w[n]) * route_weight[a].
 //   MODE 2 (dense, few rows): out[t, n] = x[t] . w[n] for one weight matrix [N, K]; tile t holds rows
 //       16 * MB * t ...; the same streaming loop serves the skinny projections of decode steps.
+//   MODE 3: MODE 2 with the weight matrix in tiles, as the expert tables are (below).
 //
 // Expert tables (MODE 0 and 1, in all three kernels of this file) lie in tiles: tile
 // (n / 16, k / 32) of an expert is 512 consecutive elements in the order [(k % 32) / 8][n % 16][k % 8],
 // which is the order of the lanes that hold the tile as an A operand, so a wavefront's load of a
 // tile is one contiguous kilobyte (kernels/hip_ops.py: tile_expert_weights puts a table into this
-// order).  Dense tables (MODE 2) lie in rows: the BLAS library reads them too.
+// order).  Dense tables lie in rows (MODE 2), as the BLAS library reads them, or in a tiled copy made
+// for steps of few rows (MODE 3): a wavefront's load of 16 rows x 32 k of a table in rows is 64 bytes
+// from each of 16 rows, which arrive at a third of the rate of one contiguous kilobyte, and a block of
+// an output projection (16 rows x 6144) then takes 6 us for its loads alone; tiled loads also take the
+// read-once hint, which on half cache lines fetches every line twice.
 //
 // Every output element is one dot product in a fixed order of K, so a row's result does not
 // depend on its place in the tile or on what else is in the batch.
@@ -46,6 +51,14 @@ __device__ __forceinline__ bool xcd_work_item(int column_blocks, int num_tiles, 
   return true;
 }
 
+// A lane's 16 bytes of a weight tile: tiled tables are read once, in whole cache lines (load16_once);
+// a table in rows gives a lane half a cache line, whose other half the next step reads.
+template <bool TILED>
+__device__ __forceinline__ uint4 load_weights(const bf16_t* p) {
+  if constexpr (TILED) return load16_once(p);
+  return *reinterpret_cast<const uint4*>(p);
+}
+
 template <int MODE, int MB, int NB, int U, int KW = 4>   // KW wavefronts split K
 __global__ void __launch_bounds__(64 * KW)
 grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
@@ -58,7 +71,8 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   constexpr int BN = 16 * NB;
   constexpr int NBT = MODE == 0 ? 2 * NB : NB;  // weight blocks per wave: gate blocks, then up blocks
   int tile, column_block;
-  if (!xcd_work_item(N / BN, MODE == 2 ? max_tiles : counters[0], tile, column_block)) return;  // uniform
+  constexpr bool DENSE = MODE >= 2;
+  if (!xcd_work_item(N / BN, DENSE ? max_tiles : counters[0], tile, column_block)) return;  // uniform
 
   constexpr bool TILED = MODE != 2;
   constexpr int KSCALE = TILED ? 16 : 1;       // a step of 32 along k is 512 elements further in a tiled table
@@ -70,10 +84,10 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 
   const int lane = threadIdx.x & (SE_WAVE - 1);
   const int wave = threadIdx.x / SE_WAVE;
-  const int expert = MODE == 2 ? 0 : tile_expert[tile];
+  const int expert = DENSE ? 0 : tile_expert[tile];
   const int n0 = column_block * BN;
   if (threadIdx.x < BM)
-    rows[threadIdx.x] = MODE == 2 ? tile * BM + static_cast<int>(threadIdx.x) : sorted[tile * BM + threadIdx.x];
+    rows[threadIdx.x] = DENSE ? tile * BM + static_cast<int>(threadIdx.x) : sorted[tile * BM + threadIdx.x];
   __syncthreads();
 
   const int col = lane & 15;   // row of the weight block (A) / row of the activation block (B)
@@ -115,7 +129,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     for (int k = k_begin; k < k_end; k += 32) {
       uint4 af[NBT], bf[MB];
 #pragma unroll
-      for (int nb = 0; nb < NBT; ++nb) af[nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + static_cast<int64_t>(k) * KSCALE);
+      for (int nb = 0; nb < NBT; ++nb) af[nb] = load_weights<TILED>(a_ptr[nb] + static_cast<int64_t>(k) * KSCALE);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) bf[mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k);
 #pragma unroll
@@ -134,7 +148,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
     for (int u = 0; u < UU; ++u) {
 #pragma unroll
       for (int nb = 0; nb < NBT; ++nb)
-        af[u][nb] = *reinterpret_cast<const uint4*>(a_ptr[nb] + static_cast<int64_t>(k + 32 * u) * KSCALE);
+        af[u][nb] = load_weights<TILED>(a_ptr[nb] + static_cast<int64_t>(k + 32 * u) * KSCALE);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) bf[u][mb] = *reinterpret_cast<const uint4*>(b_ptr[mb] + k + 32 * u);
     }
@@ -696,55 +710,61 @@ extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, co
 // wavefronts per block (up to 16) as it takes to put a few thousand of them in flight.
 template <int MB, int KW, int U>
 static void launch_dense(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
-                         hipStream_t stream) {
+                         bool tiled, hipStream_t stream) {
   const int64_t items = static_cast<int64_t>(N / 16) * tiles;
   const int grid = static_cast<int>((items + 7) / 8 * 8);
-  grouped_gemm_mfma_kernel<2, MB, 1, U, KW><<<grid, 64 * KW, 0, stream>>>(
-      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), nullptr,
-      nullptr, nullptr, nullptr, rows, 1, N, K, tiles, 0);
+  if (tiled)
+    grouped_gemm_mfma_kernel<3, MB, 1, U, KW><<<grid, 64 * KW, 0, stream>>>(
+        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), nullptr,
+        nullptr, nullptr, nullptr, rows, 1, N, K, tiles, 0);
+  else
+    grouped_gemm_mfma_kernel<2, MB, 1, U, KW><<<grid, 64 * KW, 0, stream>>>(
+        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), nullptr,
+        nullptr, nullptr, nullptr, rows, 1, N, K, tiles, 0);
 }
 
 // One choice of the stage depth U: K is split over 4, 8 or 16 wavefronts (until a few thousand are
 // in flight) if a wavefront's share of K is whole stages; false if it is not.
 template <int MB, int U>
 static bool dense_with_stage(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
-                             hipStream_t stream) {
+                             bool tiled, hipStream_t stream) {
   constexpr int STAGE = 32 * U;
   const int64_t blocks = static_cast<int64_t>(N / 16) * tiles;
   int kw = 4;
   while (kw < 16 && blocks * kw < 3072 && K % (2 * kw * STAGE) == 0) kw *= 2;
   if (K % (kw * STAGE)) return false;
-  if (kw == 4) launch_dense<MB, 4, U>(x, w, out, rows, N, K, tiles, stream);
-  else if (kw == 8) launch_dense<MB, 8, U>(x, w, out, rows, N, K, tiles, stream);
-  else launch_dense<MB, 16, U>(x, w, out, rows, N, K, tiles, stream);
+  if (kw == 4) launch_dense<MB, 4, U>(x, w, out, rows, N, K, tiles, tiled, stream);
+  else if (kw == 8) launch_dense<MB, 8, U>(x, w, out, rows, N, K, tiles, tiled, stream);
+  else launch_dense<MB, 16, U>(x, w, out, rows, N, K, tiles, tiled, stream);
   return true;
 }
 
 template <int MB>
 static void dense_by_split(const void* x, const void* w, void* out, int rows, int N, int K, int tiles,
-                           hipStream_t stream) {
+                           bool tiled, hipStream_t stream) {
   // Two stages of a wavefront are in flight at a time, so the deeper the stage the more bytes it
   // has under way: with up to 16 rows a stage of six steps (96 registers for both sets) brings a
   // share of 384 along K (MiniMax-M2's qkv and output projections) in one round trip instead of
   // three.  With one weight block per wavefront even 64 rows leave registers for stages of two.
   if constexpr (MB == 1) {
-    if (dense_with_stage<MB, 6>(x, w, out, rows, N, K, tiles, stream)) return;
-    if (dense_with_stage<MB, 4>(x, w, out, rows, N, K, tiles, stream)) return;
+    if (dense_with_stage<MB, 6>(x, w, out, rows, N, K, tiles, tiled, stream)) return;
+    if (dense_with_stage<MB, 4>(x, w, out, rows, N, K, tiles, tiled, stream)) return;
   }
-  if (dense_with_stage<MB, 2>(x, w, out, rows, N, K, tiles, stream)) return;
-  dense_with_stage<MB, 1>(x, w, out, rows, N, K, tiles, stream);   // K % 128 == 0 always holds here
+  if (dense_with_stage<MB, 2>(x, w, out, rows, N, K, tiles, tiled, stream)) return;
+  dense_with_stage<MB, 1>(x, w, out, rows, N, K, tiles, tiled, stream);   // K % 128 == 0 always holds here
 }
 
+// `tiled`: w is a copy of the matrix in tiles of 16 rows x 32 k (tile_expert_weights), not in rows.
 extern "C" int se_skinny_gemm_mfma(const void* x, const void* w, void* out, int rows, int N, int K,
-                                   hipStream_t stream) {
+                                   int tiled, hipStream_t stream) {
   if (rows <= 0) return SE_OK;
   if (K <= 0 || K % 128 || N <= 0 || N % 16 || rows > 65535 * 16) return SE_ERR_SHAPE;
   if (rows <= 16)
-    dense_by_split<1>(x, w, out, rows, N, K, 1, stream);
+    dense_by_split<1>(x, w, out, rows, N, K, 1, tiled != 0, stream);
   else if (rows <= 32)
-    dense_by_split<2>(x, w, out, rows, N, K, 1, stream);
+    dense_by_split<2>(x, w, out, rows, N, K, 1, tiled != 0, stream);
   else
-    dense_by_split<4>(x, w, out, rows, N, K, (rows + 63) / 64, stream);
+    dense_by_split<4>(x, w, out, rows, N, K, (rows + 63) / 64, tiled != 0, stream);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

@@ -14,7 +14,6 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..config.registry import Architecture, read_config_json, resolve_architecture
-from ..parts import build_model
 from ..weights import loader as weight_loader
 from ..weights import random_weights
 from .batch import BatchBuilder, StepItem
@@ -86,7 +85,7 @@ class ModelRunner:
             kernels = HipKernels()
         self.kernels = kernels
         self.spec = arch.build_spec(cfg)
-        self.model = build_model(self.spec, chunk_tokens=mlp_chunk_size)
+        self.model = arch.make_model(self.spec, chunk_tokens=mlp_chunk_size)
         if getattr(kernels, "libraries", None):
             from ..kernels import library
             library.ensure_built(sorted(self.model.all_kernel_libraries()))

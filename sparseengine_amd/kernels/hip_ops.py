@@ -107,7 +107,7 @@ _SIGNATURES = {
     "moe_mfma": {
         "se_grouped_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-        "se_skinny_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "se_skinny_gemm_mfma": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_tall": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -609,25 +609,44 @@ class HipKernels:
         _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, code,
                                             _stream()), "moe_sum")
 
-    # Up to this many rows a dense product streams the weight once on MFMA.  Measured on MI355X at
-    # 8192 x 3072 and 200064 x 3072: 8 rows 12.5 / 225 us against the library's 26 / 376; 32 rows
-    # 20 / 400 against 23 / 381; from 48 rows on the library wins (the kernel's activation loads
-    # then outweigh its weight loads).
+    # Up to this many rows a dense product streams a weight matrix in rows once on MFMA.  Measured on MI355X
+    # at 8192 x 3072 and 200064 x 3072: 8 rows 12.5 / 225 us against the library's 26 / 376; 32 rows 20 / 400
+    # against 23 / 381; from 48 rows on the library wins (the kernel's activation loads then outweigh its
+    # weight loads).  With a tiled copy of the matrix (``prepare_dense_weight``) the kernel's loads are
+    # contiguous kilobytes that take the read-once hint: 200064 x 3072 at 8 rows 173 us (7.1 TB/s) against 196.
+    # At 64 rows the library still wins (8192 x 3072: 23 against 30 us; the activation rows come from 16 rows
+    # at 64 bytes each per load), so the limit is the same for both layouts.
     SKINNY_ROWS = 32
+    TILED_SKINNY_ROWS = 32
 
-    def linear(self, x, weight, out):
+    def prepare_dense_weight(self, weight: torch.Tensor):
+        """A copy of ``weight [N, K]`` in the tiles the streaming kernel loads as contiguous kilobytes, for the
+        products of steps with few rows (decode), or None if the kernel does not take the matrix.  The matrix
+        in rows stays for the BLAS library, which takes the steps with many rows: a projection so held takes
+        twice its bytes."""
+        if (weight.dim() != 2 or weight.dtype != torch.bfloat16 or weight.shape[0] % 16 or weight.shape[1] % 128
+                or not weight.is_contiguous()):
+            return None
+        return self.tile_expert_weights(weight[None])[0]
+
+    def linear(self, x, weight, out, prepared=None):
         """``out = x @ weight.T``.  Few bfloat16 rows take the streaming matrix-core kernel (the BLAS
-        library's choice for such shapes reads the weights at a fraction of memory speed); everything
-        else goes to the BLAS library."""
+        library's choice for such shapes reads the weights at a fraction of memory speed), on ``prepared``
+        (what ``prepare_dense_weight`` made of ``weight``) if it is given; everything else goes to the BLAS
+        library."""
         rows, k = x.shape
         n = weight.shape[0]
-        if (rows <= self.SKINNY_ROWS and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        limit = self.TILED_SKINNY_ROWS if prepared is not None else self.SKINNY_ROWS
+        if (rows <= limit and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and k % 128 == 0 and n % 16 == 0 and x.is_contiguous() and weight.is_contiguous()
                 and out.is_contiguous() and out.dtype == torch.bfloat16):
             _require(weight.shape[1] == k and out.shape == (rows, n), "linear shapes")
-            _check(_fn.get("moe_mfma", "se_skinny_gemm_mfma")(_ptr(x), _ptr(weight), _ptr(out), rows, n, k,
-                                                              _stream()), "skinny gemm",
-                   "K a multiple of 128, N a multiple of 16")
+            if prepared is not None:
+                _require(prepared.shape == weight.shape and prepared.dtype == weight.dtype and prepared.is_contiguous(),
+                         "linear: the prepared copy does not belong to this weight")
+            _check(_fn.get("moe_mfma", "se_skinny_gemm_mfma")(
+                _ptr(x), _ptr(weight if prepared is None else prepared), _ptr(out), rows, n, k,
+                int(prepared is not None), _stream()), "skinny gemm", "K a multiple of 128, N a multiple of 16")
             return out
         return torch.mm(x, weight.t(), out=out)
 

@@ -4,13 +4,16 @@ Order inside the mixer, as in the reference (models/minimax_m2.py:334-359): merg
 projection -> flat QK RMSNorm over the whole q row and the whole k row (optional) -> rotation of
 the leading rotary dims of every head -> k (normed, rotated) and v written to this step's slots
 -> attention of the step's queries over everything the request has cached, its own tokens
-included -> output projection.  Norm, rotation and the cache write are one kernel.
+included -> output projection.  Norm, rotation and the cache write are one kernel when the position
+part is a rotation by a table (``fused_rotation()`` hands the kernel its arguments); a position part
+that is something else returns None there and has ``apply(fb, q, k, positions)``, which changes
+``q [T, heads, D]`` and ``k [T, kv_heads, D]`` in place between the norm and the cache write.
 """
 from __future__ import annotations
 
 from ..config.specs import AttentionSpec
 from .base import MIXERS, POSITIONS, PagedKVRequest, ParamDecl, Part
-from .linear import linear
+from .linear import linear, prepare
 
 
 class GQAAttention(Part):
@@ -28,6 +31,7 @@ class GQAAttention(Part):
         self.q_width = spec.num_heads * spec.head_dim
         self.kv_width = spec.num_kv_heads * spec.head_dim
         self.position = POSITIONS.build(spec.position, head_dim=spec.head_dim)
+        self._prepared = {"qkv": None, "o": None}
 
     def param_decls(self):
         decls = {"qkv": ParamDecl((self.q_width + 2 * self.kv_width, self.hidden_size)),
@@ -46,6 +50,9 @@ class GQAAttention(Part):
         super().bind(params)
         self.position.prepare(params["qkv"].device)
 
+    def finalize(self, kernels) -> None:
+        self._prepared = {name: prepare(kernels, self.params[name]) for name in ("qkv", "o")}
+
     def work_key(self):
         """(query heads per kv head, window): what the attention kernel's work list depends on."""
         return self.spec.num_heads // self.spec.num_kv_heads, int(self.spec.window or 0)
@@ -56,14 +63,26 @@ class GQAAttention(Part):
     def forward(self, fb, x, cache_position: int, write_cache: bool = True):
         s, p, T = self.spec, self.params, x.shape[0]
         cache, meta = fb.kv_view(cache_position)
-        qkv = linear(x, p["qkv"], out=fb.buffer("attn.qkv", (T, self.q_width + 2 * self.kv_width)), kernels=fb.kernels)
-        fb.kernels.qk_norm_rope_store(
-            qkv, meta.positions, self.position.table, p.get("q_norm"), p.get("k_norm"), s.qk_norm_eps,
-            s.num_heads, s.num_kv_heads, s.head_dim, self.position.rotary_dim,
-            cache if write_cache else None, meta.slots if write_cache else None, meta.page_size,
-            pairing=getattr(self.position, "pairing", "neox"))
-        attended = fb.buffer("attn.out", (T, self.q_width))
+        qkv = linear(x, p["qkv"], out=fb.buffer("attn.qkv", (T, self.q_width + 2 * self.kv_width)), kernels=fb.kernels,
+                     prepared=self._prepared["qkv"])
         q = qkv[:, :self.q_width].view(T, s.num_heads, s.head_dim)
+        rotation = self.position.fused_rotation()
+        store = (cache, meta.slots) if write_cache else (None, None)
+        if rotation is not None:      # a rotation by a table: norm, rotation and cache write in one launch
+            fb.kernels.qk_norm_rope_store(
+                qkv, meta.positions, rotation.table, p.get("q_norm"), p.get("k_norm"), s.qk_norm_eps,
+                s.num_heads, s.num_kv_heads, s.head_dim, rotation.rotary_dim, *store, meta.page_size,
+                pairing=rotation.pairing)
+        else:                         # the position part applies itself, between the norm and the cache write
+            if "q_norm" in p:
+                fb.kernels.qk_norm_rope_store(qkv, meta.positions, None, p["q_norm"], p["k_norm"], s.qk_norm_eps,
+                                              s.num_heads, s.num_kv_heads, s.head_dim, 0, None, None, meta.page_size)
+            k = qkv[:, self.q_width:self.q_width + self.kv_width].view(T, s.num_kv_heads, s.head_dim)
+            self.position.apply(fb, q, k, meta.positions)
+            if write_cache:
+                fb.kernels.qk_norm_rope_store(qkv, meta.positions, None, None, None, s.qk_norm_eps, s.num_heads,
+                                              s.num_kv_heads, s.head_dim, 0, *store, meta.page_size)
+        attended = fb.buffer("attn.out", (T, self.q_width))
         method = getattr(fb, "method", None)
         visible = meta if method is None else method.select(cache_position, meta)     # what this layer may read
         if getattr(fb, "check_tables", False):
@@ -73,7 +92,8 @@ class GQAAttention(Part):
             method.after_attention(cache_position, fb)
         if fb.taps is not None:
             fb.taps.setdefault("attention_inputs", []).append(qkv.clone())
-        return linear(attended, p["o"], out=fb.buffer("attn.proj", (T, self.hidden_size)), kernels=fb.kernels)
+        return linear(attended, p["o"], out=fb.buffer("attn.proj", (T, self.hidden_size)), kernels=fb.kernels,
+                      prepared=self._prepared["o"])
 
 
 MIXERS.register("gqa_attention", lambda spec, hidden_size: GQAAttention(spec, hidden_size))

@@ -42,6 +42,17 @@ class StateRequest:
     tensors: tuple[tuple[str, tuple[int, ...], torch.dtype | None], ...]
 
 
+@dataclass(frozen=True)
+class FusedRotation:
+    """What a position encoding that is a rotation by a table hands to the mixer's fused kernel (flat QK
+    norm, rotation, cache write in one launch): ``table [positions, rotary_dim]`` (cos half, sin half, float32;
+    None with ``rotary_dim`` 0: nothing is turned), the number of leading dims of a head that are turned and how
+    they pair up ("neox": ``(d, d + rotary_dim / 2)``, "interleaved": ``(2 j, 2 j + 1)``)."""
+    table: torch.Tensor | None
+    rotary_dim: int
+    pairing: str = "neox"
+
+
 class SlotSum:
     """What a feed-forward hands on when the sum over a token's slots (its chosen experts) is left
     to the reader: ``parts`` holds ``[tokens * slots, hidden]``, a token's slots one after the

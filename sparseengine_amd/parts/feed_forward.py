@@ -12,7 +12,7 @@ import torch
 
 from ..config.specs import DenseMLPSpec, MoESpec
 from .base import FEED_FORWARDS, ParamDecl, Part, SlotSum
-from .linear import linear
+from .linear import linear, prepare
 
 
 ACTIVATIONS = ("silu", "gelu_tanh")      # what the kernels' epilogues can apply to a gate
@@ -140,6 +140,10 @@ class DenseMLP(Part):
             raise NotImplementedError(f"activation {spec.activation!r} is not supported ({', '.join(ACTIVATIONS)})")
         self.spec = spec
         self.hidden_size = int(hidden_size)
+        self._prepared = {"gate_up": None, "down": None}
+
+    def finalize(self, kernels) -> None:
+        self._prepared = {name: prepare(kernels, self.params[name]) for name in ("gate_up", "down")}
 
     def param_decls(self):
         i = self.spec.intermediate_size
@@ -147,10 +151,12 @@ class DenseMLP(Part):
 
     def forward(self, fb, x):
         T, i = x.shape[0], self.spec.intermediate_size
-        gate_up = linear(x, self.params["gate_up"], out=fb.buffer("mlp.gate_up", (T, 2 * i)), kernels=fb.kernels)
+        gate_up = linear(x, self.params["gate_up"], out=fb.buffer("mlp.gate_up", (T, 2 * i)), kernels=fb.kernels,
+                         prepared=self._prepared["gate_up"])
         act = fb.buffer("mlp.act", (T, i))
         fb.kernels.silu_mul(gate_up, act, activation=self.spec.activation)
-        return linear(act, self.params["down"], out=fb.buffer("ffn.out", (T, self.hidden_size)), kernels=fb.kernels)
+        return linear(act, self.params["down"], out=fb.buffer("ffn.out", (T, self.hidden_size)), kernels=fb.kernels,
+                      prepared=self._prepared["down"])
 
 
 FEED_FORWARDS.register("moe", lambda spec, hidden_size, chunk_tokens=16384: RoutedExperts(spec, hidden_size, chunk_tokens))

@@ -10,7 +10,7 @@ import torch
 
 from ..config.specs import ModelSpec
 from .base import BLOCKS, NORMS, ParamDecl, Part, SlotSum
-from .linear import linear
+from .linear import linear, prepare
 
 
 class Embedding(Part):
@@ -39,6 +39,10 @@ class DecoderModel(Part):
                        for layer in spec.layers]
         self.final_norm = NORMS.build(spec.final_norm, hidden_size=spec.hidden_size)
         self.head = None if spec.tie_word_embeddings else OutputHead(spec.vocab_size, spec.hidden_size)
+        self._prepared_head = None
+
+    def finalize(self, kernels) -> None:
+        self._prepared_head = prepare(kernels, (self.head or self.embed).params["weight"])
 
     def children(self):
         parts = {"embed": self.embed, "final_norm": self.final_norm}
@@ -57,11 +61,25 @@ class DecoderModel(Part):
                     out[position] = request
         return out
 
+    # The two ends of the model are methods of their own, so that an architecture whose ends differ (an
+    # embedding multiplier, a scale or a cap on the logits) brings a subclass that overrides them
+    # (``Architecture.model_factory``) and leaves the run of the schedule alone.
+    def embed_tokens(self, fb) -> torch.Tensor:
+        """``[T, hidden]``: what the first layer reads."""
+        x = fb.buffer("model.hidden", (fb.num_tokens, self.spec.hidden_size))
+        fb.kernels.embedding(fb.token_ids, self.embed.params["weight"], x)
+        return x
+
+    def logits_of(self, fb, last: torch.Tensor) -> torch.Tensor:
+        """Logits ``[wanted, vocab]`` (any float type) of the final-normed rows ``last [wanted, hidden]``."""
+        weight = (self.head or self.embed).params["weight"]
+        return linear(last, weight, out=fb.buffer("model.logits", (last.shape[0], self.spec.vocab_size)),
+                      kernels=fb.kernels, prepared=self._prepared_head)
+
     def forward(self, fb) -> torch.Tensor:
         """float32 logits ``[wanted, vocab]`` of the step."""
         spec = self.spec
-        x = fb.buffer("model.hidden", (fb.num_tokens, spec.hidden_size))
-        fb.kernels.embedding(fb.token_ids, self.embed.params["weight"], x)
+        x = self.embed_tokens(fb)
         residual = None
         final = len(spec.schedule) - 1
         for position, entry in enumerate(spec.schedule):
@@ -83,9 +101,7 @@ class DecoderModel(Part):
             return torch.empty(0, spec.vocab_size, dtype=torch.float32, device=fb.device)
         last = fb.buffer("model.wanted", (wanted, spec.hidden_size))
         self.final_norm.forward_rows(fb, x, residual, fb.want_index, last)
-        weight = (self.head or self.embed).params["weight"]
-        logits = linear(last, weight, out=fb.buffer("model.logits", (wanted, spec.vocab_size)), kernels=fb.kernels)
-        return logits.to(torch.float32, copy=True)      # the caller's own tensor, not the scratch buffer
+        return self.logits_of(fb, last).to(torch.float32, copy=True)      # the caller's own tensor, not the scratch buffer
 
 
 def _stream_value(x, residual) -> torch.Tensor:

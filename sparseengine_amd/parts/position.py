@@ -13,7 +13,7 @@ import weakref
 import torch
 
 from ..config.specs import NoPositionSpec, RotarySpec
-from .base import POSITIONS, Part
+from .base import POSITIONS, FusedRotation, Part
 
 
 def rotary_inverse_frequencies(rotary_dim: int, theta: float, scaling: dict | None):
@@ -112,6 +112,10 @@ class RotaryPosition(Part):
             return torch.cat((angles.cos() * factor, angles.sin() * factor), dim=-1).contiguous().to(device)
         self.table = shared_table((spec, rows, str(torch.device(device))), build)
 
+    def fused_rotation(self) -> FusedRotation:
+        """A rotation by a table: the mixer's fused kernel applies it between the QK norm and the cache write."""
+        return FusedRotation(self.table, self.rotary_dim, self.pairing)
+
 
 class NoPosition(Part):
     rotary_dim = 0
@@ -120,6 +124,9 @@ class NoPosition(Part):
 
     def __init__(self, spec=None, head_dim: int = 0):
         pass
+
+    def fused_rotation(self) -> FusedRotation:
+        return FusedRotation(None, 0)
 
     def prepare(self, device) -> None:
         pass

@@ -41,10 +41,9 @@ def checkpoint_tensors(arch: Architecture, cfg, decls, seed: int, options: dict 
 
 def write_model_folder(folder: str, raw_config: dict, seed: int, options: dict | None = None) -> str:
     """Write ``config.json`` and ``model.safetensors`` for the configuration; returns the folder."""
-    from ..parts import build_model
     arch = resolve_architecture(raw_config)
     cfg = arch.parse_config(raw_config)
-    decls = build_model(arch.build_spec(cfg)).all_param_decls()
+    decls = arch.make_model(arch.build_spec(cfg)).all_param_decls()
     os.makedirs(folder, exist_ok=True)
     tensors = {src.name: value.contiguous() for src, value in checkpoint_tensors(arch, cfg, decls, seed, options)}
     weights_file = os.path.join(folder, "model.safetensors")

@@ -792,6 +792,18 @@ def test_skinny_linear(hip, rows, n, k):
     hip.linear(x, w, out)
     ref = x.float() @ w.float().T
     torch.testing.assert_close(out.float(), ref, rtol=1.6e-2, atol=1.6e-2)
+    # the same product on a tiled copy of the matrix: every dot product runs in the same order of k, so up
+    # to the row count that both layouts leave to the streaming kernel the results are the same bits
+    prepared = hip.prepare_dense_weight(w)
+    if k % 128 or n % 16:
+        assert prepared is None
+        return
+    assert prepared.shape == w.shape and not torch.equal(prepared, w)
+    tiled_out = torch.full_like(out, float("nan"))
+    hip.linear(x, w, tiled_out, prepared=prepared)
+    torch.testing.assert_close(tiled_out.float(), ref, rtol=1.6e-2, atol=1.6e-2)
+    if rows <= hip.SKINNY_ROWS:
+        assert torch.equal(tiled_out, out)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -1,8 +1,8 @@
 """A toy architecture defined wholly in the tests, to show that parts, cache groups, state slots
 and the run order are general: layers differ in mixer (full attention, windowed attention, a
 recurrent mixer with state of its own), in feed-forward (dense, routed experts, a feed-forward
-with a routing rule of its own), in position encoding (rotary, none, a rotation with its own
-table), in norm (the engine's, one with another statistic) and in how a layer is arranged (mixer
+with a routing rule of its own), in position encoding (rotary, a rotation with its own table, one that
+is no rotation and applies itself), in the model's two ends (an embedding multiplier, a logit scale), in norm (the engine's, one with another statistic) and in how a layer is arranged (mixer
 then feed-forward, or the two side by side), the schedule runs a layer twice and lets one position read another position's cache.  Nothing in ``sparseengine_amd``
 knows about it: it registers itself through the public registries.  It is no model of anyone's.
 """
@@ -17,7 +17,7 @@ from sparseengine_amd.config.registry import Architecture, WeightSource, registe
 from sparseengine_amd.config.specs import (AttentionSpec, DenseMLPSpec, LayerSpec, ModelSpec, MoESpec, NoPositionSpec,
                                            NormSpec, RotarySpec, ScheduleEntry)
 from sparseengine_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, ParamDecl, Part, StateRequest,
-                                     build_model)
+                                     DecoderModel, FusedRotation, build_model)
 from tests.plain import minimax_m2 as P
 
 
@@ -108,12 +108,51 @@ class LinearRotary(Part):
         angles = linear_rotary_angles(torch.arange(self.spec.max_position), self.spec.rotary_dim, self.spec.slope)
         self.table = torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous().to(device)
 
+    def fused_rotation(self):
+        return FusedRotation(self.table, self.rotary_dim, "neox")
+
 
 def linear_rotary_angles(positions, rotary_dim: int, slope: float):
     return positions.float()[:, None] * (slope * torch.arange(1, rotary_dim // 2 + 1, dtype=torch.float32))[None, :]
 
 
 POSITIONS.register("toy_linear_rotary", lambda spec, head_dim: LinearRotary(spec, head_dim))
+
+
+# ------------------------------------------------------------------ a position encoding that is no rotation by a table
+@dataclass(frozen=True)
+class DecayGainSpec:
+    kind: ClassVar[str] = "toy_decay_gain"
+    rate: float = 0.02
+
+
+class DecayGain(Part):
+    """Queries grow and keys shrink with their position: dim ``d`` of every head is multiplied by
+    ``exp(+-rate * p * (d % 4))``, so that a score depends on the distance of query and key alone.  It is no
+    rotation and has no table: it applies itself (``fused_rotation`` is None), between the mixer's QK norm and
+    its cache write."""
+
+    def __init__(self, spec: DecayGainSpec, head_dim: int):
+        self.spec, self.head_dim = spec, head_dim
+
+    def prepare(self, device) -> None:
+        self.step = (self.spec.rate * (torch.arange(self.head_dim) % 4).float()).to(device)
+
+    def fused_rotation(self):
+        return None
+
+    def apply(self, fb, q, k, positions) -> None:
+        q_gain, k_gain = decay_gains(positions, self.step)
+        q.copy_((q.float() * q_gain[:, None, :]).to(q.dtype))
+        k.copy_((k.float() * k_gain[:, None, :]).to(k.dtype))
+
+
+def decay_gains(positions, step):
+    exponent = positions.float()[:, None] * step[None, :]
+    return torch.exp(exponent), torch.exp(-exponent)
+
+
+POSITIONS.register("toy_decay_gain", lambda spec, head_dim: DecayGain(spec, head_dim))
 
 
 # ------------------------------------------------------------------ a norm of another kind
@@ -217,7 +256,9 @@ def _layer_spec(cfg, layer) -> LayerSpec:
     if layer["mixer"] == "decay":
         mixer = DecayMixerSpec(state_size=layer["state_size"], decay=layer["decay"])
     else:
-        if layer.get("linear_rotary"):
+        if layer.get("decay_gain"):
+            rotary = DecayGainSpec(rate=layer["decay_gain"])
+        elif layer.get("linear_rotary"):
             rotary = LinearRotarySpec(rotary_dim=layer["rotary_dim"], slope=layer["linear_rotary"],
                                       max_position=cfg["max_position_embeddings"])
         elif layer["rotary_dim"]:
@@ -246,12 +287,25 @@ def build_spec(cfg) -> ModelSpec:
     schedule = tuple(ScheduleEntry(e["layer"], e.get("cache_from")) for e in cfg["schedule"])
     return ModelSpec(architecture="ToyForCausalLM", hidden_size=cfg["hidden_size"], vocab_size=cfg["vocab_size"],
                      layers=layers, schedule=schedule, final_norm=NormSpec(eps=cfg["eps"]),
-                     max_position=cfg["max_position_embeddings"])
+                     max_position=cfg["max_position_embeddings"],
+                     constants=(("embedding_multiplier", float(cfg.get("embedding_multiplier", 1.0))),
+                                ("logit_scale", float(cfg.get("logit_scale", 1.0)))))
+
+
+class ToyModel(DecoderModel):
+    """The generic decoder with other ends: the embedding is multiplied by a constant and the logits are
+    scaled (named by ``Architecture.model_factory``; the run of the schedule is the framework's)."""
+
+    def embed_tokens(self, fb):
+        return super().embed_tokens(fb).mul_(dict(self.spec.constants)["embedding_multiplier"])
+
+    def logits_of(self, fb, last):
+        return super().logits_of(fb, last).float() * dict(self.spec.constants)["logit_scale"]
 
 
 def weight_sources(cfg):
     """Checkpoint names are the parameter paths with a ``toy.`` prefix, tensor for tensor."""
-    return [WeightSource("toy." + path, path) for path in build_model(build_spec(cfg)).all_param_decls()]
+    return [WeightSource("toy." + path, path) for path in ToyModel(build_spec(cfg)).all_param_decls()]
 
 
 def random_tensor(cfg, name, shape, generator, options):
@@ -269,11 +323,11 @@ TOY = register_architecture(Architecture(
     name="ToyForCausalLM", model_types=("toy",), parse_config=parse, build_spec=build_spec,
     weight_sources=weight_sources, ignored_tensor=lambda name: False, random_tensor=random_tensor,
     stored_dtype=lambda name: "float32" if name.endswith(("router", "router_bias", "probe")) else "bfloat16",
-    config_to_dict=lambda cfg: dict(cfg)))
+    config_to_dict=lambda cfg: dict(cfg), model_factory=lambda spec, chunk_tokens=16384: ToyModel(spec, chunk_tokens)))
 
 TOY_CONFIG = dict(
     architectures=["ToyForCausalLM"], model_type="toy", hidden_size=64, vocab_size=300, eps=1e-5, rope_theta=10000.0,
-    max_position_embeddings=1024,
+    max_position_embeddings=1024, embedding_multiplier=1.5, logit_scale=0.5,
     layers=[
         dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=16, pairing="interleaved", qk_norm=True,
              ffn="dense", intermediate=96),
@@ -281,13 +335,13 @@ TOY_CONFIG = dict(
              bias=False, normalize=False, scaling=1.5),
         dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, ffn="moe", experts=4, top_k=3,
              intermediate=24, activation="gelu_tanh"),
-        dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, ffn="dense", intermediate=48,
-             activation="gelu_tanh", norm="mean_abs"),
+        dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, decay_gain=0.004, qk_norm=True, ffn="dense",
+             intermediate=48, activation="gelu_tanh", norm="mean_abs"),
         # (layer 0 turns neighbouring dims together, the others dims half a rotary width apart)
         dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=8, linear_rotary=0.05, ffn="sign",
              intermediate=20),
         # mixer and feed-forward side by side behind one norm of the other kind
-        dict(mixer="attention", heads=2, kv_heads=1, head_dim=32, rotary_dim=16, ffn="dense", intermediate=32,
+        dict(mixer="attention", heads=2, kv_heads=1, head_dim=32, rotary_dim=0, decay_gain=0.003, ffn="dense", intermediate=32,
              norm="mean_abs", block="toy_side_by_side"),
     ],
     # layer 0 runs twice (two caches); position 4 reads the cache of position 0 (same geometry)
@@ -311,7 +365,7 @@ class PlainToy:
         routers, signs = iter(forced.get("router", [])), iter(forced.get("sign", []))
         T = len(tokens)
         pos = torch.arange(T)
-        x = w["embed.weight"][torch.as_tensor(tokens)]
+        x = w["embed.weight"][torch.as_tensor(tokens)] * cfg.get("embedding_multiplier", 1.0)
         residual = None
         kv_of = {}
         for position, entry in enumerate(cfg["schedule"]):
@@ -337,7 +391,10 @@ class PlainToy:
                     q = P.flat_qk_norm(q, w[p + "mixer.q_norm"], cfg["eps"])
                     k = P.flat_qk_norm(k, w[p + "mixer.k_norm"], cfg["eps"])
                 q, k, v = q.reshape(T, H, D), k.reshape(T, Hkv, D), v.reshape(T, Hkv, D)
-                if layer.get("linear_rotary"):
+                if layer.get("decay_gain"):
+                    q_gain, k_gain = decay_gains(pos, layer["decay_gain"] * (torch.arange(D) % 4).float())
+                    q, k = q * q_gain[:, None, :], k * k_gain[:, None, :]
+                elif layer.get("linear_rotary"):
                     angles = linear_rotary_angles(pos, R, layer["linear_rotary"])
                     q, k = P.partial_rope(q, angles.cos(), angles.sin(), R), P.partial_rope(k, angles.cos(), angles.sin(), R)
                 elif R and layer.get("pairing") == "interleaved":
@@ -390,4 +447,4 @@ class PlainToy:
             if side_by_side:
                 x = a + x
         y, _ = P.add_rms_norm(x, residual, w["final_norm.weight"], cfg["eps"])
-        return y @ w["head.weight"].T
+        return (y @ w["head.weight"].T) * cfg.get("logit_scale", 1.0)
