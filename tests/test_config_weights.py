@@ -71,7 +71,8 @@ def test_missing_keys_and_rope_sources():
 
 
 def test_registry_and_methods():
-    assert supported_architectures() == ["MiniMaxM2ForCausalLM"]
+    # the product registers one architecture (another test of this session may have registered its toy)
+    assert [a for a in supported_architectures() if a != "ToyForCausalLM"] == ["MiniMaxM2ForCausalLM"]
     assert resolve_architecture({"architectures": ["MiniMaxM2ForCausalLM"]}).name == "MiniMaxM2ForCausalLM"
     assert resolve_architecture({"model_type": "minimax_m2"}).name == "MiniMaxM2ForCausalLM"
     with pytest.raises(NotImplementedError, match="MiniMaxM2ForCausalLM"):
