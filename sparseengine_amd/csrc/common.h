@@ -12,6 +12,13 @@
 #define SE_ERR_SHAPE -1
 #define SE_ERR_LAUNCH -2
 
+// A kernel that waits by hand for its loads into shared memory while it also has loads into registers under
+// way marks each load with this: nothing on the GPU; a build of the sources for the host (a test aid) counts
+// the loads with it, as the chip's counter does.
+#ifndef SE_NOTE_VECTOR_LOAD
+#define SE_NOTE_VECTOR_LOAD()
+#endif
+
 #define SE_CHECK_LAUNCH()                                  \
   do {                                                     \
     hipError_t e__ = hipGetLastError();                    \

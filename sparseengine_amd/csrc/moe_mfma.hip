@@ -481,7 +481,8 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
                          const int32_t* __restrict__ tile_expert,
                          const int32_t* __restrict__ counters,
                          const float* __restrict__ route_weight, int assignments, int top_k, int N,
-                         int K, int activation) {
+                         int K, int activation, int choice) {
+  if (choice >= 0 && counters[2] != choice) return;   // the device chose the other tile height (se_moe_align_choice)
   constexpr int OUT_COLS = MODE == 0 ? 128 : 256;
   constexpr int WAVES = BM / 16;                 // 4 or 8: each wavefront 64 rows x 64 weight rows
   constexpr int WCOLS = 4;                       // wave columns: the tile's 256 weight rows in 4 parts
@@ -663,7 +664,8 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
 template <int MODE, int BM>
 static int launch_wide(const void* in, const void* w, void* out, const int32_t* sorted,
                        const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
-                       int assignments, int top_k, int N, int K, int max_tiles, int activation, hipStream_t stream) {
+                       int assignments, int top_k, int N, int K, int max_tiles, int activation, int choice,
+                       hipStream_t stream) {
   const int64_t items = static_cast<int64_t>(N / (MODE == 0 ? 128 : 256)) * max_tiles;
   const int grid = static_cast<int>((items + 7) / 8 * 8);
   constexpr size_t shared = WIDE_STAGES * (16 + BM / 16) * (WIDE_KSTEP / 32) * 1024 + BM * sizeof(int32_t);
@@ -676,14 +678,16 @@ static int launch_wide(const void* in, const void* w, void* out, const int32_t* 
   }
   grouped_gemm_wide_kernel<MODE, BM, WIDE_KSTEP><<<grid, 4 * BM, shared, stream>>>(
       static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
-      tile_expert, counters, route_weight, assignments, top_k, N, K, activation);
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation, choice);
   return SE_OK;
 }
 
+// `choice`: -1, or the value counters[2] must have for the launch to do anything (se_moe_align_choice).
 extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, const int32_t* sorted,
                                     const int32_t* tile_expert, const int32_t* counters,
                                     const float* route_weight, int assignments, int top_k, int N,
-                                    int K, int max_tiles, int mode, int tile_rows, int activation, hipStream_t stream) {
+                                    int K, int max_tiles, int mode, int tile_rows, int activation, int choice,
+                                    hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
   if (K <= 0 || K % 64 || N <= 0 || N % (mode == 0 ? 128 : 256)) return SE_ERR_SHAPE;
   if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
@@ -692,14 +696,14 @@ extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, co
   int status;
   if (mode == 0)
     status = tile_rows == 128 ? launch_wide<0, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                    top_k, N, K, max_tiles, activation, stream)
+                                                    top_k, N, K, max_tiles, activation, choice, stream)
                               : launch_wide<0, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                   top_k, N, K, max_tiles, activation, stream);
+                                                   top_k, N, K, max_tiles, activation, choice, stream);
   else
     status = tile_rows == 128 ? launch_wide<1, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                    top_k, N, K, max_tiles, activation, stream)
+                                                    top_k, N, K, max_tiles, activation, choice, stream)
                               : launch_wide<1, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                   top_k, N, K, max_tiles, activation, stream);
+                                                   top_k, N, K, max_tiles, activation, choice, stream);
   if (status != SE_OK) return status;
   SE_CHECK_LAUNCH();
   return SE_OK;
@@ -765,6 +769,231 @@ extern "C" int se_skinny_gemm_mfma(const void* x, const void* w, void* out, int 
     dense_by_split<2>(x, w, out, rows, N, K, 1, tiled != 0, stream);
   else
     dense_by_split<4>(x, w, out, rows, N, K, (rows + 63) / 64, tiled != 0, stream);
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
+// ---------------------------------------------------------------------------------------- //
+// Mid tiles (an expert has a few dozen rows: a prompt of a thousand or two thousand tokens spread
+// evenly over the experts, prompt portions beside decoded tokens).  The step is bound by the expert
+// tables it has to read, like a decode step, but the streaming kernel above reads a table once per 16
+// (32) rows, and the wide kernel, which stages everything through shared memory, has too few bytes
+// under way to fill the memory system when its tiles are half empty (5.2 of 7.1 TB/s at 64 rows per
+// expert).  Here a block of eight wavefronts takes a tile of 64 or 96 sorted rows x 128 (MODE 1: 256)
+// output columns; the output columns are split over the wavefronts, so that
+//   * every wavefront streams its own weight rows (MODE 0: 16 gate rows and the matching 16 up rows;
+//     MODE 1: 32 rows) from the tiled tables straight into matrix-core operands, read-once hint and
+//     all, three stages of 64 along K deep in registers (8 KB under way per wavefront, 128 KB per CU);
+//   * the tile's activation rows, which all eight need, go once per block from memory straight into
+//     shared memory in operand order (one or two kilobytes per wavefront and stage) and are read from
+//     there, three stages deep;
+//   * no partial sums cross wavefronts: a lane's accumulators are whole dot products in the order of K.
+// The loads into shared memory are counted by the same counter as the loads into registers, which the
+// compiler waits for by itself but does not know of the former: before each barrier the wavefront waits
+// by hand until only the loads of the stages after this one are outstanding (an exact count; the
+// compiler's own waits, which come later, then find their data there or wait a little too long, never
+// too short).
+//   MODE 0: act[a, n0 + 16 wave + ...] from gate rows n0 + 16 wave ..., up rows N + n0 + 16 wave ...
+//   MODE 1: out[a, n0 + 32 wave + ...] * route_weight[a]
+// Requires K % 64 == 0, N % 128 == 0 (MODE 0) / N % 256 == 0 (MODE 1).
+// ---------------------------------------------------------------------------------------- //
+#define MID_WAVES 8
+#define MID_STAGES 3
+#define MID_KSTEP 64
+
+// bytes of shared memory before the tile's row list: the stages of activation rows or the tile of results
+__host__ __device__ constexpr int mid_shared_bytes(int mode, int mb) {
+  const int stages = MID_STAGES * mb * (MID_KSTEP / 32) * 1024;
+  const int results = 16 * mb * ((mode == 0 ? 16 : 32) * MID_WAVES * 2 + 16);
+  return stages > results ? stages : results;
+}
+
+template <int MODE, int MB>   // MB row blocks of 16: tiles of 64 or 96 sorted rows
+__global__ void __launch_bounds__(64 * MID_WAVES, 2)
+grouped_gemm_mid_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                        bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ counters,
+                        const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                        int K, int activation, int choice) {
+  if (choice >= 0 && counters[2] != choice) return;   // the device chose the other tile height (se_moe_align_choice)
+  constexpr int BM = 16 * MB;
+  constexpr int U = MID_KSTEP / 32;              // steps of 32 per stage
+  constexpr int TILES = MB * U;                  // activation tiles (1 KB) of a stage
+  constexpr int OUT_COLS = (MODE == 0 ? 16 : 32) * MID_WAVES;
+  static_assert(TILES >= MID_WAVES && TILES <= 2 * MID_WAVES, "a wavefront brings one or two activation tiles per stage");
+  int tile, column_block;
+  if (!xcd_work_item(N / OUT_COLS, counters[0], tile, column_block)) return;  // uniform
+  // MID_STAGES x TILES x 64 vectors, which the tile of results takes over in the end; then the rows
+  extern __shared__ __align__(16) uint4 mid_shared[];
+  uint4(*stage)[TILES][SE_WAVE] = reinterpret_cast<uint4(*)[TILES][SE_WAVE]>(mid_shared);
+  int32_t* rows = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(mid_shared) + mid_shared_bytes(MODE, MB));
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (SE_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SE_WAVE);
+  const int col = lane & 15, kgroup = lane >> 4;
+  const int expert = tile_expert[tile];
+  const int n0 = column_block * OUT_COLS;
+  if (tid < BM) rows[tid] = sorted[tile * BM + tid];
+  __syncthreads();
+
+  // the wavefront's two weight row blocks, as tiles of 16 rows x 32 k (1 KB each, 512 elements apart along k)
+  const int64_t w_rows = MODE == 0 ? 2 * static_cast<int64_t>(N) : N;
+  const bf16_t* we = w + static_cast<int64_t>(expert) * w_rows * K;
+  const int64_t row_block0 = MODE == 0 ? (n0 + 16 * wave) / 16 : (n0 + 32 * wave) / 16;
+  const int64_t row_block1 = MODE == 0 ? (static_cast<int64_t>(N) + n0 + 16 * wave) / 16 : row_block0 + 1;
+  const bf16_t* a_ptr0 = we + row_block0 * (K / 32) * 512 + lane * 8;
+  const bf16_t* a_ptr1 = we + row_block1 * (K / 32) * 512 + lane * 8;
+
+  // the activation tiles this wavefront brings per stage: tile j = (step u = j / MB, row block j % MB);
+  // lane (kgroup, col) brings 8 k of row 16 (j % MB) + col: its 16 bytes are what it feeds the matrix core
+  const bool two_tiles = wave + MID_WAVES < TILES;      // the same for the whole wavefront
+  const bf16_t* x_ptr[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int j = min(wave + t * MID_WAVES, TILES - 1);
+    const int a = rows[(j % MB) * 16 + col];
+    const int64_t src = a < assignments ? (MODE == 0 ? a / top_k : a) : 0;  // padding reads row 0
+    x_ptr[t] = in + src * K + kgroup * 8 + 32 * (j / MB);
+  }
+  const uint32_t stage_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(mid_shared));
+  auto bring_rows = [&](int s) {      // the loads of stage s into shared memory
+    const uint32_t dst = stage_base + static_cast<uint32_t>((s % MID_STAGES) * TILES + wave) * 1024u;
+    load16_to_lds(x_ptr[0] + static_cast<int64_t>(s) * MID_KSTEP, dst);
+    if (two_tiles) load16_to_lds(x_ptr[1] + static_cast<int64_t>(s) * MID_KSTEP, dst + MID_WAVES * 1024u);
+  };
+
+  floatx4 acc[2][MB];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[nb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // three register sets take turns: while the matrix cores work on one stage the weights of the next two
+  // are under way
+  uint4 w0[U][2], w1[U][2], w2[U][2];
+  auto bring_weights = [&](uint4 (&wf)[U][2], int s) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      wf[u][0] = load16_once(a_ptr0 + (static_cast<int64_t>(s) * MID_KSTEP + 32 * u) * 16);
+      SE_NOTE_VECTOR_LOAD();
+      wf[u][1] = load16_once(a_ptr1 + (static_cast<int64_t>(s) * MID_KSTEP + 32 * u) * 16);
+      SE_NOTE_VECTOR_LOAD();
+    }
+  };
+  const int steps = K / MID_KSTEP;
+  auto run_stage = [&](const uint4 (&wf)[U][2], uint4 (&next)[U][2], int s) {
+    // stage s of everyone's rows is in shared memory once every wavefront has seen its own loads of it
+    // land: all but the loads of the stages after s (the weights of stage s + 1, issued before its rows)
+    if (s + 1 < steps) {
+      if (two_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * U + 2));
+      else __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * U + 1));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __builtin_amdgcn_s_barrier();   // and everyone has left stage s - 1, whose buffer stage s + 2 takes
+    asm volatile("" ::: "memory");
+    if (s + 2 < steps) {
+      bring_weights(next, s + 2);
+      bring_rows(s + 2);
+    }
+    const uint4(*rows_of)[SE_WAVE] = stage[s % MID_STAGES];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const uint4 bfrag = rows_of[u * MB + mb][lane];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+          acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf[u][nb]),
+                                                               __builtin_bit_cast(bf16x8, bfrag), acc[nb][mb], 0, 0, 0);
+      }
+    asm volatile("" ::: "memory");
+  };
+  bring_weights(w0, 0);
+  bring_rows(0);
+  if (steps > 1) {
+    bring_weights(w1, 1);
+    bring_rows(1);
+  }
+  for (int s = 0; s < steps; s += 3) {
+    run_stage(w0, w2, s);
+    if (s + 1 < steps) run_stage(w1, w0, s + 1);
+    if (s + 2 < steps) run_stage(w2, w1, s + 2);
+  }
+
+  // The results leave through shared memory, a row's columns as whole cache lines: written from the lanes
+  // that hold them (8 bytes each, 32 bytes of a row per wavefront) they take several times as long as their
+  // bytes need, measured 230 us of a 1350 us layer at 64 rows per expert.
+  // lane (kgroup, col): acc[nb][mb][i] belongs to weight row 4 * kgroup + i of the wavefront's block nb, tile row 16 mb + col
+  constexpr int ROW_BYTES = OUT_COLS * 2;
+  constexpr int ROW_STRIDE = ROW_BYTES + 16;      // rows 132 (260) words apart: the lanes of a store hit different banks
+  __syncthreads();                                // everyone has left the last stage
+  char* out_tile = reinterpret_cast<char*>(mid_shared);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    char* t_row = out_tile + (16 * mb + col) * ROW_STRIDE + 8 * kgroup;
+    if (MODE == 0) {
+      uint16_t y[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float gate = round_to<bf16_t>(acc[0][mb][i]);
+        const float up = round_to<bf16_t>(acc[1][mb][i]);
+        const float act = round_to<bf16_t>(gate_activation<true>(gate, activation));
+        y[i] = float_to_bf16_bits(act * up);
+      }
+      uint2 packed;
+      packed.x = static_cast<uint32_t>(y[0]) | (static_cast<uint32_t>(y[1]) << 16);
+      packed.y = static_cast<uint32_t>(y[2]) | (static_cast<uint32_t>(y[3]) << 16);
+      *reinterpret_cast<uint2*>(t_row + 32 * wave) = packed;
+    } else {
+      const int a = rows[16 * mb + col];
+      const float rw = a < assignments ? route_weight[a] : 0.f;
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][0] * rw)) |
+                   (static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][1] * rw)) << 16);
+        packed.y = static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][2] * rw)) |
+                   (static_cast<uint32_t>(float_to_bf16_bits(acc[nb][mb][3] * rw)) << 16);
+        *reinterpret_cast<uint2*>(t_row + 64 * wave + 32 * nb) = packed;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int LANES_PER_ROW = ROW_BYTES / 16;   // 16 bytes a thread
+  for (int r = tid / LANES_PER_ROW; r < BM; r += 64 * MID_WAVES / LANES_PER_ROW) {
+    const int a = rows[r];
+    if (a >= assignments) continue;               // padding
+    const int piece = tid % LANES_PER_ROW;
+    // written once and read by a later kernel: past the caches (measured: 1245 against 1335 us for a layer at 64 rows per expert)
+    __builtin_nontemporal_store(*reinterpret_cast<const se_u32x4*>(out_tile + r * ROW_STRIDE + 16 * piece),
+                                reinterpret_cast<se_u32x4*>(out + static_cast<int64_t>(a) * N + n0 + 8 * piece));
+  }
+}
+
+// tile_rows: 64 or 96.  MODE 0 needs N % 128 == 0, MODE 1 N % 256 == 0; K % 64 == 0.
+// `choice`: -1, or the value counters[2] must have for the launch to do anything (se_moe_align_choice).
+extern "C" int se_grouped_gemm_mid(const void* in, const void* w, void* out, const int32_t* sorted,
+                                   const int32_t* tile_expert, const int32_t* counters,
+                                   const float* route_weight, int assignments, int top_k, int N,
+                                   int K, int max_tiles, int mode, int tile_rows, int activation, int choice,
+                                   hipStream_t stream) {
+  if (assignments <= 0) return SE_OK;
+  if (K <= 0 || K % MID_KSTEP || N <= 0 || N % (mode == 0 ? 128 : 256)) return SE_ERR_SHAPE;
+  if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
+  if (tile_rows != 64 && tile_rows != 96) return SE_ERR_SHAPE;
+  if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
+  const int64_t items = static_cast<int64_t>(N / (mode == 0 ? 128 : 256)) * max_tiles;
+  const int grid = static_cast<int>((items + 7) / 8 * 8);
+#define SE_MID(MODE, MB)                                                                           \
+  grouped_gemm_mid_kernel<MODE, MB><<<grid, 64 * MID_WAVES,                                        \
+                                      mid_shared_bytes(MODE, MB) + 16 * MB * sizeof(int32_t), stream>>>( \
+      static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation, choice)
+  if (tile_rows == 64) { if (mode == 0) SE_MID(0, 4); else SE_MID(1, 4); }
+  else { if (mode == 0) SE_MID(0, 6); else SE_MID(1, 6); }
+#undef SE_MID
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

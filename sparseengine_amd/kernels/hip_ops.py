@@ -98,6 +98,7 @@ _SIGNATURES = {
         "se_router_topk_align": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                  c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_moe_align": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+        "se_moe_align_choice": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_grouped_gemm_generic": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_void_p],
@@ -111,7 +112,9 @@ _SIGNATURES = {
         "se_grouped_gemm_tall": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "se_grouped_gemm_mid": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "memory_probe": {
         "se_stream_read": [c_void_p, c_int64, c_void_p, c_int, c_void_p],
@@ -167,7 +170,7 @@ class MoeWorkspace:
         self.hidden, self.intermediate, self.dtype = hidden, intermediate, dtype
         self.sorted = torch.empty(capacity, dtype=torch.int32, device=device)
         self.tile_expert = torch.empty(max_tiles, dtype=torch.int32, device=device)
-        self.counters = torch.zeros(2, dtype=torch.int32, device=device)
+        self.counters = torch.zeros(4, dtype=torch.int32, device=device)     # tiles, sorted entries, the device's choice
         self.grouped = None      # set by router_topk when its launch has grouped the assignments already
         # rows by assignment, or (the direct kernel) by sorted position, padding included
         self.act = torch.empty(capacity, intermediate, dtype=dtype, device=device)
@@ -505,6 +508,10 @@ class HipKernels:
         return True
 
     ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}      # what a gated feed-forward applies to its gate
+    # the device's choice between the mid kernel (tiles of 96 rows) and the wide one (tiles of 128): mid if the
+    # experts that got rows got at most this many on average (with 72, hardly one of them overflows a tile of 96)
+    AUTO_TILE_ROWS = (96, 128)
+    AUTO_FEW_ROWS = 72
 
     def _activation(self, name: str) -> int:
         if name not in self.ACTIVATIONS:
@@ -540,40 +547,60 @@ class HipKernels:
         if self.takes_tiled_expert_weights(x.dtype, hidden, inter):
             if not tiled:
                 w13, w2 = self.tile_expert_weights(w13), self.tile_expert_weights(w2)
-            # matrix-core path, three kernels:
+            # matrix-core path, four kernels:
             #   "stream"  weights from memory straight into operands, tiles of 16 (32, 64) rows: an
             #             expert's table is read once per tile;
-            #   "tall"    64 x 128 tiles, operands through registers into LDS, an expert's tiles side by side;
+            #   "mid"     tiles of 64 or 96 rows: the output columns split over eight wavefronts that each stream
+            #             their own weight rows into operands; the tile's rows shared through LDS;
             #   "direct"  64 or 128 rows x 256 weight rows, operands straight into LDS as contiguous
-            #             kilobytes of the tiled tables, two blocks per CU.
-            # Which experts a step uses is known on the device only: the choice goes by the average
-            # rows per expert and has to hold for even and for lumpy routing alike.  Measured at
-            # MiniMax-M2 sizes (256 experts, top 8): with even routing "stream" wins by 3 to 5 % up to
-            # 128 tokens and loses by 11 % at 512; when the tokens of a step agree on a few dozen
-            # experts (deep layers of a prompt) it loses from 48 tokens on, by a factor of two at
-            # 512.  So: "stream" below three rows per expert (a decode batch of 64 keeps it, a
-            # prompt portion of 96 does not).  "direct" with 128 rows equals "tall" at 384 tokens of
-            # a prompt and is 6 % faster at 512, 15 % at 1024, 23 % at 2048 (registers are fed at a
-            # third of the rate of direct loads); with tiles of 64 rows it equals "tall" from 96 to
-            # 384 tokens, so that one stays for three to sixteen rows per expert.
+            #             kilobytes of the tiled tables, two blocks per CU;
+            #   "tall"    64 x 128 tiles, operands through registers into LDS (sizes the two above do not take).
+            # Which experts a step uses is known on the device only.  The host goes by the average rows per
+            # expert: below three, "stream" (a decode batch of 64 keeps it; when the tokens of a step agree on a
+            # few dozen experts it would read their tables once per 16 rows, and loses from 48 tokens on).  From
+            # there on the device chooses between "mid" and "direct" ("auto", below).
             share = assignments / min(experts, assignments)
             direct_ok = inter % 128 == 0 and hidden % 256 == 0
             if kernel is None:
                 if tile_rows is not None:
                     kernel = "stream" if tile_rows < 64 else ("direct" if tile_rows == 128 and direct_ok else "tall")
                 else:
-                    kernel = "stream" if share < 3 else ("direct" if share >= 16 and direct_ok else "tall")
-            if kernel not in ("stream", "tall", "direct"):
-                raise ValueError(f"expert kernel {kernel!r} is unknown (stream, tall, direct)")
-            if kernel == "direct" and not direct_ok:
-                raise KernelShapeError("the direct expert kernel takes hidden sizes in steps of 256 and "
+                    kernel = "stream" if share < 3 else ("auto" if direct_ok else "tall")
+            if kernel not in ("stream", "tall", "direct", "mid", "auto"):
+                raise ValueError(f"expert kernel {kernel!r} is unknown (stream, tall, direct, mid, auto)")
+            if kernel in ("direct", "mid", "auto") and not direct_ok:
+                raise KernelShapeError(f"the {kernel} expert kernel takes hidden sizes in steps of 256 and "
                                        "intermediate sizes in steps of 128")
-            if tile_rows is None:
-                tile_rows = {"stream": 16, "tall": 64, "direct": 128 if share >= 16 else 64}[kernel]
-            max_tiles = self._grouped_tiles(ids, experts, ws, tile_rows)
-            if max_tiles > 65535:
-                raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
             takes = "hidden and intermediate sizes in multiples of 128"
+            if kernel == "auto":
+                # "mid" or "direct", chosen where the spread of the rows over the experts is known: on the device.
+                # Both pairs of launches are made; the pair that was not chosen leaves at once (4 us a layer).
+                # Measured at MiniMax-M2 sizes with the rows spread evenly: 64 rows per expert 1245 (mid) against
+                # 1373 us (direct), 32 rows 1190 against 1290, 16 rows 1150 against 1250, 4 rows 1075 against 1164
+                # (the tall kernel, which this replaces); at 128 rows per expert, and whenever the tokens of a prompt
+                # agree on a few dozen experts, direct wins (an expert's table is then read once per 96 rows by mid).
+                few_tile, many_tile = self.AUTO_TILE_ROWS
+                max_tiles = max(moe_tile_bounds(assignments, experts, few_tile)[1],
+                                moe_tile_bounds(assignments, experts, many_tile)[1])
+                if max_tiles > 65535:
+                    raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
+                ws.grouped = None
+                _check(_fn.get("moe", "se_moe_align_choice")(
+                    _ptr(ids), assignments, experts, few_tile, many_tile, self.AUTO_FEW_ROWS, _ptr(ws.sorted),
+                    _ptr(ws.tile_expert), _ptr(ws.counters), _stream()), "moe_align (choice)")
+                mid, wide = _fn.get("moe_mfma", "se_grouped_gemm_mid"), _fn.get("moe_mfma", "se_grouped_gemm_wide")
+                for mode, (src, w, dst, rw, n, k) in enumerate(((x, w13, ws.act, None, inter, hidden),
+                                                               (ws.act, w2, ws.slot_out, weights, hidden, inter))):
+                    for choice, (fn, rows) in enumerate(((mid, few_tile), (wide, many_tile))):
+                        _check(fn(_ptr(src), _ptr(w), _ptr(dst), _ptr(ws.sorted), _ptr(ws.tile_expert), _ptr(ws.counters),
+                                  _ptr(rw), assignments, top_k, n, k, max_tiles, mode, rows, act, choice, _stream()),
+                               f"moe {'down' if mode else 'gate-up'} ({'direct' if choice else 'mid'})", takes)
+            else:
+                if tile_rows is None:
+                    tile_rows = {"stream": 16, "tall": 64, "direct": 128 if share >= 16 else 64, "mid": 96}[kernel]
+                max_tiles = self._grouped_tiles(ids, experts, ws, tile_rows)
+                if max_tiles > 65535:
+                    raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
             if kernel == "stream":
                 gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
                 if column_blocks is None:
@@ -584,14 +611,16 @@ class HipKernels:
                 _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
                           tile_rows, column_blocks, act, _stream()), "moe down (stream)", takes)
-            else:
-                gt = _fn.get("moe_mfma", "se_grouped_gemm_wide" if kernel == "direct" else "se_grouped_gemm_tall")
+            elif kernel != "auto":
+                gt = _fn.get("moe_mfma", {"direct": "se_grouped_gemm_wide", "tall": "se_grouped_gemm_tall",
+                                          "mid": "se_grouped_gemm_mid"}[kernel])
+                extra = () if kernel == "tall" else (-1,)      # no choice was made on the device: the launch runs
                 _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                          act, _stream()), f"moe gate-up ({kernel})", takes)
+                          act, *extra, _stream()), f"moe gate-up ({kernel})", takes)
                 _check(gt(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                          tile_rows, act, _stream()), f"moe down ({kernel})", takes)
+                          tile_rows, act, *extra, _stream()), f"moe down ({kernel})", takes)
         else:
             _require(not tiled, "the general expert kernel reads row-major tables")
             max_tiles = self._grouped_tiles(ids, experts, ws, 16)

@@ -142,7 +142,8 @@ inline void emu_yield() { swapcontext(&emu.current->context, &emu.scheduler); }
 inline void emu_complete_lds(EmuThread* t, size_t leave) {
   const size_t n = t->lds_loads.size();
   if (n <= leave) return;
-  for (size_t i = 0; i < n - leave; ++i) memcpy(t->lds_loads[i].dst, t->lds_loads[i].src, 16);
+  for (size_t i = 0; i < n - leave; ++i)
+    if (t->lds_loads[i].dst) memcpy(t->lds_loads[i].dst, t->lds_loads[i].src, 16);      // a load into registers: counted only
   t->lds_loads.erase(t->lds_loads.begin(), t->lds_loads.begin() + (n - leave));
 }
 
@@ -515,6 +516,12 @@ inline void emu_load16_to_lds(const void* src, uint32_t lds_address) {
   }
   t->lds_loads.push_back({src, dst});
 }
+// A load into registers of a kernel that waits by hand (SE_NOTE_VECTOR_LOAD): it takes its place in the queue
+// that s_waitcnt counts, as on the chip, and has nothing to do when it completes.
+inline void emu_note_vector_load() {
+  if (emu_rt_lds_mode() != 1) emu.current->lds_loads.push_back({nullptr, nullptr});
+}
+#define SE_NOTE_VECTOR_LOAD() emu_note_vector_load()
 // s_waitcnt: only the count of vector memory operations matters here (bits 3:0 and 15:14)
 inline void emu_s_waitcnt(int imm) {
   const size_t vmcnt = static_cast<size_t>((imm & 0xf) | (((imm >> 14) & 0x3) << 4));

@@ -173,10 +173,10 @@ def _outputs(hip, twin):
     ids = torch.stack([torch.randperm(experts, generator=torch.Generator().manual_seed(t))[:k] for t in range(tokens)]).int()
     weights = torch.full((tokens, k), 0.5)
     ws = MoeWorkspace(tokens, k, experts, hidden, inter, BF16, "cpu")
-    for kernel, rows in (("stream", 16), ("tall", 64), ("direct", 128)):
+    for kernel, rows in (("stream", 16), ("tall", 64), ("direct", 128), ("mid", 64), ("mid", 96)):
         y = torch.empty_like(x)
         hip.moe_experts(x, w13, w2, ids, weights, y, ws, kernel=kernel, tile_rows=rows)
-        out[kernel] = y
+        out[f"{kernel}{rows}"] = y
     logits = G.randn(5, 40, dtype=F32, seed=6)
     ids5 = torch.empty(5, 3, dtype=torch.int32)
     w5 = torch.empty(5, 3)

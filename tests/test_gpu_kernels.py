@@ -321,7 +321,7 @@ def test_router_with_grouping_in_one_launch(hip, tokens, experts, k):
     assert ws_b.grouped is not None and ws_b.grouped[5] == tiles_a
     assert torch.equal(ids_a, ids_b) and torch.equal(w_a, w_b)
     assert torch.equal(ws_a.counters, ws_b.counters)
-    n_tiles, n_sorted = ws_a.counters.tolist()
+    n_tiles, n_sorted = ws_a.counters.tolist()[:2]
     assert torch.equal(ws_a.tile_expert[:n_tiles], ws_b.tile_expert[:n_tiles])
     # the order inside an expert's run is free: compare the runs as sets
     sa, sb = ws_a.sorted[:n_sorted].view(n_tiles, 16), ws_b.sorted[:n_sorted].view(n_tiles, 16)
@@ -364,7 +364,7 @@ def test_whole_router(hip, dtype, tokens, experts, k, hidden):
         torch.testing.assert_close(logits_b, (x.double() @ w.double().T).float(), rtol=1e-5, atol=1e-5)
         assert torch.equal(logits_a, logits_b) and torch.equal(ids_a, ids_b) and torch.equal(w_a, w_b)
         assert torch.equal(ws_a.counters, ws_b.counters)
-        n_tiles, n_sorted = ws_a.counters.tolist()
+        n_tiles, n_sorted = ws_a.counters.tolist()[:2]
         assert torch.equal(ws_a.tile_expert[:n_tiles], ws_b.tile_expert[:n_tiles])
         sa, sb = ws_a.sorted[:n_sorted].view(n_tiles, 16), ws_b.sorted[:n_sorted].view(n_tiles, 16)
         assert torch.equal(sa.sort(-1).values, sb.sort(-1).values)
@@ -421,7 +421,7 @@ def test_moe_align_groups_every_assignment_once(hip):
         for rows in (16, 32, 64):
             ws.sorted.fill_(-7); ws.tile_expert.fill_(-7)
             hip.moe_align(ids, experts, ws, rows)
-            n_tiles, n_sorted = ws.counters.tolist()
+            n_tiles, n_sorted = ws.counters.tolist()[:2]
             assert n_sorted == n_tiles * rows
             sorted_ids = ws.sorted[:n_sorted].cpu()
             real = sorted_ids[sorted_ids < tokens * k]
@@ -459,7 +459,8 @@ def test_moe_experts(hip, twin, dtype, tokens, hidden, inter, experts, k, activa
     torch.testing.assert_close(out_h, out_t, **tol(dtype))
     if dtype == torch.bfloat16 and hidden % 256 == 0 and inter % 128 == 0 and tokens <= 200:
         # every kernel and tile on a step that would not choose it (mostly padding): same result
-        for kernel, rows in (("direct", 128), ("direct", 64), ("tall", 64), ("stream", 16), ("stream", 32)):
+        for kernel, rows in (("direct", 128), ("direct", 64), ("tall", 64), ("stream", 16), ("stream", 32), ("mid", 64),
+                             ("mid", 96), ("auto", None)):
             out_w = torch.empty_like(x)
             hip.moe_experts(x, w13, w2, ids, weights, out_w, ws, kernel=kernel, tile_rows=rows, activation=activation)
             torch.testing.assert_close(out_w, out_t, **tol(dtype))
@@ -489,9 +490,9 @@ def test_wide_tiles_leave_out_row_blocks_of_padding(hip, twin, counts):
     ws = MoeWorkspace(tokens, 1, experts, hidden, inter, dtype, DEV)
     out_t = torch.empty_like(x)
     twin.moe_experts(x, w13, w2, ids, weights, out_t)
-    for rows in (128, 64):
+    for kernel, rows in (("direct", 128), ("direct", 64), ("mid", 64), ("mid", 96)):
         out_h = torch.full_like(x, float("nan"))
-        hip.moe_experts(x, w13, w2, ids, weights, out_h, ws, kernel="direct", tile_rows=rows)
+        hip.moe_experts(x, w13, w2, ids, weights, out_h, ws, kernel=kernel, tile_rows=rows)
         torch.testing.assert_close(out_h, out_t, **tol(dtype))
 
 
@@ -1036,11 +1037,41 @@ def test_experts_on_random_shapes_and_lumpy_routing(hip, twin):
         twin.moe_experts(x, w13, w2, ids, weights, ref)
         a13, a2 = w13.clone(), w2.clone()
         assert hip.arrange_expert_weights(a13, a2)
-        for kernel, rows in ((None, None), ("stream", 16), ("tall", 64), ("direct", 64), ("direct", 128)):
+        for kernel, rows in ((None, None), ("stream", 16), ("tall", 64), ("direct", 64), ("direct", 128), ("mid", 64),
+                             ("mid", 96), ("auto", None)):
             out = torch.full_like(x, float("nan"))
             hip.moe_experts(x, a13, a2, ids, weights, out, ws, kernel=kernel, tile_rows=rows, tiled=True)
             torch.testing.assert_close(out, ref, **tol(dtype), msg=lambda m: (
                 f"case {case}: {tokens} tokens, {experts} experts, top {k}, hidden {hidden}, width {inter}, kernel {kernel}: {m}"))
+
+
+def test_the_device_chooses_the_expert_kernel_by_the_spread_of_the_rows(hip, twin):
+    """"auto": the grouping kernel counts the experts that got rows and chooses tiles of 96 rows (the mid kernel)
+    if they got at most 72 each on average, else tiles of 128 (the wide kernel); the launches of the other kernel
+    leave at once.  The same tokens spread evenly and crowded onto two experts: the choice differs, the results
+    are the twin's both times."""
+    from sparseengine_amd.kernels.hip_ops import MoeWorkspace
+    tokens, hidden, inter, experts, k = 400, 256, 128, 16, 2
+    emulator_skips(tokens * k * hidden * inter, 1.2e8)
+    dtype = torch.bfloat16
+    x = randn(tokens, hidden, dtype=dtype, seed=31)
+    w13 = randn(experts, 2 * inter, hidden, dtype=dtype, scale=hidden ** -0.5, seed=32)
+    w2 = randn(experts, hidden, inter, dtype=dtype, scale=inter ** -0.5, seed=33)
+    weights = torch.full((tokens, k), 0.5).to(DEV)
+    ws = MoeWorkspace(tokens, k, experts, hidden, inter, dtype, DEV)
+    g = torch.Generator().manual_seed(34)
+    even = torch.stack([torch.randperm(experts, generator=g)[:k] for _ in range(tokens)]).to(torch.int32).to(DEV)   # 50 rows each
+    crowded = torch.tensor([[3, 11]] * tokens, dtype=torch.int32).to(DEV)                                            # 400 rows each
+    for ids, choice, tile_rows in ((even, 0, 96), (crowded, 1, 128)):
+        ref = torch.empty_like(x)
+        twin.moe_experts(x, w13, w2, ids, weights, ref)
+        out = torch.full_like(x, float("nan"))
+        hip.moe_experts(x, w13, w2, ids, weights, out, ws, kernel="auto")
+        torch.testing.assert_close(out, ref, **tol(dtype))
+        counters = ws.counters.tolist()
+        assert counters[2] == choice
+        rows = torch.bincount(ids.flatten().long().cpu(), minlength=experts)
+        assert counters[0] == int(((rows + tile_rows - 1) // tile_rows).sum()) and counters[1] == counters[0] * tile_rows
 
 
 def test_memory_probe_reads_and_copies_every_byte(hip):
