@@ -475,14 +475,12 @@ extern "C" int se_grouped_gemm_tall(const void* in, const void* w, void* out, co
 #endif
 
 template <int MODE, int BM, int KSTEP>   // BM: 64 or 128 rows per tile; KSTEP: 32 or 64 along K per stage
-__global__ void __launch_bounds__(4 * BM, KSTEP == 32 ? 2 : 1)
-grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
-                         bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
-                         const int32_t* __restrict__ tile_expert,
-                         const int32_t* __restrict__ counters,
-                         const float* __restrict__ route_weight, int assignments, int top_k, int N,
-                         int K, int activation, int choice) {
-  if (choice >= 0 && counters[2] != choice) return;   // the device chose the other tile height (se_moe_align_choice)
+__device__ __forceinline__ void wide_tile(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                                          bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                                          const int32_t* __restrict__ tile_expert,
+                                          const int32_t* __restrict__ counters,
+                                          const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                                          int K, int activation) {
   constexpr int OUT_COLS = MODE == 0 ? 128 : 256;
   constexpr int WAVES = BM / 16;                 // 4 or 8: each wavefront 64 rows x 64 weight rows
   constexpr int WCOLS = 4;                       // wave columns: the tile's 256 weight rows in 4 parts
@@ -660,12 +658,22 @@ grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict
   }
 }
 
+template <int MODE, int BM, int KSTEP>
+__global__ void __launch_bounds__(4 * BM, KSTEP == 32 ? 2 : 1)
+grouped_gemm_wide_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                         bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                         const int32_t* __restrict__ tile_expert,
+                         const int32_t* __restrict__ counters,
+                         const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                         int K, int activation) {
+  wide_tile<MODE, BM, KSTEP>(in, w, out, sorted, tile_expert, counters, route_weight, assignments, top_k, N, K, activation);
+}
+
 // tile_rows: 64 or 128.  MODE 0 needs N % 128 == 0, MODE 1 N % 256 == 0; K % 64 == 0.
 template <int MODE, int BM>
 static int launch_wide(const void* in, const void* w, void* out, const int32_t* sorted,
                        const int32_t* tile_expert, const int32_t* counters, const float* route_weight,
-                       int assignments, int top_k, int N, int K, int max_tiles, int activation, int choice,
-                       hipStream_t stream) {
+                       int assignments, int top_k, int N, int K, int max_tiles, int activation, hipStream_t stream) {
   const int64_t items = static_cast<int64_t>(N / (MODE == 0 ? 128 : 256)) * max_tiles;
   const int grid = static_cast<int>((items + 7) / 8 * 8);
   constexpr size_t shared = WIDE_STAGES * (16 + BM / 16) * (WIDE_KSTEP / 32) * 1024 + BM * sizeof(int32_t);
@@ -678,16 +686,14 @@ static int launch_wide(const void* in, const void* w, void* out, const int32_t* 
   }
   grouped_gemm_wide_kernel<MODE, BM, WIDE_KSTEP><<<grid, 4 * BM, shared, stream>>>(
       static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
-      tile_expert, counters, route_weight, assignments, top_k, N, K, activation, choice);
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation);
   return SE_OK;
 }
 
-// `choice`: -1, or the value counters[2] must have for the launch to do anything (se_moe_align_choice).
 extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, const int32_t* sorted,
                                     const int32_t* tile_expert, const int32_t* counters,
                                     const float* route_weight, int assignments, int top_k, int N,
-                                    int K, int max_tiles, int mode, int tile_rows, int activation, int choice,
-                                    hipStream_t stream) {
+                                    int K, int max_tiles, int mode, int tile_rows, int activation, hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
   if (K <= 0 || K % 64 || N <= 0 || N % (mode == 0 ? 128 : 256)) return SE_ERR_SHAPE;
   if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
@@ -696,14 +702,14 @@ extern "C" int se_grouped_gemm_wide(const void* in, const void* w, void* out, co
   int status;
   if (mode == 0)
     status = tile_rows == 128 ? launch_wide<0, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                    top_k, N, K, max_tiles, activation, choice, stream)
+                                                    top_k, N, K, max_tiles, activation, stream)
                               : launch_wide<0, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                   top_k, N, K, max_tiles, activation, choice, stream);
+                                                   top_k, N, K, max_tiles, activation, stream);
   else
     status = tile_rows == 128 ? launch_wide<1, 128>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                    top_k, N, K, max_tiles, activation, choice, stream)
+                                                    top_k, N, K, max_tiles, activation, stream)
                               : launch_wide<1, 64>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
-                                                   top_k, N, K, max_tiles, activation, choice, stream);
+                                                   top_k, N, K, max_tiles, activation, stream);
   if (status != SE_OK) return status;
   SE_CHECK_LAUNCH();
   return SE_OK;
@@ -809,13 +815,11 @@ __host__ __device__ constexpr int mid_shared_bytes(int mode, int mb) {
 }
 
 template <int MODE, int MB>   // MB row blocks of 16: tiles of 64 or 96 sorted rows
-__global__ void __launch_bounds__(64 * MID_WAVES, 2)
-grouped_gemm_mid_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
-                        bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
-                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ counters,
-                        const float* __restrict__ route_weight, int assignments, int top_k, int N,
-                        int K, int activation, int choice) {
-  if (choice >= 0 && counters[2] != choice) return;   // the device chose the other tile height (se_moe_align_choice)
+__device__ __forceinline__ void mid_tile(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                                         bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ counters,
+                                         const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                                         int K, int activation) {
   constexpr int BM = 16 * MB;
   constexpr int U = MID_KSTEP / 32;              // steps of 32 per stage
   constexpr int TILES = MB * U;                  // activation tiles (1 KB) of a stage
@@ -972,13 +976,81 @@ grouped_gemm_mid_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict_
   }
 }
 
+template <int MODE, int MB>
+__global__ void __launch_bounds__(64 * MID_WAVES, 2)
+grouped_gemm_mid_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                        bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ counters,
+                        const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                        int K, int activation) {
+  mid_tile<MODE, MB>(in, w, out, sorted, tile_expert, counters, route_weight, assignments, top_k, N, K, activation);
+}
+
+// The device's choice between the two (se_moe_align_choice leaves it in counters[2], with the sorted list in
+// tiles of the height that goes with it): tiles of 96 rows through the mid kernel's code, tiles of 128 through
+// the wide kernel's.  One launch serves both, since the host cannot know which it will be; both have blocks of
+// eight wavefronts, two to a CU, and the same output columns per block.
+#define CHOICE_MID_MB 6
+#define CHOICE_WIDE_BM 128
+template <int MODE>
+__global__ void __launch_bounds__(512, 2)
+grouped_gemm_choice_kernel(const bf16_t* __restrict__ in, const bf16_t* __restrict__ w,
+                           bf16_t* __restrict__ out, const int32_t* __restrict__ sorted,
+                           const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ counters,
+                           const float* __restrict__ route_weight, int assignments, int top_k, int N,
+                           int K, int activation) {
+  if (counters[2] == 0)    // the same in the whole grid
+    mid_tile<MODE, CHOICE_MID_MB>(in, w, out, sorted, tile_expert, counters, route_weight, assignments, top_k, N, K, activation);
+  else
+    wide_tile<MODE, CHOICE_WIDE_BM, WIDE_KSTEP>(in, w, out, sorted, tile_expert, counters, route_weight, assignments, top_k, N,
+                                                K, activation);
+}
+
+template <int MODE>
+static int launch_choice(const void* in, const void* w, void* out, const int32_t* sorted, const int32_t* tile_expert,
+                         const int32_t* counters, const float* route_weight, int assignments, int top_k, int N, int K,
+                         int max_tiles, int activation, hipStream_t stream) {
+  const int64_t items = static_cast<int64_t>(N / (MODE == 0 ? 128 : 256)) * max_tiles;
+  const int grid = static_cast<int>((items + 7) / 8 * 8);
+  constexpr size_t wide = WIDE_STAGES * (16 + CHOICE_WIDE_BM / 16) * (WIDE_KSTEP / 32) * 1024 + CHOICE_WIDE_BM * sizeof(int32_t);
+  constexpr size_t mid = mid_shared_bytes(MODE, CHOICE_MID_MB) + 16 * CHOICE_MID_MB * sizeof(int32_t);
+  constexpr size_t shared = wide > mid ? wide : mid;
+  static bool allowed = false;   // more than 64 KB of shared memory has to be asked for, once
+  if (!allowed) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_choice_kernel<MODE>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared)) != hipSuccess)
+      return SE_ERR_LAUNCH;
+    allowed = true;
+  }
+  grouped_gemm_choice_kernel<MODE><<<grid, 512, shared, stream>>>(
+      static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted,
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation);
+  return SE_OK;
+}
+
+// max_tiles: a bound for either tile height.  MODE 0 needs N % 128 == 0, MODE 1 N % 256 == 0; K % 64 == 0.
+extern "C" int se_grouped_gemm_choice(const void* in, const void* w, void* out, const int32_t* sorted,
+                                      const int32_t* tile_expert, const int32_t* counters,
+                                      const float* route_weight, int assignments, int top_k, int N,
+                                      int K, int max_tiles, int mode, int activation, hipStream_t stream) {
+  if (assignments <= 0) return SE_OK;
+  if (K <= 0 || K % 64 || N <= 0 || N % (mode == 0 ? 128 : 256)) return SE_ERR_SHAPE;
+  if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
+  if (max_tiles <= 0 || max_tiles > (1 << 22) || (mode != 0 && mode != 1)) return SE_ERR_SHAPE;
+  const int status = mode == 0 ? launch_choice<0>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
+                                                  top_k, N, K, max_tiles, activation, stream)
+                               : launch_choice<1>(in, w, out, sorted, tile_expert, counters, route_weight, assignments,
+                                                  top_k, N, K, max_tiles, activation, stream);
+  if (status != SE_OK) return status;
+  SE_CHECK_LAUNCH();
+  return SE_OK;
+}
+
 // tile_rows: 64 or 96.  MODE 0 needs N % 128 == 0, MODE 1 N % 256 == 0; K % 64 == 0.
-// `choice`: -1, or the value counters[2] must have for the launch to do anything (se_moe_align_choice).
 extern "C" int se_grouped_gemm_mid(const void* in, const void* w, void* out, const int32_t* sorted,
                                    const int32_t* tile_expert, const int32_t* counters,
                                    const float* route_weight, int assignments, int top_k, int N,
-                                   int K, int max_tiles, int mode, int tile_rows, int activation, int choice,
-                                   hipStream_t stream) {
+                                   int K, int max_tiles, int mode, int tile_rows, int activation, hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
   if (K <= 0 || K % MID_KSTEP || N <= 0 || N % (mode == 0 ? 128 : 256)) return SE_ERR_SHAPE;
   if (activation != SE_ACT_SILU && activation != SE_ACT_GELU_TANH) return SE_ERR_SHAPE;
@@ -990,7 +1062,7 @@ extern "C" int se_grouped_gemm_mid(const void* in, const void* w, void* out, con
   grouped_gemm_mid_kernel<MODE, MB><<<grid, 64 * MID_WAVES,                                        \
                                       mid_shared_bytes(MODE, MB) + 16 * MB * sizeof(int32_t), stream>>>( \
       static_cast<const bf16_t*>(in), static_cast<const bf16_t*>(w), static_cast<bf16_t*>(out), sorted, \
-      tile_expert, counters, route_weight, assignments, top_k, N, K, activation, choice)
+      tile_expert, counters, route_weight, assignments, top_k, N, K, activation)
   if (tile_rows == 64) { if (mode == 0) SE_MID(0, 4); else SE_MID(1, 4); }
   else { if (mode == 0) SE_MID(0, 6); else SE_MID(1, 6); }
 #undef SE_MID

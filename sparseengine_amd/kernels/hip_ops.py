@@ -112,9 +112,11 @@ _SIGNATURES = {
         "se_grouped_gemm_tall": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_wide": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "se_grouped_gemm_mid": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "se_grouped_gemm_choice": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "memory_probe": {
         "se_stream_read": [c_void_p, c_int64, c_void_p, c_int, c_void_p],
@@ -573,8 +575,8 @@ class HipKernels:
                                        "intermediate sizes in steps of 128")
             takes = "hidden and intermediate sizes in multiples of 128"
             if kernel == "auto":
-                # "mid" or "direct", chosen where the spread of the rows over the experts is known: on the device.
-                # Both pairs of launches are made; the pair that was not chosen leaves at once (4 us a layer).
+                # the code of "mid" or of "direct", chosen where the spread of the rows over the experts is known: on
+                # the device, by the kernel that groups the assignments; one launch holds both.
                 # Measured at MiniMax-M2 sizes with the rows spread evenly: 64 rows per expert 1245 (mid) against
                 # 1373 us (direct), 32 rows 1190 against 1290, 16 rows 1150 against 1250, 4 rows 1075 against 1164
                 # (the tall kernel, which this replaces); at 128 rows per expert, and whenever the tokens of a prompt
@@ -588,13 +590,12 @@ class HipKernels:
                 _check(_fn.get("moe", "se_moe_align_choice")(
                     _ptr(ids), assignments, experts, few_tile, many_tile, self.AUTO_FEW_ROWS, _ptr(ws.sorted),
                     _ptr(ws.tile_expert), _ptr(ws.counters), _stream()), "moe_align (choice)")
-                mid, wide = _fn.get("moe_mfma", "se_grouped_gemm_mid"), _fn.get("moe_mfma", "se_grouped_gemm_wide")
-                for mode, (src, w, dst, rw, n, k) in enumerate(((x, w13, ws.act, None, inter, hidden),
-                                                               (ws.act, w2, ws.slot_out, weights, hidden, inter))):
-                    for choice, (fn, rows) in enumerate(((mid, few_tile), (wide, many_tile))):
-                        _check(fn(_ptr(src), _ptr(w), _ptr(dst), _ptr(ws.sorted), _ptr(ws.tile_expert), _ptr(ws.counters),
-                                  _ptr(rw), assignments, top_k, n, k, max_tiles, mode, rows, act, choice, _stream()),
-                               f"moe {'down' if mode else 'gate-up'} ({'direct' if choice else 'mid'})", takes)
+                either = _fn.get("moe_mfma", "se_grouped_gemm_choice")
+                _check(either(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert), _ptr(ws.counters),
+                              None, assignments, top_k, inter, hidden, max_tiles, 0, act, _stream()), "moe gate-up (auto)", takes)
+                _check(either(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
+                              _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1, act,
+                              _stream()), "moe down (auto)", takes)
             else:
                 if tile_rows is None:
                     tile_rows = {"stream": 16, "tall": 64, "direct": 128 if share >= 16 else 64, "mid": 96}[kernel]
@@ -614,13 +615,12 @@ class HipKernels:
             elif kernel != "auto":
                 gt = _fn.get("moe_mfma", {"direct": "se_grouped_gemm_wide", "tall": "se_grouped_gemm_tall",
                                           "mid": "se_grouped_gemm_mid"}[kernel])
-                extra = () if kernel == "tall" else (-1,)      # no choice was made on the device: the launch runs
                 _check(gt(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), None, assignments, top_k, inter, hidden, max_tiles, 0, tile_rows,
-                          act, *extra, _stream()), f"moe gate-up ({kernel})", takes)
+                          act, _stream()), f"moe gate-up ({kernel})", takes)
                 _check(gt(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), _ptr(ws.sorted), _ptr(ws.tile_expert),
                           _ptr(ws.counters), _ptr(weights), assignments, top_k, hidden, inter, max_tiles, 1,
-                          tile_rows, act, *extra, _stream()), f"moe down ({kernel})", takes)
+                          tile_rows, act, _stream()), f"moe down ({kernel})", takes)
         else:
             _require(not tiled, "the general expert kernel reads row-major tables")
             max_tiles = self._grouped_tiles(ids, experts, ws, 16)

@@ -16,6 +16,7 @@ pytestmark = pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
 # kernels that may use scratch memory: (source, part of the mangled name) -> bytes per lane
 ALLOWED_SCRATCH = {
     ("moe_mfma", "grouped_gemm_mfma_kernelILi2ELi4ELi1ELi2ELi16E"): 64,       # dense product of 33..64 rows, K split 16 ways
+    ("moe_mfma", "grouped_gemm_mfma_kernelILi3ELi4ELi1ELi2ELi16E"): 64,       # the same on a tiled copy of the matrix
     # prompt attention at head size 128 on pages that are no multiple of 32 keys: the lanes' own page
     # counters on top of a loop that fills the register file (two or three registers, outside the loop's core)
     ("attention_mfma", "paged_attention_tiled_kernelILi4ELi2ELi4ELb0E"): 16,
