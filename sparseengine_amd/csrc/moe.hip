@@ -181,14 +181,17 @@ router_logits_kernel(const T* __restrict__ x, int64_t x_stride, const float* __r
 // computed independently of its neighbours, so results do not depend on it.
 // ---------------------------------------------------------------------------------------- //
 // The work of one block of 64 ... 1024 threads (a multiple of 64); sh holds 3 * experts + 1 ints.
-// `other_rows` > 0: the tile height is chosen here, where the counts are known: `tile_rows` if the experts
-// that got any rows got at most `few_rows` on average, else `other_rows`; counters[2] says which (0 / 1),
-// and the kernels made for the other height leave at once.
+// `other_rows` > 0: the tile height is chosen here, where the counts are known, between `tile_rows` (the kernel
+// that streams an expert's table once per tile) and `other_rows` (the kernel that shares a table among many rows):
+// with t tiles of `tile_rows` the former reads t tables; the latter reads one table per expert that got rows,
+// or, when the rows are many, is bound by its arithmetic, which takes as long as reading a table per
+// `heavy_rows` rows.  The former is chosen if t * percent / 100 is at most the larger of the two (percent: how
+// much faster it reads).  counters[2] says which (0 / 1); the launch that follows holds both kernels' code.
 __device__ __forceinline__ void align_assignments(const int32_t* __restrict__ ids, int assignments,
                                                   int experts, int tile_rows, int32_t* __restrict__ sorted,
                                                   int32_t* __restrict__ tile_expert,
                                                   int32_t* __restrict__ counters, int32_t* sh,
-                                                  int other_rows = 0, int few_rows = 0) {
+                                                  int other_rows = 0, int percent = 0, int heavy_rows = 1) {
   int32_t* counts = sh;                 // [experts]
   int32_t* offsets = sh + experts;      // [experts + 1] start of each run in `sorted`
   int32_t* cursor = offsets + experts + 1;  // [experts]
@@ -209,14 +212,21 @@ __device__ __forceinline__ void align_assignments(const int32_t* __restrict__ id
   }
   __syncthreads();
   if (other_rows > 0) {
-    __shared__ int32_t touched;
-    if (threadIdx.x == 0) touched = 0;
+    __shared__ int32_t touched, tiles;
+    if (threadIdx.x == 0) touched = tiles = 0;
     __syncthreads();
-    int32_t mine = 0;
-    for (int e = threadIdx.x; e < experts; e += blockDim.x) mine += counts[e] > 0;
-    if (mine) atomicAdd(&touched, mine);
+    int32_t mine = 0, my_tiles = 0;
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+      mine += counts[e] > 0;
+      my_tiles += (counts[e] + tile_rows - 1) / tile_rows;
+    }
+    if (mine) {
+      atomicAdd(&touched, mine);
+      atomicAdd(&tiles, my_tiles);
+    }
     __syncthreads();
-    const bool few = static_cast<int64_t>(assignments) <= static_cast<int64_t>(few_rows) * touched;
+    const int64_t tables = max(touched, assignments / heavy_rows);
+    const bool few = static_cast<int64_t>(tiles) * percent <= 100 * tables;
     if (!few) tile_rows = other_rows;
     if (threadIdx.x == 0) counters[2] = few ? 0 : 1;
   }
@@ -298,9 +308,10 @@ __device__ __forceinline__ void align_assignments(const int32_t* __restrict__ id
 __global__ void moe_align_kernel(const int32_t* __restrict__ ids, int assignments, int experts,
                                  int tile_rows, int32_t* __restrict__ sorted,
                                  int32_t* __restrict__ tile_expert, int32_t* __restrict__ counters,
-                                 int other_rows, int few_rows) {
+                                 int other_rows, int percent, int heavy_rows) {
   extern __shared__ int32_t sh[];
-  align_assignments(ids, assignments, experts, tile_rows, sorted, tile_expert, counters, sh, other_rows, few_rows);
+  align_assignments(ids, assignments, experts, tile_rows, sorted, tile_expert, counters, sh, other_rows, percent,
+                    heavy_rows);
 }
 
 // A step with few tokens (at most 16): one block routes them, a wavefront each, and then groups
@@ -537,23 +548,24 @@ int se_moe_align(const int32_t* ids, int assignments, int experts, int tile_rows
   if (experts <= 0 || experts > 4096 || tile_rows <= 0) return SE_ERR_SHAPE;
   const size_t shmem = (3 * static_cast<size_t>(experts) + 1) * sizeof(int32_t);
   moe_align_kernel<<<1, 1024, shmem, stream>>>(ids, assignments, experts, tile_rows, sorted,
-                                               tile_expert, counters, 0, 0);
+                                               tile_expert, counters, 0, 0, 1);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }
 
-// The same with the tile height chosen on the device, where the counts are: tiles of `few_tile_rows` if the
-// experts that got rows got at most `few_rows` each on average, else of `many_tile_rows`; counters[2] = 0 / 1.
-// (The host knows how many tokens a step has, not how they spread over the experts: a prompt whose tokens
-// agree on a few dozen experts and one that uses them all want different kernels.)
+// The same with the tile height chosen on the device, where the counts are (see align_assignments): tiles of
+// `few_tile_rows` or of `many_tile_rows`; counters[2] = 0 / 1.  (The host knows how many tokens a step has, not
+// how they spread over the experts: a prompt whose tokens agree on a few dozen experts and one that uses them all
+// want different kernels.)
 int se_moe_align_choice(const int32_t* ids, int assignments, int experts, int few_tile_rows, int many_tile_rows,
-                        int few_rows, int32_t* sorted, int32_t* tile_expert, int32_t* counters,
+                        int percent, int heavy_rows, int32_t* sorted, int32_t* tile_expert, int32_t* counters,
                         hipStream_t stream) {
   if (assignments <= 0) return SE_OK;
-  if (experts <= 0 || experts > 4096 || few_tile_rows <= 0 || many_tile_rows <= 0 || few_rows <= 0) return SE_ERR_SHAPE;
+  if (experts <= 0 || experts > 4096 || few_tile_rows <= 0 || many_tile_rows <= 0 || percent <= 0 || heavy_rows <= 0)
+    return SE_ERR_SHAPE;
   const size_t shmem = (3 * static_cast<size_t>(experts) + 1) * sizeof(int32_t);
   moe_align_kernel<<<1, 1024, shmem, stream>>>(ids, assignments, experts, few_tile_rows, sorted,
-                                               tile_expert, counters, many_tile_rows, few_rows);
+                                               tile_expert, counters, many_tile_rows, percent, heavy_rows);
   SE_CHECK_LAUNCH();
   return SE_OK;
 }

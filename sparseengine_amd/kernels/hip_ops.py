@@ -98,7 +98,7 @@ _SIGNATURES = {
         "se_router_topk_align": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                  c_int, c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_moe_align": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
-        "se_moe_align_choice": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+        "se_moe_align_choice": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
         "se_grouped_gemm_generic": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_void_p],
@@ -510,10 +510,13 @@ class HipKernels:
         return True
 
     ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}      # what a gated feed-forward applies to its gate
-    # the device's choice between the mid kernel (tiles of 96 rows) and the wide one (tiles of 128): mid if the
-    # experts that got rows got at most this many on average (with 72, hardly one of them overflows a tile of 96)
+    # The device's choice between the mid kernel (tiles of 96 rows) and the wide one (tiles of 128).  The mid kernel
+    # reads an expert's table once per tile, at 6.3 TB/s; the wide one reads it once (5.3 TB/s), or is bound by its
+    # arithmetic, about 0.8 PFLOP/s, which is the time of reading one table per 151 rows.  Mid is chosen if its
+    # tiles, times 84 %, are at most the larger of the experts that got rows and the rows / 151.
     AUTO_TILE_ROWS = (96, 128)
-    AUTO_FEW_ROWS = 72
+    AUTO_READ_PERCENT = 84
+    AUTO_HEAVY_ROWS = 151
 
     def _activation(self, name: str) -> int:
         if name not in self.ACTIVATIONS:
@@ -588,7 +591,8 @@ class HipKernels:
                     raise KernelShapeError("moe: too many tokens in one call; lower mlp_chunk_size")
                 ws.grouped = None
                 _check(_fn.get("moe", "se_moe_align_choice")(
-                    _ptr(ids), assignments, experts, few_tile, many_tile, self.AUTO_FEW_ROWS, _ptr(ws.sorted),
+                    _ptr(ids), assignments, experts, few_tile, many_tile, self.AUTO_READ_PERCENT, self.AUTO_HEAVY_ROWS,
+                    _ptr(ws.sorted),
                     _ptr(ws.tile_expert), _ptr(ws.counters), _stream()), "moe_align (choice)")
                 either = _fn.get("moe_mfma", "se_grouped_gemm_choice")
                 _check(either(_ptr(x), _ptr(w13), _ptr(ws.act), _ptr(ws.sorted), _ptr(ws.tile_expert), _ptr(ws.counters),

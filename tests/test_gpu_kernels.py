@@ -1046,10 +1046,10 @@ def test_experts_on_random_shapes_and_lumpy_routing(hip, twin):
 
 
 def test_the_device_chooses_the_expert_kernel_by_the_spread_of_the_rows(hip, twin):
-    """"auto": the grouping kernel counts the experts that got rows and chooses tiles of 96 rows (the mid kernel)
-    if they got at most 72 each on average, else tiles of 128 (the wide kernel); the launches of the other kernel
-    leave at once.  The same tokens spread evenly and crowded onto two experts: the choice differs, the results
-    are the twin's both times."""
+    """"auto": the grouping kernel counts the experts that got rows and the tiles of 96 rows they fill, and chooses
+    those tiles (the mid kernel's code) if reading a table per tile is less than what the wide kernel has to do
+    (a table per expert, or its arithmetic), else tiles of 128.  The same tokens spread evenly and crowded onto
+    two experts: the choice differs, the results are the twin's both times."""
     from sparseengine_amd.kernels.hip_ops import MoeWorkspace
     tokens, hidden, inter, experts, k = 400, 256, 128, 16, 2
     emulator_skips(tokens * k * hidden * inter, 1.2e8)
