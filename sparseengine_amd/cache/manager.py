@@ -57,21 +57,18 @@ class StepAllocation:
 
 class CacheManager:
     def __init__(self, requests: dict[int, object], *, max_rows: int, max_model_len: int,
-                 page_size: int, num_pages: int | dict | None, dtype: torch.dtype, device,
-                 allocate_tensors: bool = True):
+                 page_size: int, num_pages: int | dict | None = None, num_tokens: int | None = None,
+                 dtype: torch.dtype, device, allocate_tensors: bool = True):
         """``requests``: schedule position -> PagedKVRequest | StateRequest (positions that read
-        another position's cache are not listed).  ``num_pages``: pages of every group's pool
-        (an int for all groups or {group index: pages})."""
+        another position's cache are not listed).  ``page_size``: tokens per page of the groups whose
+        request names none.  The pools' sizes: ``num_tokens`` (every group gets the pages that hold so
+        many tokens) or ``num_pages`` (an int for all groups or {group index: pages})."""
         if page_size <= 0 or max_rows <= 0 or max_model_len <= 0:
             raise ValueError("page_size, max_rows and max_model_len must be positive")
-        if page_size % 8:
-            raise ValueError(f"page_size must be a multiple of 8 (a page keeps its elements in groups of "
-                             f"eight, cache/layout.py), got {page_size}")
-        self.page_size = int(page_size)
+        self.page_size = int(page_size)          # the default; a group's own is ``group.page_size``
         self.max_rows = int(max_rows)
         self.max_model_len = int(max_model_len)
         self.dtype, self.device = dtype, device
-        self.max_pages_per_row = -(-self.max_model_len // self.page_size)
 
         by_geometry: dict[PagedKVRequest, list[int]] = {}
         self.state_positions: dict[int, StateRequest] = {}
@@ -85,16 +82,23 @@ class CacheManager:
         self.groups: list[KVGroup] = []
         self.group_of_position: dict[int, int] = {}
         for index, (req, positions) in enumerate(by_geometry.items()):
-            pages = num_pages[index] if isinstance(num_pages, dict) else num_pages
+            ps = int(req.page_size or self.page_size)
+            if ps <= 0 or ps % 8:
+                raise ValueError(f"a cache page holds a multiple of 8 tokens (it keeps its elements in groups of "
+                                 f"eight, cache/layout.py), got {ps}")
+            if num_tokens is not None:
+                pages = max(1, -(-int(num_tokens) // ps))      # a last page may be partly beyond the count
+            else:
+                pages = num_pages[index] if isinstance(num_pages, dict) else num_pages
             if pages is None:
-                raise ValueError("num_pages must be given")
-            group = KVGroup(index, req, positions, self.page_size, PagePool(int(pages)),
-                            np.full((self.max_rows, self.max_pages_per_row), -1, dtype=np.int32),
+                raise ValueError("num_pages or num_tokens must be given")
+            group = KVGroup(index, req, positions, ps, PagePool(int(pages)),
+                            np.full((self.max_rows, -(-self.max_model_len // ps)), -1, dtype=np.int32),
                             np.zeros(self.max_rows, dtype=np.int64))
             if allocate_tensors:
                 for position in positions:
                     group.layers[position] = torch.zeros(
-                        int(pages), 2, req.kv_heads, self.page_size, req.head_dim, dtype=dtype, device=device)
+                        int(pages), 2, req.kv_heads, ps, req.head_dim, dtype=dtype, device=device)
             self.groups.append(group)
             for position in positions:
                 self.group_of_position[position] = index
@@ -156,7 +160,7 @@ class CacheManager:
     # ------------------------------------------------------------------ capacity questions
     def _plan(self, group: KVGroup, row: int, new_tokens: int, length: int | None = None):
         """(pages to release first, pages to allocate) for appending ``new_tokens`` to the row."""
-        ps = self.page_size
+        ps = group.page_size
         length = int(self.row_len[row]) if length is None else length
         have_until = -(-length // ps)                       # pages [first_live, have_until) are held
         need_until = -(-(length + new_tokens) // ps)
@@ -174,8 +178,9 @@ class CacheManager:
             out[group.index] = alloc - (release_until - int(group.first_live[row]))
         return out
 
-    def pages_for_tokens(self, tokens: int) -> int:
-        return -(-int(tokens) // self.page_size)
+    def pages_for_tokens(self, tokens: int) -> dict[int, int]:
+        """Pages of every group that a request of ``tokens`` tokens takes from an empty row."""
+        return {g.index: -(-int(tokens) // g.page_size) for g in self.groups}
 
     def free_pages(self) -> dict[int, int]:
         return {g.index: g.pool.free_count for g in self.groups}
@@ -210,9 +215,9 @@ class CacheManager:
         if not self.can_append(items):
             raise OutOfPages(f"step of {sum(n for _, n in items)} tokens does not fit: free pages "
                              f"{self.free_pages()}")
-        ps = self.page_size
         slots = {g.index: np.empty(sum(n for _, n in items), dtype=np.int32) for g in self.groups}
         for group in self.groups:
+            ps = group.page_size
             # every release of the step comes before its first allocation: the check above
             # counted the pages that this step itself gives back
             for row, n in items:
@@ -241,8 +246,8 @@ class CacheManager:
         """Forget the tokens beyond ``length`` (undo of an append whose step failed)."""
         if length > self.row_len[row]:
             raise ValueError("truncate cannot lengthen a row")
-        ps = self.page_size
         for group in self.groups:
+            ps = group.page_size
             keep_until = -(-length // ps)
             have_until = -(-int(self.row_len[row]) // ps)
             first = max(int(group.first_live[row]), keep_until)
@@ -261,13 +266,13 @@ class CacheManager:
 
     # ------------------------------------------------------------------ invariants
     def check_invariants(self) -> None:
-        ps = self.page_size
         held_rows = set(self._row_of.values())
         if len(held_rows) != len(self._row_of) or held_rows & set(self._free_rows):
             raise PageOwnershipError("a row is held twice or is both held and free")
         if len(held_rows) + len(self._free_rows) != self.max_rows:
             raise PageOwnershipError("a row was lost")
         for group in self.groups:
+            ps = group.page_size
             group.pool.check()
             seen: dict[int, int] = {}
             for row in range(self.max_rows):

@@ -46,6 +46,7 @@ class AttentionSpec:
     qk_norm_eps: float = 1e-6
     window: int | None = None       # keys further back than this are not read (None: all keys)
     position: Any = field(default_factory=NoPositionSpec)
+    kv_page_size: int | None = None  # tokens per cache page of this layer's group (None: the engine's)
 
 
 @dataclass(frozen=True)

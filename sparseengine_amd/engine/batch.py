@@ -181,7 +181,7 @@ class BatchBuilder:
 
         tables = {}
         for group in cache.groups:
-            width = max(1, -(-int(ctx_len.max()) // cache.page_size))
+            width = max(1, -(-int(ctx_len.max()) // group.page_size))
             tables[group.index] = np.ascontiguousarray(group.table[rows, :width])
 
         item_meta_host = np.stack([q_start, q_len, ctx_len]).astype(np.int32)      # one part: [3, items]
@@ -228,7 +228,7 @@ class BatchBuilder:
                 block_table=view(6 + 2 * gi + 1, tables[group.index].shape),
                 block_table_host=tables[group.index],
                 token_row=fb.token_item, positions=fb.positions, slots=view(6 + 2 * gi),
-                page_size=cache.page_size, item_q_start=q_start, item_q_len=q_len,
+                page_size=group.page_size, item_q_start=q_start, item_q_len=q_len,
                 item_ctx_len=ctx_len, item_meta=item_meta, max_ctx_len=int(ctx_len.max()),
                 max_q_len=int(q_len.max()))
         for group_index, key, work, at in works:

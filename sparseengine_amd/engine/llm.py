@@ -24,41 +24,44 @@ from .sequence import Sequence
 
 
 class CacheOracle(MemoryOracle):
-    """The scheduler's view of the cache manager, in pages of the tightest group."""
+    """The scheduler's view of the cache manager, in tokens of cache (whole pages of the tightest group)."""
 
     def __init__(self, cache, method=None):
         self.cache = cache
         self.method = method
 
-    def free_pages(self):
-        return min(g.pool.free_count for g in self.cache.groups) if self.cache.groups else 1 << 30
+    def free_tokens(self):
+        return min((g.pool.free_count * g.page_size for g in self.cache.groups), default=1 << 40)
 
-    def total_pages(self):
-        return min(g.pool.num_pages for g in self.cache.groups) if self.cache.groups else 1 << 30
+    def total_tokens(self):
+        return min((g.pool.num_pages * g.page_size for g in self.cache.groups), default=1 << 40)
 
     def free_rows(self):
         return self.cache.num_free_rows
 
-    def pages_for_tokens(self, tokens):
-        return self.cache.pages_for_tokens(tokens)
+    def _cost(self, pages: dict[int, int], row, new_tokens) -> int:
+        if self.method is not None:       # what the sparse method keeps for itself on top
+            for group, extra in self.method.extra_pages(row, new_tokens).items():
+                pages[group] = pages.get(group, 0) + extra
+        sizes = {g.index: g.page_size for g in self.cache.groups}
+        return max((n * sizes[group] for group, n in pages.items()), default=0)
 
-    def pages_to_append(self, seq_id, new_tokens):
+    def cost_of_new(self, tokens):
+        return self._cost(self.cache.pages_for_tokens(tokens), None, tokens)
+
+    def cost_to_append(self, seq_id, new_tokens):
         if new_tokens <= 0:
             return 0
-        row = self.cache.row_of(seq_id) if self.cache.has_row(seq_id) else None
-        if row is None:
-            needed = {g.index: self.cache.pages_for_tokens(new_tokens) for g in self.cache.groups}
-        else:
-            needed = self.cache.pages_needed(row, new_tokens)
-        if self.method is not None:       # what the sparse method keeps for itself on top
-            for group, pages in self.method.extra_pages(row, new_tokens).items():
-                needed[group] = needed.get(group, 0) + pages
-        return max(needed.values()) if needed else 0
+        if not self.cache.has_row(seq_id):
+            return self.cost_of_new(new_tokens)
+        row = self.cache.row_of(seq_id)
+        return self._cost(self.cache.pages_needed(row, new_tokens), row, new_tokens)
 
-    def tokens_that_fit(self, seq_id, pages):
-        ps = self.cache.page_size
+    def tokens_that_fit(self, seq_id, room):
         length = int(self.cache.row_len[self.cache.row_of(seq_id)]) if self.cache.has_row(seq_id) else 0
-        return (-length) % ps + max(0, pages) * ps
+        # per group: what is left of the row's last page, and the whole pages that the room holds
+        return min(((-length) % g.page_size + max(0, room) // g.page_size * g.page_size for g in self.cache.groups),
+                   default=1 << 40)
 
     def admit(self, seq_id):
         self.cache.admit(seq_id)

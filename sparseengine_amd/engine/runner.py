@@ -102,10 +102,10 @@ class ModelRunner:
         requests = self.model.cache_requests()
         if num_kvcache_tokens is None or int(num_kvcache_tokens) <= 0:
             num_kvcache_tokens = self.derive_cache_tokens(requests, max_num_seqs, gpu_memory_utilization)
-        num_pages = max(1, -(-int(num_kvcache_tokens) // self.kv_page_size))      # a last page may be partly beyond the count
         self.cache = (cache_manager_cls or CacheManager)(requests, max_rows=max_num_seqs,
-                                  max_model_len=self.max_model_len, page_size=self.kv_page_size,
-                                  num_pages=num_pages, dtype=self.dtype, device=self.device)
+                                                         max_model_len=self.max_model_len, page_size=self.kv_page_size,
+                                                         num_tokens=int(num_kvcache_tokens), dtype=self.dtype,
+                                                         device=self.device)
         shapes = {}
         if getattr(kernels, "libraries", None):
             for position in requests:
@@ -133,7 +133,8 @@ class ModelRunner:
             return cap
         free, total = torch.cuda.mem_get_info(self.device)
         usable = free - int((1.0 - utilization) * total) - (2 << 30)      # 2 GiB kept for step buffers
-        if usable <= per_token * self.kv_page_size:
+        if usable <= per_token * max([self.kv_page_size] + [r.page_size or 0 for r in requests.values()
+                                                            if isinstance(r, PagedKVRequest)]):
             raise RuntimeError("no GPU memory is left for the cache after the weights")
         return min(cap, usable // per_token)
 
@@ -185,8 +186,8 @@ class ModelRunner:
                     need[gi] += pages
             else:
                 new_rows += 1
-                for gi in need:
-                    need[gi] += self.cache.pages_for_tokens(n)
+                for gi, pages in self.cache.pages_for_tokens(n).items():
+                    need[gi] += pages
             for gi, pages in self.method.extra_pages(row, n).items():
                 need[gi] += pages
         free = self.cache.free_pages()

@@ -26,14 +26,17 @@ from .sequence import Sequence, SequenceStatus
 
 
 class MemoryOracle:
-    """What the scheduler asks of the cache.  Counts are pages of the tightest group."""
+    """What the scheduler asks of the cache.  Every count is in tokens of cache, taken in whole pages: the
+    cache's groups may have pages of different sizes, so pages are no common unit; an answer is that of the
+    group for which it is tightest (what is free: the least; what something costs: the most), which makes
+    the sum of several costs an upper bound for every group."""
 
-    def free_pages(self) -> int: raise NotImplementedError
-    def total_pages(self) -> int: raise NotImplementedError
+    def free_tokens(self) -> int: raise NotImplementedError
+    def total_tokens(self) -> int: raise NotImplementedError
     def free_rows(self) -> int: raise NotImplementedError
-    def pages_for_tokens(self, tokens: int) -> int: raise NotImplementedError
-    def pages_to_append(self, seq_id, new_tokens: int) -> int: raise NotImplementedError
-    def tokens_that_fit(self, seq_id, pages: int) -> int: raise NotImplementedError
+    def cost_of_new(self, tokens: int) -> int: raise NotImplementedError              # a request of so many tokens, from nothing
+    def cost_to_append(self, seq_id, new_tokens: int) -> int: raise NotImplementedError
+    def tokens_that_fit(self, seq_id, room: int) -> int: raise NotImplementedError     # new tokens of the request that `room` holds
     def admit(self, seq_id) -> None: raise NotImplementedError
     def holds(self, seq_id) -> bool: raise NotImplementedError
     def release(self, seq_id) -> None: raise NotImplementedError
@@ -101,8 +104,8 @@ class Scheduler:
         return max(0, min(self.decode_reservation_tokens, seq.tokens_left_to_generate()))
 
     def _promised(self, seq: Sequence) -> int:
-        """Pages a running request may still take: the rest of its known tokens + its decode window."""
-        return self.oracle.pages_to_append(seq.seq_id, seq.num_remaining_tokens + self._window(seq))
+        """Cache a running request may still take: the rest of its known tokens + its decode window."""
+        return self.oracle.cost_to_append(seq.seq_id, seq.num_remaining_tokens + self._window(seq))
 
     def _preempt(self, victim: Sequence, schedule: Schedule) -> None:
         self.running.remove(victim)
@@ -120,17 +123,17 @@ class Scheduler:
         schedule = Schedule()
         oracle = self.oracle
         budget = self.max_num_batched_tokens
-        taken = 0                                  # pages this step's items will take
+        taken = 0                                  # cache this step's items will take
 
         def room() -> int:
-            return oracle.free_pages() - taken
+            return oracle.free_tokens() - taken
 
         # 1. every decoding request feeds its last token
         decoders = [s for s in self.running if s.num_remaining_tokens == 1][:min(self.max_decoding_seqs, self.max_num_seqs_in_batch)]
         for seq in decoders:
             if seq not in self.running:            # preempted a moment ago
                 continue
-            need = oracle.pages_to_append(seq.seq_id, 1)
+            need = oracle.cost_to_append(seq.seq_id, 1)
             while need > room():
                 scheduled = {i.seq.seq_id for i in schedule.items}
                 victims = [s for s in self.running if s.seq_id not in scheduled and s is not seq]
@@ -142,8 +145,8 @@ class Scheduler:
                     break
                 raise RuntimeError(
                     "KV cache is too small for the only running request to go on: "
-                    f"seq_id={seq.seq_id} tokens={seq.num_tokens} free_pages={oracle.free_pages()} "
-                    f"total_pages={oracle.total_pages()}; recomputing it would end in the same place")
+                    f"seq_id={seq.seq_id} tokens={seq.num_tokens} free cache tokens={oracle.free_tokens()} "
+                    f"of {oracle.total_tokens()}; recomputing it would end in the same place")
             if seq not in self.running:
                 continue
             taken += need
@@ -157,7 +160,7 @@ class Scheduler:
             n = min(n, oracle.tokens_that_fit(seq.seq_id, room()))
             if n <= 0:
                 return False
-            taken += oracle.pages_to_append(seq.seq_id, n)
+            taken += oracle.cost_to_append(seq.seq_id, n)
             budget -= n
             schedule.items.append(ScheduledItem(seq, n, n == seq.num_remaining_tokens))
             return True
@@ -175,15 +178,15 @@ class Scheduler:
             seq = self.waiting[0]
             if len(self.running) >= self.max_decoding_seqs or oracle.free_rows() <= 0:
                 break
-            need = oracle.pages_for_tokens(seq.num_tokens + self._window(seq))
-            if need > oracle.total_pages():
+            need = oracle.cost_of_new(seq.num_tokens + self._window(seq))
+            if need > oracle.total_tokens():
                 if not self.running:
                     raise ValueError(
-                        f"request {seq.seq_id} needs {need} pages for {seq.num_tokens} tokens and its "
-                        f"decode window; the cache has {oracle.total_pages()}")
+                        f"request {seq.seq_id} needs cache for {need} tokens ({seq.num_tokens} tokens and its "
+                        f"decode window, in whole pages); the cache holds {oracle.total_tokens()}")
                 break
             promised = sum(self._promised(s) for s in self.running)
-            if need + promised > oracle.free_pages():
+            if need + promised > oracle.free_tokens():
                 break                                            # deferred: stays at the head
             self.waiting.popleft()
             oracle.admit(seq.seq_id)
@@ -195,7 +198,7 @@ class Scheduler:
         if not schedule.items and not schedule.preempted and not self.is_finished():
             raise RuntimeError(
                 f"nothing can run: {len(self.waiting)} waiting, {len(self.running)} running, "
-                f"{oracle.free_pages()} of {oracle.total_pages()} pages free")
+                f"{oracle.free_tokens()} of {oracle.total_tokens()} cache tokens free")
         return schedule
 
     # ------------------------------------------------------------------ after the step

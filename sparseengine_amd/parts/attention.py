@@ -58,7 +58,7 @@ class GQAAttention(Part):
         return self.spec.num_heads // self.spec.num_kv_heads, int(self.spec.window or 0)
 
     def cache_request(self):
-        return PagedKVRequest(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
+        return PagedKVRequest(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window, self.spec.kv_page_size)
 
     def forward(self, fb, x, cache_position: int, write_cache: bool = True):
         s, p, T = self.spec, self.params, x.shape[0]

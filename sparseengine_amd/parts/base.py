@@ -29,10 +29,12 @@ class ParamDecl:
 
 @dataclass(frozen=True)
 class PagedKVRequest:
-    """A mixer that keeps keys and values of ``window`` (None: all) past tokens in pages."""
+    """A mixer that keeps keys and values of ``window`` (None: all) past tokens in pages of ``page_size``
+    tokens (None: the engine's ``kv_page_size``).  Positions whose requests are equal share a pool."""
     kv_heads: int
     head_dim: int
     window: int | None = None
+    page_size: int | None = None
 
 
 @dataclass(frozen=True)

@@ -110,12 +110,51 @@ def test_state_slots_are_zeroed_on_admission():
     assert m.state[1]["s"].shape == (4, 3, 2) and m.state[1]["count"].dtype == torch.int32
 
 
-@pytest.mark.parametrize("seed", range(6))
+def test_groups_may_have_pages_of_different_sizes_and_the_oracle_counts_tokens():
+    """A group's request may name its own page size; tables, slots and window release follow it, and the
+    scheduler's oracle answers in tokens of cache (whole pages of the tightest group), pages being no
+    common unit."""
+    from sparseengine_amd.engine.llm import CacheOracle
+    small = PagedKVRequest(2, 16, 40, page_size=8)
+    m = CacheManager({0: FULL, 1: small}, max_rows=3, max_model_len=256, page_size=32, num_tokens=192,
+                     dtype=torch.float32, device="cpu", allocate_tensors=True)
+    full, windowed = m.groups
+    assert (full.page_size, windowed.page_size) == (32, 8) and (full.pool.num_pages, windowed.pool.num_pages) == (6, 24)
+    assert m.kv_layer(0).shape == (6, 2, 2, 32, 16) and m.kv_layer(1).shape == (24, 2, 2, 8, 16)
+    assert full.table.shape[1] == 8 and windowed.table.shape[1] == 32
+    oracle = CacheOracle(m)
+    assert oracle.free_tokens() == 192 and oracle.total_tokens() == 192
+    assert oracle.cost_of_new(33) == 64 and oracle.cost_of_new(5) == 32          # the pages of 32 are the tighter ones
+    row = m.admit("a")
+    alloc = m.append([(row, 37)])
+    assert alloc.slots[0][36] == full.table[row, 1] * 32 + 4 and alloc.slots[1][36] == windowed.table[row, 4] * 8 + 4
+    assert oracle.free_tokens() == min(4 * 32, 19 * 8) == 128
+    assert oracle.cost_to_append("a", 27) == 24 and oracle.cost_to_append("a", 28) == 32    # three pages of 8; one of 32
+    assert oracle.tokens_that_fit("a", 40) == 3 + 40        # the rest of the last page of 8, and five more
+    assert oracle.tokens_that_fit("a", 8) == 3 + 8
+    for _ in range(7):                                       # through the window of 40: the small pages come back
+        m.append([(row, 20)])
+        m.check_invariants()
+    # 177 tokens: all six pages of 32; the last step's first query sat at 157 and read the keys from 118 on
+    assert int(m.row_len[row]) == 177 and full.pool.free_count == 0
+    assert int(windowed.first_live[row]) == 118 // 8 and windowed.pool.free_count == 24 - (23 - 14)
+    assert oracle.free_tokens() == 0 and oracle.cost_to_append("a", 15) == 0 and oracle.cost_to_append("a", 16) == 32
+    m.free("a")
+    assert oracle.free_tokens() == 192
+    with pytest.raises(ValueError, match="multiple of 8"):
+        CacheManager({0: PagedKVRequest(2, 16, None, page_size=12)}, max_rows=1, max_model_len=64, page_size=16,
+                     num_tokens=64, dtype=torch.float32, device="cpu", allocate_tensors=False)
+
+
+@pytest.mark.parametrize("seed", range(8))
 def test_random_orders_keep_every_page_accounted_for(seed):
     rng = random.Random(seed)
     windowed = seed % 2 == 1
-    requests = {0: FULL, 1: WINDOW if windowed else FULL, 2: StateRequest((("h", (4,), None),))}
-    m = manager(requests, pages={0: 24, 1: 9} if windowed else 24, rows=5, max_len=200, tensors=False)
+    second = (PagedKVRequest(2, 16, 40, page_size=8) if seed >= 6 else WINDOW) if windowed else \
+        (PagedKVRequest(2, 16, None, page_size=32) if seed >= 6 else FULL)
+    requests = {0: FULL, 1: second, 2: StateRequest((("h", (4,), None),))}
+    m = manager(requests, pages={0: 24, 1: 9 if seed < 6 else 18} if len({FULL, second}) > 1 else 24, rows=5, max_len=200,
+                tensors=False)
     live, next_id, reference = {}, 0, {}
     for _ in range(600):
         action = rng.random()

@@ -438,4 +438,4 @@ def run_toy_architecture(tmp_path, dtype, lengths):
         assert_close_to_plain(dtype, got[rid], ref, f"toy architecture, request {rid}", layers=len(TOY_CONFIG["schedule"]))
     assert all(g.pool.free_count == g.pool.num_pages for g in runner.cache.groups)
     windowed = runner.cache.groups[1]
-    assert windowed.pool.num_pages >= 4      # and a window of 24 never held more than 4 pages of 16 per request
+    assert windowed.window == 24 and windowed.page_size == 8 and runner.cache.groups[0].page_size == 16   # pages of its own size

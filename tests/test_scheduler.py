@@ -17,15 +17,16 @@ class FakeCache(MemoryOracle):
     def used(self):
         return sum(-(-n // self.page) for n in self.held.values())
 
-    def free_pages(self): return self.pages - self.used()
-    def total_pages(self): return self.pages
+    # the scheduler's unit is tokens of cache in whole pages
+    def free_tokens(self): return (self.pages - self.used()) * self.page
+    def total_tokens(self): return self.pages * self.page
     def free_rows(self): return self.rows - len(self.held)
-    def pages_for_tokens(self, tokens): return -(-tokens // self.page)
-    def pages_to_append(self, seq_id, n):
+    def cost_of_new(self, tokens): return -(-tokens // self.page) * self.page
+    def cost_to_append(self, seq_id, n):
         have = self.held.get(seq_id, 0)
-        return -(-(have + n) // self.page) - -(-have // self.page)
-    def tokens_that_fit(self, seq_id, pages):
-        return (-self.held.get(seq_id, 0)) % self.page + max(0, pages) * self.page
+        return (-(-(have + n) // self.page) - -(-have // self.page)) * self.page
+    def tokens_that_fit(self, seq_id, room):
+        return (-self.held.get(seq_id, 0)) % self.page + max(0, room) // self.page * self.page
     def admit(self, seq_id): self.held[seq_id] = 0
     def holds(self, seq_id): return seq_id in self.held
     def release(self, seq_id): del self.held[seq_id]
@@ -46,7 +47,7 @@ def run_step(sched, cache, token=lambda s: 7):
     """The engine's step with a fake model: appends to the fake cache, 'samples' a token."""
     schedule = sched.schedule()
     for item in schedule.items:
-        assert cache.pages_to_append(item.seq.seq_id, item.num_tokens) <= cache.free_pages()
+        assert cache.cost_to_append(item.seq.seq_id, item.num_tokens) <= cache.free_tokens()
         cache.held[item.seq.seq_id] += item.num_tokens
     sampled = {i.seq.seq_id: token(i.seq) for i in schedule.items if i.wants_logits}
     return schedule, sched.postprocess(schedule, sampled)

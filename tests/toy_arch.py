@@ -268,7 +268,8 @@ def _layer_spec(cfg, layer) -> LayerSpec:
             rotary = NoPositionSpec()
         mixer = AttentionSpec(num_heads=layer["heads"], num_kv_heads=layer["kv_heads"], head_dim=layer["head_dim"],
                               scale=layer["head_dim"] ** -0.5, qk_norm="flat" if layer.get("qk_norm") else "none",
-                              qk_norm_eps=cfg["eps"], window=layer.get("window"), position=rotary)
+                              qk_norm_eps=cfg["eps"], window=layer.get("window"), position=rotary,
+                              kv_page_size=layer.get("page_size"))
     if layer["ffn"] == "dense":
         ffn = DenseMLPSpec(intermediate_size=layer["intermediate"], activation=layer.get("activation", "silu"))
     elif layer["ffn"] == "sign":
@@ -333,8 +334,9 @@ TOY_CONFIG = dict(
              ffn="dense", intermediate=96),
         dict(mixer="decay", state_size=12, decay=0.8, ffn="moe", experts=6, top_k=2, intermediate=40, scoring="softmax",
              bias=False, normalize=False, scaling=1.5),
-        dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, ffn="moe", experts=4, top_k=3,
-             intermediate=24, activation="gelu_tanh"),
+        # a window of 24 keys on pages of 8 tokens (the other groups take the engine's page size)
+        dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, page_size=8, ffn="moe", experts=4,
+             top_k=3, intermediate=24, activation="gelu_tanh"),
         dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, decay_gain=0.004, qk_norm=True, ffn="dense",
              intermediate=48, activation="gelu_tanh", norm="mean_abs"),
         # (layer 0 turns neighbouring dims together, the others dims half a rotary width apart)
