@@ -59,9 +59,10 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     }
   }
   // k rounds of arg-max (largest value, lowest index among equals); the last value is the threshold.
-  // A round is two plain reductions over the wave, the maximum of the values and then the lowest index
-  // among the elements that hold it (a reduction over (value, index) pairs costs twice the instructions,
-  // and with few tokens this kernel is a lone wavefront's chain of dependent instructions).
+  // A round is one reduction over the wave, the maximum of the values, and a few ballots for the lowest index
+  // among the elements that hold it (a reduction over (value, index) pairs costs twice the instructions, a
+  // second reduction for the index half as many again, and with few tokens this kernel is a lone
+  // wavefront's chain of dependent instructions).
   float threshold = 0.f;
   for (int round = 0; round < top_k; ++round) {
     float best = -INFINITY;
@@ -69,11 +70,14 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     for (int i = 0; i < PER_LANE; ++i)
       if (!((taken | excluded) & (1u << i)) && sel[i] > best) best = sel[i];
     const float top = wave_max(best);
-    int lowest = 0x7fffffff;
+    // the lowest index among the elements that hold it: the lowest element slot i that any lane holds it in
+    // (index = 64 i + lane), then the lowest such lane; the lanes' answers are masks in scalar registers
+    int winner = -1;
 #pragma unroll
-    for (int i = PER_LANE - 1; i >= 0; --i)
-      if (!((taken | excluded) & (1u << i)) && sel[i] == top) lowest = i * SE_WAVE + lane;
-    const int winner = wave_reduce(lowest, [](int a, int b) { return a < b ? a : b; });
+    for (int i = 0; i < PER_LANE; ++i) {
+      const uint64_t holders = __ballot(!((taken | excluded) & (1u << i)) && sel[i] == top);
+      if (winner < 0 && holders) winner = i * SE_WAVE + __builtin_ctzll(holders);
+    }
     if ((winner & (SE_WAVE - 1)) == lane) taken |= 1u << (winner / SE_WAVE);
     threshold = top;
   }
@@ -331,6 +335,24 @@ __global__ void router_topk_align_kernel(const float* __restrict__ logits, int64
   route_token<PER_LANE>(logits, stride, bias, ids, weights, threadIdx.x / SE_WAVE, experts, top_k,
                         softmax_scoring, normalize, scaling, chosen);
   __syncthreads();
+  if (tokens == 1 && top_k <= SE_WAVE) {
+    // One token: its experts are all different, every run is one row.  Tile t belongs to the t-th smallest of
+    // them (the order the general grouping gives); nothing has to be counted or scanned.
+    const int lane = threadIdx.x;
+    if (lane < top_k) {
+      const int mine = chosen[lane];
+      int tile = 0;
+      for (int j = 0; j < top_k; ++j) tile += chosen[j] < mine;
+      tile_expert[tile] = mine;
+      sorted[tile * tile_rows] = lane;
+      for (int r = 1; r < tile_rows; ++r) sorted[tile * tile_rows + r] = top_k;     // padding
+    }
+    if (lane == 0) {
+      counters[0] = top_k;
+      counters[1] = top_k * tile_rows;
+    }
+    return;
+  }
   align_assignments(chosen, tokens * top_k, experts, tile_rows, sorted, tile_expert, counters, sh);
 }
 
