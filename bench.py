@@ -6,18 +6,19 @@ Model: the sizes of MiniMax M2 (hidden 3072, 48 query / 8 kv heads of 128, rotar
 top-8 of width 1536, vocabulary 200064) cut to 16 of its 62 layers, random weights, bfloat16.
 A "step" is one decode step of a batch of 8 requests whose prompts were 2048 random token ids
 (sampling greedily, token ids read back each step).  One JSON line is printed: ``value`` is decoded
-tokens per second at batch 8; ``prefill`` is a 2048-token prompt in one step (``frac``: its flops
-against the matrix peak, ``hbm_frac``: the bytes it has to read against 8 TB/s, ``experts_touched``:
-the mean number of experts per layer that its tokens chose); ``points`` holds decode at batch 1 and
+tokens per second at batch 8; ``prefill`` is a 2048-token prompt in one step with its tokens spread evenly
+over all experts (``frac``: its flops against the matrix peak, ``hbm_frac``: the bytes it has to read against
+8 TB/s, ``experts_touched``: the experts per layer that its tokens take); ``points`` holds decode at batch 1 and
 64 and the prefill of eight 2048-token prompts in one step; ``roofline`` prices the batch-8 decode
 step against 8 TB/s and ``point_rooflines`` the other decode points the same way (every weight the
 step uses once - the experts it touched are counted from the step's own routing - and the cache of
-the live requests).  ``roofline.measured_peak`` is what a kernel of this engine that does nothing but read 8 GiB
+the live requests).  With random weights the router itself sends the tokens of a prompt to a few dozen experts
+past the first layer, which makes a prompt cheaper than real weights would: ``prefill_natural_routing`` is that
+step (``experts_touched``: the mean number of experts per layer that its tokens chose); in ``prefill`` every token
+is sent to eight experts drawn evenly from all 256 instead (the routing is replaced after the router has run, so
+the router's own work is still in the time).  ``roofline.measured_peak`` is what a kernel of this engine that does nothing but read 8 GiB
 reaches on this box at the start of the run (``memory`` holds that and the rate of a copy), and ``measured_frac`` /
-``point_rooflines_measured`` price the same steps against it.  With random weights the tokens of a prompt agree on a few dozen experts past
-the first layer, which makes a prompt cheaper than real weights would: ``prefill_uniform`` is the
-same step with every token sent to eight experts drawn evenly from all 256 (the routing is replaced
-after the router has run, so the router's own work is still in the time).  ``kernels`` holds, for the prefill
+``point_rooflines_measured`` price the same steps against it.  ``kernels`` holds, for the prefill
 and for every decode point, one further step with events around each call of the kernels object: the time of
 experts, attention, the dense products and the head, with the bytes (decode) or flops (prefill) each has to do
 per second.  ``--prompt-len C --no-prefill --fake-context`` gives decode steps at other context lengths.
@@ -214,9 +215,9 @@ def main() -> int:
         runner.release("p_calls")
         work = {"moe_experts": ("experts", 2 * T * K * 3 * I * h * L), "paged_attention": ("attention", 4 * H * D * T * (T + 1) / 2 * L),
                 f"linear_{(H + 2 * Hkv) * D}": ("qkv", 2 * T * h * (H + 2 * Hkv) * D * L), f"linear_{h}": ("o", 2 * T * H * D * h * L)}
-        kernels[f"prefill_{T}"] = {name: {"ms": round(calls[k], 3), "TFLOP/s": round(flops / calls[k] / 1e9, 1)}
-                                   for k, (name, flops) in work.items() if calls.get(k)}
-        kernels[f"prefill_{T}"]["rest"] = {"ms": round(sum(v for k, v in calls.items() if k not in work), 3)}
+        kernels[f"prefill_{T}_natural_routing"] = {name: {"ms": round(calls[k], 3), "TFLOP/s": round(flops / calls[k] / 1e9, 1)}
+                                                   for k, (name, flops) in work.items() if calls.get(k)}
+        kernels[f"prefill_{T}_natural_routing"]["rest"] = {"ms": round(sum(v for k, v in calls.items() if k not in work), 3)}
     if not args.no_prefill and args.prefill_routing != "natural":
         # the same step with even expert load: eight distinct experts per token, drawn uniformly
         dev_gen = torch.Generator(device="cuda").manual_seed(1)
@@ -232,6 +233,16 @@ def main() -> int:
             runner.release(f"u{i}")
         uniform_s = min(uniform_times[1:])
         uniform_bytes = L * dense_layer + L * min(E, T * K) * expert_bytes + V * h * itemsize
+        calls = time_calls(runner.kernels, lambda: runner.step([StepEntry("u_calls", prompt(), [PROMPT_LEN - 1])],
+                                                               forced_routing=even))
+        runner.release("u_calls")
+        work = {"moe_experts": ("experts", 2 * T * K * 3 * I * h * L), "paged_attention": ("attention", 4 * H * D * T * (T + 1) / 2 * L),
+                f"linear_{(H + 2 * Hkv) * D}": ("qkv", 2 * T * h * (H + 2 * Hkv) * D * L), f"linear_{h}": ("o", 2 * T * H * D * h * L)}
+        kernels[f"prefill_{T}"] = {name: {"ms": round(calls[k], 3), "TFLOP/s": round(flops / calls[k] / 1e9, 1)}
+                                   for k, (name, flops) in work.items() if calls.get(k)}
+        if calls.get("moe_experts"):      # every expert table is read once: the experts' share is a matter of memory
+            kernels[f"prefill_{T}"]["experts"]["GB/s"] = round(L * min(E, T * K) * expert_bytes / calls["moe_experts"] / 1e6, 1)
+        kernels[f"prefill_{T}"]["rest"] = {"ms": round(sum(v for k, v in calls.items() if k not in work), 3)}
         del even
     prefill_flops = L * (2 * T * h * (H + 2 * Hkv) * D + 2 * T * H * D * h + 2 * T * h * E + 2 * T * K * 3 * I * h
                          + 4 * H * D * T * (T + 1) / 2) + 2 * V * h
@@ -275,6 +286,18 @@ def main() -> int:
     if many_prompts:
         points[many_prompts[0]] = many_prompts[1]
     achieved = decode_bytes(args.batch, distinct, context) / step_s
+    natural_record = None if not natural else {
+        "value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3), "routing": "the model's own (random weights)",
+        "frac": round(prefill_flops / prefill_s / peak, 5),
+        # a 2048-token step reads every expert it touches for a few dozen rows each: memory bound too
+        "hbm_frac": round(prefill_bytes / prefill_s / HBM_PEAK, 4),
+        "hbm_measured_frac": round(prefill_bytes / prefill_s / measured_peak, 4),
+        "flops": prefill_flops, "bytes": prefill_bytes, "experts_touched": round(sum(touched) / len(touched), 1)}
+    uniform_record = None if uniform_s is None else {
+        "value": round(T / uniform_s, 1), "tokens": T, "ms": round(uniform_s * 1e3, 3), "routing": "even over all experts",
+        "frac": round(prefill_flops / uniform_s / peak, 5), "hbm_frac": round(uniform_bytes / uniform_s / HBM_PEAK, 4),
+        "hbm_measured_frac": round(uniform_bytes / uniform_s / measured_peak, 4),
+        "flops": prefill_flops, "bytes": uniform_bytes, "experts_touched": min(E, T * K)}
     line = {
         "metric": f"decode tok/s @ batch {args.batch} (MiniMax-M2 sizes, {L} layers, 1 GPU)", "value": round(args.batch / step_s, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -286,18 +309,11 @@ def main() -> int:
                    "num_local_experts": E, "num_experts_per_tok": K, "intermediate_size": I, "vocab_size": V,
                    "kv_page_size": 64, "kv_cache_tokens": args.kv_requests * CONTEXT_LEN,
                    "max_position_embeddings": cfg["max_position_embeddings"], "parallelism": "single GPU"},
-        "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
-                    "frac": round(prefill_flops / prefill_s / peak, 5),
-                    # a 2048-token step reads every expert it touches for a few dozen rows each: memory bound too
-                    "hbm_frac": None if prefill_bytes is None else round(prefill_bytes / prefill_s / HBM_PEAK, 4),
-                    "hbm_measured_frac": None if prefill_bytes is None else round(prefill_bytes / prefill_s / measured_peak, 4),
-                    "flops": prefill_flops, "bytes": prefill_bytes,
-                    "experts_touched": None if touched is None else round(sum(touched) / len(touched), 1)},
-        "prefill_uniform": None if uniform_s is None else {
-            "value": round(T / uniform_s, 1), "tokens": T, "ms": round(uniform_s * 1e3, 3),
-            "frac": round(prefill_flops / uniform_s / peak, 5), "hbm_frac": round(uniform_bytes / uniform_s / HBM_PEAK, 4),
-            "hbm_measured_frac": round(uniform_bytes / uniform_s / measured_peak, 4),
-            "bytes": uniform_bytes, "experts_touched": min(E, T * K)},
+        # The 2048-token prompt with its tokens spread evenly over all experts, as a trained router spreads them: every
+        # expert table is read.  With this model's random weights the router sends a prompt's tokens to a few dozen
+        # experts per layer, which is the cheaper step reported beside it.
+        "prefill": uniform_record if uniform_record is not None else natural_record,
+        "prefill_natural_routing": natural_record,
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4), "measured_peak": round(measured_peak / 1e9, 1),
                      "measured_frac": round(achieved / measured_peak, 4)},
