@@ -387,6 +387,11 @@ def run_workload(args) -> int:
         json.dump(dict(MODEL, num_hidden_layers=layers, max_position_embeddings=196608), fh)
     sync = torch.cuda.synchronize
     page = {"kv_page_size": args.kv_page_size} if args.kv_page_size else {}
+    from sparseengine_amd.kernels.hip_ops import HipKernels
+    memory = HipKernels().measure_memory(gib=8.0)       # before the model is there: what this box's memory delivers
+    torch.cuda.empty_cache()
+    print(f"[bench] memory: a kernel that only reads 8 GiB {memory['read_GBps']:.0f} GB/s, a copy "
+          f"{memory['copy_GBps']:.0f} GB/s (read + written)", file=sys.stderr, flush=True)
     t0 = time.time()
     if long_context:
         length, batch, output_len = 131072, 4, args.output_len or 1024
@@ -420,16 +425,43 @@ def run_workload(args) -> int:
             llm.add_request(prompt, sampling)
         # a step's time by what it holds: portions of prompts beside decoded tokens, or decoded tokens alone
         mixed_ms, decode_ms, output_tokens = [], [], 0
+        # What a step with a prompt portion has to read: the dense weights once, the tables of the experts its
+        # tokens chose (counted in every sixteenth such step, which is then left out of the times: the router's
+        # choices are copied out layer by layer) and the cache of every request that is running after it (the
+        # portion's own request and the decoding ones).
+        itemsize = 2 if args.dtype == "bfloat16" else 4
+        h, H, Hkv, D, E, I, V = (MODEL["hidden_size"], MODEL["num_attention_heads"], MODEL["num_key_value_heads"],
+                                 MODEL["head_dim"], MODEL["num_local_experts"], MODEL["intermediate_size"], MODEL["vocab_size"])
+        dense_once = layers * (((H + 2 * Hkv) * D * h + h * H * D) * itemsize + E * h * 4) + V * h * itemsize
+        expert_bytes = 3 * I * h * itemsize
+        kv_token = 2 * Hkv * D * itemsize * layers
+        run_step, taps_of_step = llm.runner.step, [None]
+        llm.runner.step = lambda entries, **kw: run_step(entries, taps=taps_of_step[0], **kw)
+        mixed_steps, chosen = [], []           # (seconds, tokens of context), experts chosen per layer in the counted steps
         sync()
         start = time.perf_counter()
+        steps_done = 0
         while not llm.is_finished():
+            counted = steps_done % 16 == 8
+            taps_of_step[0] = {} if counted else None
             t1 = time.perf_counter()
             finished, count = llm.step()
             sync()
-            (mixed_ms if count > 0 else decode_ms).append((time.perf_counter() - t1) * 1e3)
+            took = time.perf_counter() - t1
+            steps_done += 1
+            if counted and count > 0:
+                chosen.append(sum(int(torch.unique(ids).numel()) for ids, _ in taps_of_step[0]["router"]) / layers)
+            elif not counted:
+                (mixed_ms if count > 0 else decode_ms).append(took * 1e3)
+                if count > 0:
+                    mixed_steps.append((took, sum(s.num_computed_tokens for s in llm.scheduler.running)))
             output_tokens += sum(len(f[1]) for f in finished)
         seconds = time.perf_counter() - start
         prompt_tokens = sum(len(p) for p in prompts)
+        experts_read = sum(chosen) / len(chosen) if chosen else float(E)
+        weights_once = dense_once + layers * experts_read * expert_bytes
+        mixed_rates = sorted((weights_once + context * kv_token) / took / 1e9 for took, context in mixed_steps)
+        typical = mixed_rates[len(mixed_rates) // 2] if mixed_rates else 0.0
 
         def spread(ms):
             ms = sorted(ms)
@@ -443,6 +475,13 @@ def run_workload(args) -> int:
                 "config": {"num_layers": layers, "requests": requests, "portion": 512, "output_len": output_len},
                 "prompt_tokens": prompt_tokens, "output_tokens": output_tokens, "total_s": round(seconds, 3),
                 "step_ms_with_prompt_portions": spread(mixed_ms), "step_ms_decode_only": spread(decode_ms),
+                # the median step with a prompt portion: the bytes it has to read over its time
+                "mixed_step_roofline": {"bound": "hbm", "achieved": round(typical, 1), "peak": 8000.0, "unit": "GB/s",
+                                        "frac": round(typical / 8000.0, 4), "measured_peak": round(memory["read_GBps"], 1),
+                                        "measured_frac": round(typical / memory["read_GBps"], 4),
+                                        "weights_GB": round(weights_once / 1e9, 2),
+                                        "experts_read_per_layer": round(experts_read, 1), "steps_counted": len(chosen)},
+                "memory": {k: round(v, 1) for k, v in memory.items()},
                 "preemptions": llm.scheduler.total_preemptions}
     print(json.dumps(line), flush=True)
     return 0
