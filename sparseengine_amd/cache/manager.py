@@ -109,6 +109,7 @@ class CacheManager:
                 name: torch.zeros((self.max_rows, *shape), dtype=dt or dtype, device=device)
                 for name, shape, dt in req.tensors} if allocate_tensors else {}
 
+        self._no_window = all(group.window is None for group in self.groups)
         self.row_len = np.zeros(self.max_rows, dtype=np.int64)
         self.row_owner: list[object | None] = [None] * self.max_rows
         self._free_rows = deque(range(self.max_rows))
@@ -204,6 +205,8 @@ class CacheManager:
         rows = [row for row, _ in items]
         if len(set(rows)) != len(rows):
             raise ValueError("a row appears twice in one step")
+        if self._no_window and all(n == 1 for _, n in items):
+            return self._append_one_token_each(rows)
         for row, n in items:
             if self.row_owner[row] is None:
                 raise PageOwnershipError(f"row {row} is not held by a request")
@@ -240,6 +243,34 @@ class CacheManager:
                 cursor += n
         for row, n in items:
             self.row_len[row] += n
+        return StepAllocation(slots)
+
+    def _append_one_token_each(self, rows: list[int]) -> StepAllocation:
+        """``append`` for a step of single tokens where no group has a window (a decode step, whose time on the
+        host is time the device waits): nothing is given back, and a row takes a new page exactly when its length
+        is a multiple of the page size.  The same checks in the same order, the same pages in the same order."""
+        limit = self.max_model_len
+        for row in rows:
+            if self.row_owner[row] is None:
+                raise PageOwnershipError(f"row {row} is not held by a request")
+            if self.row_len[row] + 1 > limit:
+                raise ValueError(f"row {row}: {self.row_len[row]} + 1 tokens exceed max_model_len {limit}")
+        index = np.asarray(rows, dtype=np.int64)
+        lengths = self.row_len[index]
+        fresh = []                               # per group: which items start a new page
+        for group in self.groups:
+            starts_page = np.nonzero(lengths % group.page_size == 0)[0]
+            if starts_page.size > group.pool.free_count:
+                raise OutOfPages(f"step of {len(rows)} tokens does not fit: free pages {self.free_pages()}")
+            fresh.append(starts_page)
+        slots = {}
+        for group, starts_page in zip(self.groups, fresh):
+            ps = group.page_size
+            page_index = lengths // ps
+            for i in starts_page.tolist():
+                group.table[rows[i], page_index[i]] = group.pool.allocate(1, rows[i])[0]
+            slots[group.index] = (group.table[index, page_index] * ps + lengths % ps).astype(np.int32)
+        self.row_len[index] += 1
         return StepAllocation(slots)
 
     def truncate(self, row: int, length: int) -> None:

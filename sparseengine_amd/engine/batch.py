@@ -89,11 +89,7 @@ class ForwardBatch:
 
     def buffer(self, key: str, shape, dtype=None) -> torch.Tensor:
         """A reusable scratch tensor whose leading dims are cut to ``shape``."""
-        shape = tuple(int(s) for s in shape)
-        dtype = dtype or self.dtype
-        # one buffer per (purpose, row shape): only the leading dim is ever cut, so views stay dense
-        full = self.scratch.get(f"{key}{shape[1:]}", shape, dtype, self.device)
-        return full if full.shape[0] == shape[0] else full.narrow(0, 0, shape[0])
+        return self.scratch.view(key, shape if type(shape) is tuple else tuple(shape), dtype or self.dtype, self.device)
 
 
 class BlockTableError(RuntimeError):
@@ -157,27 +153,45 @@ class BatchBuilder:
             raise ValueError("a step needs at least one item")
         cache = self.cache
         lengths = [len(it.tokens) for it in items]
-        for it in items:
-            if not it.tokens:
-                raise ValueError("an item without tokens")
-            bad = [t for t in it.tokens if not 0 <= t < self.vocab_size]
-            if bad:
-                raise ValueError(f"token id {bad[0]} is outside the vocabulary [0, {self.vocab_size})")
-            if any(not 0 <= w < len(it.tokens) for w in it.want):
-                raise ValueError("a wanted place lies outside the item's tokens")
-        starts = [int(cache.row_len[it.row]) for it in items]
-        allocation = cache.append([(it.row, n) for it, n in zip(items, lengths)])   # all or nothing
-
         T, B = sum(lengths), len(items)
-        q_start = np.zeros(B, dtype=np.int32)
-        q_start[1:] = np.cumsum(lengths[:-1])
-        q_len = np.asarray(lengths, dtype=np.int32)
-        ctx_len = np.asarray([s + n for s, n in zip(starts, lengths)], dtype=np.int32)
-        token_ids = np.concatenate([np.asarray(it.tokens, dtype=np.int32) for it in items])
-        positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, lengths)])
-        token_item = np.repeat(np.arange(B, dtype=np.int32), lengths)
-        want = np.asarray([q_start[i] + w for i, it in enumerate(items) for w in it.want], dtype=np.int32)
-        rows = np.asarray([it.row for it in items], dtype=np.int32)
+        if T == B and min(lengths) == 1:
+            # a step of single tokens (decoding): the same checks and the same arrays without a loop over the items;
+            # what the host spends here is time the device waits between two steps
+            rows = np.asarray([it.row for it in items], dtype=np.int32)
+            token_ids = np.asarray([it.tokens[0] for it in items], dtype=np.int64)
+            if token_ids.min() < 0 or token_ids.max() >= self.vocab_size:
+                bad = token_ids[(token_ids < 0) | (token_ids >= self.vocab_size)]
+                raise ValueError(f"token id {int(bad[0])} is outside the vocabulary [0, {self.vocab_size})")
+            token_ids = token_ids.astype(np.int32)
+            for it in items:
+                if it.want and any(w != 0 for w in it.want):
+                    raise ValueError("a wanted place lies outside the item's tokens")
+            positions = cache.row_len[rows].astype(np.int32)
+            allocation = cache.append([(it.row, 1) for it in items])   # all or nothing
+            q_start = token_item = np.arange(B, dtype=np.int32)
+            q_len = np.ones(B, dtype=np.int32)
+            ctx_len = positions + 1
+            want = np.asarray([i for i, it in enumerate(items) for _ in it.want], dtype=np.int32)
+        else:
+            for it in items:
+                if not it.tokens:
+                    raise ValueError("an item without tokens")
+                bad = [t for t in it.tokens if not 0 <= t < self.vocab_size]
+                if bad:
+                    raise ValueError(f"token id {bad[0]} is outside the vocabulary [0, {self.vocab_size})")
+                if any(not 0 <= w < len(it.tokens) for w in it.want):
+                    raise ValueError("a wanted place lies outside the item's tokens")
+            starts = [int(cache.row_len[it.row]) for it in items]
+            allocation = cache.append([(it.row, n) for it, n in zip(items, lengths)])   # all or nothing
+            q_start = np.zeros(B, dtype=np.int32)
+            q_start[1:] = np.cumsum(lengths[:-1])
+            q_len = np.asarray(lengths, dtype=np.int32)
+            ctx_len = np.asarray([s + n for s, n in zip(starts, lengths)], dtype=np.int32)
+            token_ids = np.concatenate([np.asarray(it.tokens, dtype=np.int32) for it in items])
+            positions = np.concatenate([np.arange(s, s + n, dtype=np.int32) for s, n in zip(starts, lengths)])
+            token_item = np.repeat(np.arange(B, dtype=np.int32), lengths)
+            want = np.asarray([q_start[i] + w for i, it in enumerate(items) for w in it.want], dtype=np.int32)
+            rows = np.asarray([it.row for it in items], dtype=np.int32)
 
         tables = {}
         for group in cache.groups:

@@ -223,6 +223,36 @@ class HipKernels:
         sum of rows ``r * slots ...`` of ``x`` (``[rows * slots, hidden]``, contiguous), added up in
         float in slot order and rounded to the storage type first: the sum over a token's expert
         slots done while the norm reads, bit for bit what a separate sum would give."""
+        # The two calls every layer of every step makes (a few hundred launches a step: what the host spends per
+        # launch is what a short step waits for) go through their checks in one expression; a call that fails one,
+        # and every other kind of call, takes the long way below, which names what is wrong.
+        if rows is None:
+            shape = out.shape
+            hidden = shape[-1]
+            if (len(shape) == 2 and out.stride(1) == 1 and out.dtype == x.dtype and hidden <= 15360
+                    and weight.shape == shape[1:] and weight.is_contiguous()
+                    and (residual is None or (residual.shape == shape and residual.dtype == x.dtype
+                                              and residual.stride(1) == 1))):
+                aligned = not ((x.data_ptr() | out.data_ptr() | weight.data_ptr()
+                                | (0 if residual is None else residual.data_ptr())) & 15)
+                res_stride = 0 if residual is None else residual.stride(0)
+                if slots == 1:
+                    if x.shape == shape and x.stride(1) == 1:
+                        _check(_fn.get("norm", "se_rms_norm")(
+                            _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), None, shape[0], hidden, float(eps),
+                            x.stride(0), res_stride, out.stride(0), int(bool(write_residual)), _code(x.dtype),
+                            _code(weight.dtype), int(aligned), _stream()), "rms_norm")
+                        return
+                elif (x.dim() == 2 and x.shape[0] == shape[0] * slots and x.shape[1] == hidden and x.is_contiguous()
+                      and out.data_ptr() != x.data_ptr()):
+                    status = _fn.get("norm", "se_rms_norm_slots")(
+                        _ptr(x), _ptr(residual), _ptr(weight), _ptr(out), None, shape[0], hidden, float(eps),
+                        x.stride(0), res_stride, out.stride(0), int(bool(write_residual)), _code(x.dtype),
+                        _code(weight.dtype), int(aligned), int(slots), _stream())
+                    if status == 0:
+                        return
+                    if status != -1:
+                        _check(status, "rms_norm (slot rows)")
         hidden = x.shape[-1]
         n_out = out.shape[0]
         if slots > 1:
@@ -287,6 +317,28 @@ class HipKernels:
         last two sizes are a page's geometry; the order of its elements is cache/layout.py's)."""
         tokens = qkv.shape[0]
         width = (heads + 2 * kv_heads) * head_dim
+        int32 = torch.int32
+        # the call of every layer (norm weights, a rotation table, the cache write) in one expression; a call that
+        # fails a check, and every other kind of call, takes the long way below, which names what is wrong
+        if (q_weight is not None and cache is not None and rotary_dim and pairing in self.ROTARY_PAIRINGS
+                and qkv.dim() == 2 and qkv.shape[1] == width and qkv.stride(1) == 1
+                and positions.dtype == int32 and positions.is_contiguous() and positions.numel() == tokens
+                and rotary_dim % 2 == 0 and 0 < rotary_dim <= head_dim
+                and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
+                and q_weight.shape == (heads * head_dim,) and k_weight.shape == (kv_heads * head_dim,)
+                and q_weight.dtype == k_weight.dtype
+                and slots.dtype == int32 and slots.is_contiguous() and slots.numel() == tokens
+                and cache.dtype == qkv.dtype and cache.is_contiguous() and cache.dim() == 5
+                and tuple(cache.shape[1:]) == (2, kv_heads, page_size, head_dim)
+                and page_size % 8 == 0 and head_dim % 8 == 0):
+            aligned = not ((qkv.data_ptr() | q_weight.data_ptr() | k_weight.data_ptr() | cache.data_ptr()
+                            | cos_sin.data_ptr()) & 15)
+            _check(_fn.get("rope_kv", "se_qk_norm_rope_store")(
+                _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(cos_sin), _ptr(q_weight), _ptr(k_weight), float(eps),
+                tokens, heads, kv_heads, head_dim, rotary_dim, _ptr(cache), _ptr(slots), page_size, 1,
+                _code(qkv.dtype), _code(q_weight.dtype), int(aligned), self.ROTARY_PAIRINGS[pairing], _stream()),
+                "qk_norm_rope_store")
+            return
         _require(qkv.dim() == 2 and qkv.shape[1] == width and qkv.stride(1) == 1, "qkv shape")
         _i32(positions, "positions")
         _require(positions.numel() == tokens, "positions length")
@@ -539,6 +591,38 @@ class HipKernels:
         experts, two_i, _ = w13.shape
         inter = two_i // 2
         top_k = ids.shape[1]
+        # The call of a decode step (tables in tiles, the router's launch has grouped the assignments, fewer than
+        # three rows per expert: the streaming kernel on tiles of 16) in one expression; a call that fails a check,
+        # and every other kind of call, takes the long way below, which names what is wrong.
+        grouped = ws.grouped
+        if (tiled and kernel is None and tile_rows is None and column_blocks is None and grouped is not None
+                and x.dtype == torch.bfloat16 and hidden % 128 == 0 and inter % 128 == 0
+                and tokens * top_k < 3 * min(experts, tokens * top_k)
+                and grouped[:5] == (ids.data_ptr(), tokens, top_k, experts, 16) and grouped[5] <= 65535
+                and x.is_contiguous() and out.is_contiguous() and out.shape == x.shape
+                and w13.shape == (experts, 2 * inter, hidden) and w2.shape == (experts, hidden, inter)
+                and w13.is_contiguous() and w2.is_contiguous()
+                and w13.dtype == x.dtype and w2.dtype == x.dtype and out.dtype == x.dtype
+                and ids.dtype == torch.int32 and ids.is_contiguous() and ids.shape[0] == tokens and weights.shape == ids.shape
+                and weights.dtype == torch.float32 and weights.is_contiguous()
+                and ws.fits(tokens, top_k, experts, hidden, inter, x.dtype)):
+            ws.grouped = None
+            max_tiles, assignments = grouped[5], tokens * top_k
+            act = self._activation(activation)
+            blocks = 2 if max_tiles * (inter // 32) >= 2048 else 1
+            takes = "hidden and intermediate sizes in multiples of 128"
+            gg = _fn.get("moe_mfma", "se_grouped_gemm_mfma")
+            sorted_, tile_expert, counters = _ptr(ws.sorted), _ptr(ws.tile_expert), _ptr(ws.counters)
+            stream = _stream()
+            _check(gg(_ptr(x), _ptr(w13), _ptr(ws.act), sorted_, tile_expert, counters, None, assignments, top_k, inter,
+                      hidden, max_tiles, 0, 16, blocks, act, stream), "moe gate-up (stream)", takes)
+            _check(gg(_ptr(ws.act), _ptr(w2), _ptr(ws.slot_out), sorted_, tile_expert, counters, _ptr(weights), assignments,
+                      top_k, hidden, inter, max_tiles, 1, 16, blocks, act, stream), "moe down (stream)", takes)
+            if not sum_slots:
+                return ws.slot_out[:assignments]
+            _check(_fn.get("moe", "se_moe_sum")(_ptr(ws.slot_out), _ptr(out), tokens, top_k, hidden, _code(x.dtype),
+                                                stream), "moe_sum")
+            return
         _require(x.is_contiguous() and out.is_contiguous() and out.shape == x.shape, "moe x/out")
         _require(w13.shape == (experts, 2 * inter, hidden) and w2.shape == (experts, hidden, inter)
                  and w13.is_contiguous() and w2.is_contiguous(), "expert weight shapes")
@@ -669,10 +753,20 @@ class HipKernels:
         library."""
         rows, k = x.shape
         n = weight.shape[0]
+        bf16 = torch.bfloat16
+        if prepared is not None:      # the call of a decode step: one expression, or the long way below
+            if (rows <= self.TILED_SKINNY_ROWS and x.dtype == bf16 and prepared.dtype == bf16 and out.dtype == bf16
+                    and weight.dtype == bf16 and k % 128 == 0 and n % 16 == 0 and prepared.shape == weight.shape
+                    and weight.shape[1] == k and out.shape == (rows, n) and x.is_contiguous()
+                    and prepared.is_contiguous() and weight.is_contiguous() and out.is_contiguous()):
+                _check(_fn.get("moe_mfma", "se_skinny_gemm_mfma")(
+                    _ptr(x), _ptr(prepared), _ptr(out), rows, n, k, 1, _stream()),
+                    "skinny gemm", "K a multiple of 128, N a multiple of 16")
+                return out
         limit = self.TILED_SKINNY_ROWS if prepared is not None else self.SKINNY_ROWS
-        if (rows <= limit and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        if (rows <= limit and x.dtype == bf16 and weight.dtype == bf16
                 and k % 128 == 0 and n % 16 == 0 and x.is_contiguous() and weight.is_contiguous()
-                and out.is_contiguous() and out.dtype == torch.bfloat16):
+                and out.is_contiguous() and out.dtype == bf16):
             _require(weight.shape[1] == k and out.shape == (rows, n), "linear shapes")
             if prepared is not None:
                 _require(prepared.shape == weight.shape and prepared.dtype == weight.dtype and prepared.is_contiguous(),

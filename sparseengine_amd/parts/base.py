@@ -153,10 +153,25 @@ BLOCKS = PartRegistry("block", attribute="block")
 class StepScratch:
     """Buffers a part asks for once and reuses every step, sized for the largest step."""
     tensors: dict[str, torch.Tensor] = field(default_factory=dict)
+    views: dict[tuple, torch.Tensor] = field(default_factory=dict)     # (purpose, shape, dtype) -> the view handed out
 
     def get(self, key: str, shape: tuple[int, ...], dtype: torch.dtype, device) -> torch.Tensor:
         t = self.tensors.get(key)
         if t is None or t.dtype != dtype or t.shape[1:] != tuple(shape[1:]) or t.shape[0] < shape[0]:
             t = torch.empty(shape, dtype=dtype, device=device)
             self.tensors[key] = t
+            self.views.clear()       # views of the buffer this one replaces must not be handed out again
         return t
+
+    def view(self, key: str, shape: tuple[int, ...], dtype: torch.dtype, device) -> torch.Tensor:
+        """The buffer for ``key`` and these trailing sizes, its leading dim cut to ``shape[0]``.  A step
+        asks for the same few dozen views layer after layer and step after step; they are kept."""
+        at = (key, shape, dtype)
+        v = self.views.get(at)
+        if v is None:
+            shape = tuple(int(s) for s in shape)
+            full = self.get(f"{key}{shape[1:]}", shape, dtype, device)
+            # one buffer per (purpose, row shape): only the leading dim is ever cut, so views stay dense
+            v = full if full.shape[0] == shape[0] else full.narrow(0, 0, shape[0])
+            self.views[at] = v
+        return v

@@ -199,3 +199,56 @@ def test_truncate_undoes_an_append():
     m.truncate(row, 20)
     m.check_invariants()
     assert m.groups[0].pool.free_count == 3 and int(m.row_len[row]) == 20
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_a_step_of_single_tokens_takes_the_short_way_to_the_same_state(seed):
+    """Decode steps (one token per item, no windowed group) are appended by a vectorised routine; it leaves the
+    tables, the pools, the lengths and the slots that the general routine leaves, and refuses what that refuses."""
+    rng = random.Random(seed)
+    requests = {0: PagedKVRequest(2, 16), 1: PagedKVRequest(2, 16), 2: PagedKVRequest(1, 32, page_size=8)}
+    fast, slow = (manager(requests, pages={0: 24, 1: 40}, rows=6, page_size=16, max_len=150) for _ in range(2))
+    slow._no_window = False                     # the general routine
+    live = []
+    for step in range(400):
+        action = rng.random()
+        if (action < 0.15 or not live) and len(live) < 6:
+            name = f"r{step}"
+            rows = [m.admit(name) for m in (fast, slow)]
+            assert rows[0] == rows[1]
+            prompt = rng.randrange(1, 40)
+            outcome = []
+            for m in (fast, slow):
+                try:
+                    outcome.append(m.append([(rows[0], prompt)]).slots)
+                except OutOfPages:
+                    outcome.append(None)
+                    m.free(name)
+            assert (outcome[0] is None) == (outcome[1] is None)
+            if outcome[0] is not None:
+                live.append(name)
+        elif action < 0.25 and live:
+            name = live.pop(rng.randrange(len(live)))
+            fast.free(name); slow.free(name)
+        else:
+            chosen = rng.sample(live, rng.randrange(1, len(live) + 1))
+            results = []
+            for m in (fast, slow):
+                try:
+                    results.append(m.append([(m.row_of(name), 1) for name in chosen]).slots)
+                except (OutOfPages, ValueError) as exc:
+                    results.append(type(exc))
+            if isinstance(results[0], dict):
+                assert isinstance(results[1], dict)
+                for gi in results[0]:
+                    assert results[0][gi].dtype == results[1][gi].dtype == np.int32
+                    assert np.array_equal(results[0][gi], results[1][gi])
+            else:
+                assert results[0] is results[1]
+                if results[0] is ValueError:            # a request at its longest: it ends
+                    for name in [n for n in chosen if fast.row_len[fast.row_of(n)] + 1 > fast.max_model_len]:
+                        live.remove(name); fast.free(name); slow.free(name)
+        assert np.array_equal(fast.row_len, slow.row_len)
+        for a, b in zip(fast.groups, slow.groups):
+            assert np.array_equal(a.table, b.table) and a.pool._free == b.pool._free and a.pool._owner == b.pool._owner
+        fast.check_invariants()
