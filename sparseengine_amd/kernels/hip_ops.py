@@ -151,6 +151,11 @@ class _Functions:
 
 _fn = _Functions()
 
+# The calls a decode step makes hundreds of times take a short way through their checks (one expression each); a call
+# that fails one of them, and every other kind of call, takes the long way, which names what is wrong.  The tests
+# switch the short ways off to see that both pass the same arguments to the same entry points.
+_SHORT_WAYS = True
+
 
 def moe_tile_bounds(assignments: int, experts: int, tile_rows: int) -> tuple[int, int]:
     """(capacity of the sorted list, largest possible number of tiles) for an alignment."""
@@ -226,7 +231,7 @@ class HipKernels:
         # The two calls every layer of every step makes (a few hundred launches a step: what the host spends per
         # launch is what a short step waits for) go through their checks in one expression; a call that fails one,
         # and every other kind of call, takes the long way below, which names what is wrong.
-        if rows is None:
+        if _SHORT_WAYS and rows is None:
             shape = out.shape
             hidden = shape[-1]
             if (len(shape) == 2 and out.stride(1) == 1 and out.dtype == x.dtype and hidden <= 15360
@@ -320,7 +325,7 @@ class HipKernels:
         int32 = torch.int32
         # the call of every layer (norm weights, a rotation table, the cache write) in one expression; a call that
         # fails a check, and every other kind of call, takes the long way below, which names what is wrong
-        if (q_weight is not None and cache is not None and rotary_dim and pairing in self.ROTARY_PAIRINGS
+        if (_SHORT_WAYS and q_weight is not None and cache is not None and rotary_dim and pairing in self.ROTARY_PAIRINGS
                 and qkv.dim() == 2 and qkv.shape[1] == width and qkv.stride(1) == 1
                 and positions.dtype == int32 and positions.is_contiguous() and positions.numel() == tokens
                 and rotary_dim % 2 == 0 and 0 < rotary_dim <= head_dim
@@ -595,7 +600,7 @@ class HipKernels:
         # three rows per expert: the streaming kernel on tiles of 16) in one expression; a call that fails a check,
         # and every other kind of call, takes the long way below, which names what is wrong.
         grouped = ws.grouped
-        if (tiled and kernel is None and tile_rows is None and column_blocks is None and grouped is not None
+        if (_SHORT_WAYS and tiled and kernel is None and tile_rows is None and column_blocks is None and grouped is not None
                 and x.dtype == torch.bfloat16 and hidden % 128 == 0 and inter % 128 == 0
                 and tokens * top_k < 3 * min(experts, tokens * top_k)
                 and grouped[:5] == (ids.data_ptr(), tokens, top_k, experts, 16) and grouped[5] <= 65535
@@ -754,7 +759,7 @@ class HipKernels:
         rows, k = x.shape
         n = weight.shape[0]
         bf16 = torch.bfloat16
-        if prepared is not None:      # the call of a decode step: one expression, or the long way below
+        if _SHORT_WAYS and prepared is not None:      # the call of a decode step: one expression, or the long way below
             if (rows <= self.TILED_SKINNY_ROWS and x.dtype == bf16 and prepared.dtype == bf16 and out.dtype == bf16
                     and weight.dtype == bf16 and k % 128 == 0 and n % 16 == 0 and prepared.shape == weight.shape
                     and weight.shape[1] == k and out.shape == (rows, n) and x.is_contiguous()
