@@ -42,7 +42,7 @@ class AttentionSpec:
     num_kv_heads: int = 0
     head_dim: int = 0
     scale: float = 1.0
-    qk_norm: str = "none"          # "none" | "flat" (one RMS statistic per token over all heads)
+    qk_norm: str = "none"          # "none" | "flat" (one RMS statistic per token over all heads) | "per_head" (one per token and head)
     qk_norm_eps: float = 1e-6
     window: int | None = None       # keys further back than this are not read (None: all keys)
     position: Any = field(default_factory=NoPositionSpec)

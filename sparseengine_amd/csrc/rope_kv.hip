@@ -1,5 +1,7 @@
 // Fused per-token attention input preparation for gfx950:
-//   flat QK RMSNorm (one statistic per token over all heads, optional)
+//   QK RMSNorm, optional: flat (one statistic per token over all heads of q, one over all of k; weights
+//      [heads * head_dim]) or per head (one statistic per token and head; weights [head_dim], the general
+//      kernel only)
 //   -> partial rotation of dims [0, R) of every q and k head: pairs (d, d + R/2) ("NeoX", pairing 0)
 //      or pairs (2 j, 2 j + 1) ("interleaved", pairing 1; the general kernel only); pair j turns by
 //      the angle whose cosine and sine are the table's entries j and R/2 + j
@@ -7,7 +9,8 @@
 //
 // Statistics, rsqrt and the rotation are float.  The flat norm rounds (x * inv_rms) to the
 // storage type and multiplies by the weight in the storage type before the rotation, as a
-// two-step tensor expression would; in float storage both roundings are the identity.
+// two-step tensor expression would; the norm per head multiplies in float and rounds once, as a norm
+// kernel does.  In float storage the roundings are the identity.
 //
 // Cache layer layout: [num_pages, 2 (k, v), kv_heads, page_size * head_dim]; inside a page a kv
 // head's keys and values lie in groups of eight elements (key_place / value_place in common.h),
@@ -38,11 +41,11 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
                                           const W* __restrict__ k_weight, float eps, int heads,
                                           int kv_heads, int head_dim, int rotary_dim, T* cache,
                                           const int32_t* __restrict__ slots, int page_size,
-                                          int write_kv, int pairing) {
+                                          int write_kv, int pairing, int per_head) {
   // General sizes, one element at a time.  The token's whole q|k|v row is first brought into shared
   // memory (as float); everything after the barrier reads from there, so no global load waits
   // behind a store to the same row.
-  extern __shared__ float row[];
+  extern __shared__ float row[];      // the row; then (norm per head) heads + kv_heads reciprocal roots
   __shared__ float scratch[16];
   const int token = blockIdx.x;
   const int position = positions[token];
@@ -61,7 +64,16 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
     else if (c < q_width + k_width) k_sq += x * x;
   }
   float q_inv = 1.f, k_inv = 1.f;
-  if (use_norm) {
+  float* head_inv = row + width;      // [heads + kv_heads], q heads first
+  if (use_norm && per_head) {
+    __syncthreads();
+    for (int h = threadIdx.x; h < heads + kv_heads; h += blockDim.x) {   // a thread adds up a head's squares, in order
+      float sq = 0.f;
+      for (int d = 0; d < head_dim; ++d) sq += row[h * head_dim + d] * row[h * head_dim + d];
+      head_inv[h] = rsqrtf(sq / static_cast<float>(head_dim) + eps);
+    }
+    __syncthreads();
+  } else if (use_norm) {
     q_inv = rsqrtf(block_sum(q_sq, scratch) / static_cast<float>(q_width) + eps);
     k_inv = rsqrtf(block_sum(k_sq, scratch) / static_cast<float>(k_width) + eps);
   } else {
@@ -91,6 +103,8 @@ __global__ void qk_norm_rope_store_kernel(T* qkv, int64_t row_stride,
     auto normed = [&](int idx) {        // idx: element of q or of k
       const float x = row[(is_q ? 0 : q_width) + idx];
       if (!use_norm) return x;
+      if (per_head)                     // q heads, then k heads: head (is_q ? 0 : heads) + idx / head_dim of the row
+        return round_to<T>(x * head_inv[(is_q ? 0 : heads) + idx / head_dim] * to_float(weight[idx % head_dim]));
       const float scaled = round_to<T>(x * inv);
       return round_to<T>(scaled * round_to<T>(to_float(weight[idx])));
     };
@@ -303,10 +317,10 @@ template <typename T, typename W>
 static int launch(void* qkv, int64_t row_stride, const int32_t* positions, const float* cos_sin,
                   const void* qw, const void* kw, float eps, int tokens, int heads, int kv_heads,
                   int head_dim, int rotary_dim, void* cache, const int32_t* slots, int page_size,
-                  int write_kv, int vector_ok, int pairing, hipStream_t stream) {
+                  int write_kv, int vector_ok, int pairing, int per_head, hipStream_t stream) {
   // wide path: 16-byte aligned rows, vectors that never straddle a head or a rotary boundary
   constexpr int VN = Vec16<T>::N;
-  const bool vector_path = vector_ok && pairing == 0 && head_dim % VN == 0 && (rotary_dim / 2) % VN == 0 && row_stride % VN == 0 &&
+  const bool vector_path = vector_ok && pairing == 0 && !(per_head && qw) && head_dim % VN == 0 && (rotary_dim / 2) % VN == 0 && row_stride % VN == 0 &&
                            (rotary_dim / 2) % 4 == 0 && (Vec16<W>::N <= VN);
   const int width = (heads + 2 * kv_heads) * head_dim;
   if (vector_path) {
@@ -326,11 +340,11 @@ static int launch(void* qkv, int64_t row_stride, const int32_t* positions, const
     } else return SE_ERR_SHAPE;
 #undef SE_QK_VEC
   } else {
-    const size_t shmem = static_cast<size_t>(width) * sizeof(float);
+    const size_t shmem = static_cast<size_t>(width + heads + kv_heads) * sizeof(float);
     qk_norm_rope_store_kernel<T, W><<<tokens, 256, shmem, stream>>>(
         static_cast<T*>(qkv), row_stride, positions, cos_sin, static_cast<const W*>(qw),
         static_cast<const W*>(kw), eps, heads, kv_heads, head_dim, rotary_dim, static_cast<T*>(cache),
-        slots, page_size, write_kv, pairing);
+        slots, page_size, write_kv, pairing, per_head);
   }
   SE_CHECK_LAUNCH();
   return SE_OK;
@@ -341,8 +355,11 @@ extern "C" int se_qk_norm_rope_store(void* qkv, int64_t row_stride, const int32_
                                      const void* k_weight, float eps, int tokens, int heads,
                                      int kv_heads, int head_dim, int rotary_dim, void* cache,
                                      const int32_t* slots, int page_size, int write_kv, int dtype,
-                                     int weight_dtype, int vector_ok, int pairing, hipStream_t stream) {
+                                     int weight_dtype, int vector_ok, int pairing, int per_head,
+                                     hipStream_t stream) {
+  // per_head: the norm's statistic is one per token and head, its weights are [head_dim] (else flat, see above)
   if (tokens <= 0) return SE_OK;
+  if (per_head != 0 && per_head != 1) return SE_ERR_SHAPE;
   if (rotary_dim < 0 || rotary_dim % 2 || rotary_dim > head_dim) return SE_ERR_SHAPE;
   if (pairing != 0 && pairing != 1) return SE_ERR_SHAPE;
   if ((q_weight == nullptr) != (k_weight == nullptr)) return SE_ERR_SHAPE;
@@ -352,13 +369,13 @@ extern "C" int se_qk_norm_rope_store(void* qkv, int64_t row_stride, const int32_
     if (q_weight && weight_dtype != SE_F32) return SE_ERR_SHAPE;
     return launch<float, float>(qkv, row_stride, positions, cos_sin, q_weight, k_weight, eps, tokens,
                                 heads, kv_heads, head_dim, rotary_dim, cache, slots, page_size,
-                                write_kv, vector_ok, pairing, stream);
+                                write_kv, vector_ok, pairing, per_head, stream);
   }
   if (q_weight && weight_dtype == SE_F32)
     return launch<bf16_t, float>(qkv, row_stride, positions, cos_sin, q_weight, k_weight, eps,
                                  tokens, heads, kv_heads, head_dim, rotary_dim, cache, slots,
-                                 page_size, write_kv, vector_ok, pairing, stream);
+                                 page_size, write_kv, vector_ok, pairing, per_head, stream);
   return launch<bf16_t, bf16_t>(qkv, row_stride, positions, cos_sin, q_weight, k_weight, eps, tokens,
                                 heads, kv_heads, head_dim, rotary_dim, cache, slots, page_size,
-                                write_kv, vector_ok, pairing, stream);
+                                write_kv, vector_ok, pairing, per_head, stream);
 }

@@ -71,7 +71,7 @@ _SIGNATURES = {
     "rope_kv": {
         "se_qk_norm_rope_store": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                   c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int,
-                                  c_int, c_int, c_int, c_int, c_int, c_void_p],
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     },
     "attention_generic": {
         "se_paged_attention_generic": [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p,
@@ -314,9 +314,11 @@ class HipKernels:
     ROTARY_PAIRINGS = {"neox": 0, "interleaved": 1}
 
     def qk_norm_rope_store(self, qkv, positions, cos_sin, q_weight, k_weight, eps, heads, kv_heads,
-                           head_dim, rotary_dim, cache=None, slots=None, page_size=0, pairing="neox"):
-        """In place on ``qkv [T, (heads + 2 kv_heads) * head_dim]``: flat QK norm (if weights are
-        given), partial rotation by ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half; ``pairing``
+                           head_dim, rotary_dim, cache=None, slots=None, page_size=0, pairing="neox",
+                           per_head_norm: bool = False):
+        """In place on ``qkv [T, (heads + 2 kv_heads) * head_dim]``: QK norm (if weights are given: flat, one
+        statistic per token over all heads, weights ``[heads * head_dim]`` and ``[kv_heads * head_dim]``; or
+        ``per_head_norm``, one statistic per token and head, weights ``[head_dim]``), partial rotation by ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half; ``pairing``
         "neox" turns dims ``(d, d + rotary_dim / 2)`` together, "interleaved" dims ``(2 j, 2 j + 1)``), and
         the write of k and v to ``cache [pages, 2, kv_heads, page_size, head_dim]`` at ``slots`` (the
         last two sizes are a page's geometry; the order of its elements is cache/layout.py's)."""
@@ -325,13 +327,14 @@ class HipKernels:
         int32 = torch.int32
         # the call of every layer (norm weights, a rotation table, the cache write) in one expression; a call that
         # fails a check, and every other kind of call, takes the long way below, which names what is wrong
-        if (_SHORT_WAYS and q_weight is not None and cache is not None and rotary_dim and pairing in self.ROTARY_PAIRINGS
+        if (_SHORT_WAYS and not per_head_norm and q_weight is not None and cache is not None and rotary_dim
+                and pairing in self.ROTARY_PAIRINGS
                 and qkv.dim() == 2 and qkv.shape[1] == width and qkv.stride(1) == 1
                 and positions.dtype == int32 and positions.is_contiguous() and positions.numel() == tokens
                 and rotary_dim % 2 == 0 and 0 < rotary_dim <= head_dim
                 and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
                 and q_weight.shape == (heads * head_dim,) and k_weight.shape == (kv_heads * head_dim,)
-                and q_weight.dtype == k_weight.dtype
+                and q_weight.dtype == k_weight.dtype and q_weight.is_contiguous() and k_weight.is_contiguous()
                 and slots.dtype == int32 and slots.is_contiguous() and slots.numel() == tokens
                 and cache.dtype == qkv.dtype and cache.is_contiguous() and cache.dim() == 5
                 and tuple(cache.shape[1:]) == (2, kv_heads, page_size, head_dim)
@@ -341,7 +344,7 @@ class HipKernels:
             _check(_fn.get("rope_kv", "se_qk_norm_rope_store")(
                 _ptr(qkv), qkv.stride(0), _ptr(positions), _ptr(cos_sin), _ptr(q_weight), _ptr(k_weight), float(eps),
                 tokens, heads, kv_heads, head_dim, rotary_dim, _ptr(cache), _ptr(slots), page_size, 1,
-                _code(qkv.dtype), _code(q_weight.dtype), int(aligned), self.ROTARY_PAIRINGS[pairing], _stream()),
+                _code(qkv.dtype), _code(q_weight.dtype), int(aligned), self.ROTARY_PAIRINGS[pairing], 0, _stream()),
                 "qk_norm_rope_store")
             return
         _require(qkv.dim() == 2 and qkv.shape[1] == width and qkv.stride(1) == 1, "qkv shape")
@@ -352,8 +355,10 @@ class HipKernels:
             _require(cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
                      and cos_sin.shape[1] == rotary_dim, "cos_sin table shape/dtype")
         if q_weight is not None:
-            _require(q_weight.shape == (heads * head_dim,) and k_weight.shape == (kv_heads * head_dim,)
-                     and q_weight.dtype == k_weight.dtype, "qk norm weight shapes")
+            widths = ((head_dim,), (head_dim,)) if per_head_norm else ((heads * head_dim,), (kv_heads * head_dim,))
+            _require(k_weight is not None and (tuple(q_weight.shape), tuple(k_weight.shape)) == widths
+                     and q_weight.dtype == k_weight.dtype and q_weight.is_contiguous() and k_weight.is_contiguous(),
+                     "qk norm weight shapes")
         if pairing not in self.ROTARY_PAIRINGS:
             raise ValueError(f"rotary pairing {pairing!r} is unknown ({', '.join(self.ROTARY_PAIRINGS)})")
         write_kv = cache is not None
@@ -370,7 +375,8 @@ class HipKernels:
             _ptr(q_weight), _ptr(k_weight), float(eps), tokens, heads, kv_heads, head_dim, rotary_dim,
             _ptr(cache), _ptr(slots), page_size, int(write_kv), _code(qkv.dtype), wd,
             int(all(t is None or t.data_ptr() % 16 == 0 for t in (qkv, q_weight, k_weight, cache, cos_sin))),
-            self.ROTARY_PAIRINGS[pairing], _stream()), "qk_norm_rope_store")
+            self.ROTARY_PAIRINGS[pairing], int(bool(per_head_norm and q_weight is not None)), _stream()),
+            "qk_norm_rope_store")
 
     def paged_attention(self, q, cache, meta, out, scale: float, window: int = 0):
         """Causal attention of every token of the step against its request's pages.

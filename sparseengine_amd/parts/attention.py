@@ -1,7 +1,8 @@
 """Causal grouped-query attention over the paged cache.
 
 Order inside the mixer, as in the reference (models/minimax_m2.py:334-359): merged q/k/v
-projection -> flat QK RMSNorm over the whole q row and the whole k row (optional) -> rotation of
+projection -> QK RMSNorm (optional: flat, over the whole q row and the whole k row, which is MiniMax M2's; or
+per head with weights of one head's size, models/qwen3.py:116-118,151-153) -> rotation of
 the leading rotary dims of every head -> k (normed, rotated) and v written to this step's slots
 -> attention of the step's queries over everything the request has cached, its own tokens
 included -> output projection.  Norm, rotation and the cache write are one kernel when the position
@@ -24,8 +25,8 @@ class GQAAttention(Part):
             raise ValueError(f"{spec.num_heads} query heads do not divide into {spec.num_kv_heads} kv heads")
         if spec.head_dim % 16:
             raise ValueError(f"head_dim must be a multiple of 16, got {spec.head_dim}")
-        if spec.qk_norm not in ("none", "flat"):
-            raise ValueError(f"qk_norm {spec.qk_norm!r} is unknown (none, flat)")
+        if spec.qk_norm not in ("none", "flat", "per_head"):
+            raise ValueError(f"qk_norm {spec.qk_norm!r} is unknown (none, flat, per_head)")
         self.spec = spec
         self.hidden_size = int(hidden_size)
         self.q_width = spec.num_heads * spec.head_dim
@@ -39,6 +40,9 @@ class GQAAttention(Part):
         if self.spec.qk_norm == "flat":
             decls["q_norm"] = ParamDecl((self.q_width,))
             decls["k_norm"] = ParamDecl((self.kv_width,))
+        elif self.spec.qk_norm == "per_head":
+            decls["q_norm"] = ParamDecl((self.spec.head_dim,))
+            decls["k_norm"] = ParamDecl((self.spec.head_dim,))
         return decls
 
     def limit_positions(self, positions: int) -> None:
@@ -68,15 +72,17 @@ class GQAAttention(Part):
         q = qkv[:, :self.q_width].view(T, s.num_heads, s.head_dim)
         rotation = self.position.fused_rotation()
         store = (cache, meta.slots) if write_cache else (None, None)
+        per_head = s.qk_norm == "per_head"
         if rotation is not None:      # a rotation by a table: norm, rotation and cache write in one launch
             fb.kernels.qk_norm_rope_store(
                 qkv, meta.positions, rotation.table, p.get("q_norm"), p.get("k_norm"), s.qk_norm_eps,
                 s.num_heads, s.num_kv_heads, s.head_dim, rotation.rotary_dim, *store, meta.page_size,
-                pairing=rotation.pairing)
+                pairing=rotation.pairing, per_head_norm=per_head)
         else:                         # the position part applies itself, between the norm and the cache write
             if "q_norm" in p:
                 fb.kernels.qk_norm_rope_store(qkv, meta.positions, None, p["q_norm"], p["k_norm"], s.qk_norm_eps,
-                                              s.num_heads, s.num_kv_heads, s.head_dim, 0, None, None, meta.page_size)
+                                              s.num_heads, s.num_kv_heads, s.head_dim, 0, None, None, meta.page_size,
+                                              per_head_norm=per_head)
             k = qkv[:, self.q_width:self.q_width + self.kv_width].view(T, s.num_kv_heads, s.head_dim)
             self.position.apply(fb, q, k, meta.positions)
             if write_cache:

@@ -104,24 +104,30 @@ def rope_table(max_pos, rotary_dim, theta):
 @pytest.mark.parametrize("heads,kv_heads,head_dim,rotary,norm,page", [
     (4, 2, 16, 8, True, 16), (6, 3, 32, 32, False, 16), (48, 8, 128, 64, True, 64),
     (5, 5, 48, 16, True, 32), (6, 1, 128, 64, True, 16), (3, 1, 80, 0, False, 16)])
-def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary, norm, page, pairing="neox"):
+def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary, norm, page, pairing="neox",
+                            per_head=False):
     tokens, pages = 9, 7
     width = (heads + 2 * kv_heads) * head_dim
     qkv = randn(tokens, width, dtype=dtype, seed=3)
     positions = torch.tensor([0, 1, 17, 127, 1023, 5, 6, 7, 300], dtype=torch.int32).to(DEV)
     table = rope_table(2048, rotary, 5e6) if rotary else torch.zeros(1, 1, device=DEV)
-    qw = (1 + 0.1 * torch.randn(heads * head_dim)).to(dtype).to(DEV) if norm else None
-    kw = (1 + 0.1 * torch.randn(kv_heads * head_dim)).to(dtype).to(DEV) if norm else None
+    qw = (1 + 0.1 * torch.randn(head_dim if per_head else heads * head_dim)).to(dtype).to(DEV) if norm else None
+    kw = (1 + 0.1 * torch.randn(head_dim if per_head else kv_heads * head_dim)).to(dtype).to(DEV) if norm else None
     slots = torch.tensor([3 * page + 1, 0, page - 1, 5 * page, -1, 2 * page + 3, 2 * page + 4, 6 * page + page - 1, page],
                          dtype=torch.int32).to(DEV)
     cache_h = torch.zeros(pages, 2, kv_heads, page, head_dim, dtype=dtype, device=DEV)
     cache_t = cache_h.clone()
     a, b = qkv.clone(), qkv.clone()
     hip.qk_norm_rope_store(a, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_h, slots, page,
-                           pairing=pairing)
+                           pairing=pairing, per_head_norm=per_head)
     twin.qk_norm_rope_store(b, positions, table, qw, kw, 1e-6, heads, kv_heads, head_dim, rotary, cache_t, slots, page,
-                            pairing=pairing)
+                            pairing=pairing, per_head_norm=per_head)
     torch.testing.assert_close(a, b, **tol(dtype))
+    if per_head and norm and not rotary:
+        # every head by its own statistic: the library's norm over the last dim of [tokens, heads, head_dim]
+        q_in = qkv[:, :heads * head_dim].view(tokens, heads, head_dim).float()
+        ref = torch.nn.functional.rms_norm(q_in, (head_dim,), qw.float(), 1e-6)
+        torch.testing.assert_close(a[:, :heads * head_dim].view(tokens, heads, head_dim).float(), ref, **tol(dtype))
     if pairing == "interleaved" and not norm and rotary:
         # neighbours as complex numbers: the rotation is a multiplication by exp(i * angle) (a library routine)
         q_in = qkv[:, :heads * head_dim].view(tokens, heads, head_dim)[..., :rotary].float()
@@ -143,6 +149,30 @@ def test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary,
             at = (torch.tensor([s // page]).to(DEV), torch.tensor([s % page]).to(DEV))
             assert torch.equal(layout.read_keys(cache_h, *at)[0], kq[t])
             assert torch.equal(layout.read_values(cache_h, *at)[0], a[t, (heads + kv_heads) * head_dim:].view(kv_heads, head_dim))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("pairing", ["neox", "interleaved"])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rotary,page", [(4, 2, 16, 8, 16), (6, 3, 32, 32, 16), (5, 5, 48, 0, 32),
+                                                                 (48, 8, 128, 64, 64)])
+def test_qk_norm_of_every_head_by_itself(hip, twin, dtype, pairing, heads, kv_heads, head_dim, rotary, page):
+    """The other QK norm (one statistic per token and head, weights of one head's size), through the same checks
+    as the flat one: against the twin, against the library's norm where nothing rotates, into the cache."""
+    if pairing == "interleaved" and not rotary:
+        pytest.skip("nothing turns")
+    test_qk_norm_rope_store(hip, twin, dtype, heads, kv_heads, head_dim, rotary, True, page, pairing=pairing, per_head=True)
+    # and it is not the flat norm: a row whose heads differ in size by a factor of a hundred
+    qkv = randn(2, (heads + 2 * kv_heads) * head_dim, dtype=dtype, seed=8)
+    qkv[:, :head_dim] *= 100
+    positions, table = torch.zeros(2, dtype=torch.int32, device=DEV), torch.zeros(1, 1, device=DEV)
+    w = torch.ones(head_dim, dtype=dtype, device=DEV)
+    hip.qk_norm_rope_store(qkv, positions, table, w, w, 1e-6, heads, kv_heads, head_dim, 0, per_head_norm=True)
+    per_head_rms = qkv[:, :heads * head_dim].view(2, heads, head_dim).float().square().mean(-1).sqrt()
+    torch.testing.assert_close(per_head_rms, torch.ones_like(per_head_rms), rtol=2e-2, atol=2e-2)
+    with pytest.raises(ValueError, match="weight shapes"):
+        hip.qk_norm_rope_store(qkv, positions, table, torch.ones(heads * head_dim, dtype=dtype, device=DEV),
+                               torch.ones(kv_heads * head_dim, dtype=dtype, device=DEV), 1e-6, heads, kv_heads, head_dim, 0,
+                               per_head_norm=True)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

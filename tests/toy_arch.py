@@ -267,7 +267,8 @@ def _layer_spec(cfg, layer) -> LayerSpec:
         else:
             rotary = NoPositionSpec()
         mixer = AttentionSpec(num_heads=layer["heads"], num_kv_heads=layer["kv_heads"], head_dim=layer["head_dim"],
-                              scale=layer["head_dim"] ** -0.5, qk_norm="flat" if layer.get("qk_norm") else "none",
+                              scale=layer["head_dim"] ** -0.5,
+                              qk_norm={None: "none", False: "none", True: "flat"}.get(layer.get("qk_norm"), layer.get("qk_norm")),
                               qk_norm_eps=cfg["eps"], window=layer.get("window"), position=rotary,
                               kv_page_size=layer.get("page_size"))
     if layer["ffn"] == "dense":
@@ -335,16 +336,17 @@ TOY_CONFIG = dict(
         dict(mixer="decay", state_size=12, decay=0.8, ffn="moe", experts=6, top_k=2, intermediate=40, scoring="softmax",
              bias=False, normalize=False, scaling=1.5),
         # a window of 24 keys on pages of 8 tokens (the other groups take the engine's page size)
-        dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, page_size=8, ffn="moe", experts=4,
-             top_k=3, intermediate=24, activation="gelu_tanh"),
+        # (its QK norm has one statistic per head and weights of one head's size)
+        dict(mixer="attention", heads=6, kv_heads=2, head_dim=32, rotary_dim=32, window=24, page_size=8, qk_norm="per_head",
+             ffn="moe", experts=4, top_k=3, intermediate=24, activation="gelu_tanh"),
         dict(mixer="attention", heads=2, kv_heads=2, head_dim=32, rotary_dim=0, decay_gain=0.004, qk_norm=True, ffn="dense",
              intermediate=48, activation="gelu_tanh", norm="mean_abs"),
         # (layer 0 turns neighbouring dims together, the others dims half a rotary width apart)
         dict(mixer="attention", heads=4, kv_heads=2, head_dim=32, rotary_dim=8, linear_rotary=0.05, ffn="sign",
              intermediate=20),
         # mixer and feed-forward side by side behind one norm of the other kind
-        dict(mixer="attention", heads=2, kv_heads=1, head_dim=32, rotary_dim=0, decay_gain=0.003, ffn="dense", intermediate=32,
-             norm="mean_abs", block="toy_side_by_side"),
+        dict(mixer="attention", heads=2, kv_heads=1, head_dim=32, rotary_dim=0, decay_gain=0.003, qk_norm="per_head", ffn="dense",
+             intermediate=32, norm="mean_abs", block="toy_side_by_side"),
     ],
     # layer 0 runs twice (two caches); position 4 reads the cache of position 0 (same geometry)
     schedule=[dict(layer=0), dict(layer=1), dict(layer=2), dict(layer=0), dict(layer=3, cache_from=0), dict(layer=5),
@@ -352,6 +354,13 @@ TOY_CONFIG = dict(
 
 
 # ------------------------------------------------------------------ its plain implementation
+def per_head_qk_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, head_dim: int) -> torch.Tensor:
+    """RMS norm of every head by itself, one weight vector of a head's size for all heads
+    (the reference's dense attention, models/qwen3.py:116-118,151-153: ``RMSNorm(head_dim)`` on ``[T, heads, D]``)."""
+    heads = x.view(x.shape[0], -1, head_dim)
+    return (heads * torch.rsqrt(heads.square().mean(-1, keepdim=True) + eps) * weight).reshape(x.shape)
+
+
 class PlainToy:
     def __init__(self, folder: str):
         import json, os
@@ -389,7 +398,10 @@ class PlainToy:
                 H, Hkv, D, R = layer["heads"], layer["kv_heads"], layer["head_dim"], layer["rotary_dim"]
                 qkv = u @ w[p + "mixer.qkv"].T
                 q, k, v = qkv[:, :H * D], qkv[:, H * D:(H + Hkv) * D], qkv[:, (H + Hkv) * D:]
-                if layer.get("qk_norm"):
+                if layer.get("qk_norm") == "per_head":       # every head of a token by its own root mean square
+                    q = per_head_qk_norm(q, w[p + "mixer.q_norm"], cfg["eps"], D)
+                    k = per_head_qk_norm(k, w[p + "mixer.k_norm"], cfg["eps"], D)
+                elif layer.get("qk_norm"):
                     q = P.flat_qk_norm(q, w[p + "mixer.q_norm"], cfg["eps"])
                     k = P.flat_qk_norm(k, w[p + "mixer.k_norm"], cfg["eps"])
                 q, k, v = q.reshape(T, H, D), k.reshape(T, Hkv, D), v.reshape(T, Hkv, D)

@@ -54,7 +54,8 @@ class TwinKernels:
 
     # ------------------------------------------------------------------ attention inputs
     def qk_norm_rope_store(self, qkv, positions, cos_sin, q_weight, k_weight, eps, heads, kv_heads,
-                           head_dim, rotary_dim, cache=None, slots=None, page_size=0, pairing="neox"):
+                           head_dim, rotary_dim, cache=None, slots=None, page_size=0, pairing="neox",
+                           per_head_norm=False):
         T = qkv.shape[0]
         dt = qkv.dtype
         qw, kw = heads * head_dim, kv_heads * head_dim
@@ -65,7 +66,15 @@ class TwinKernels:
             def flat(x, w):
                 inv = torch.rsqrt(x.square().sum(-1, keepdim=True) / x.shape[-1] + eps)
                 return _r(_r(x * inv, dt) * _r(w.float(), dt), dt)
-            q, k = flat(q, q_weight), flat(k, k_weight)
+
+            def per_head(x, w, n):       # one statistic per token and head; the product in float, rounded once
+                x = x.view(T, n, head_dim)
+                inv = torch.rsqrt(x.square().sum(-1, keepdim=True) / head_dim + eps)
+                return _r(x * inv * w.float(), dt).reshape(T, n * head_dim)
+            if per_head_norm:
+                q, k = per_head(q, q_weight, heads), per_head(k, k_weight, kv_heads)
+            else:
+                q, k = flat(q, q_weight), flat(k, k_weight)
         if rotary_dim:
             half = rotary_dim // 2
             cs = cos_sin[positions.long()]
