@@ -318,8 +318,8 @@ class HipKernels:
                            per_head_norm: bool = False):
         """In place on ``qkv [T, (heads + 2 kv_heads) * head_dim]``: QK norm (if weights are given: flat, one
         statistic per token over all heads, weights ``[heads * head_dim]`` and ``[kv_heads * head_dim]``; or
-        ``per_head_norm``, one statistic per token and head, weights ``[head_dim]``), partial rotation by ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half; ``pairing``
-        "neox" turns dims ``(d, d + rotary_dim / 2)`` together, "interleaved" dims ``(2 j, 2 j + 1)``), and
+        ``per_head_norm``, one statistic per token and head, weights ``[head_dim]``), partial rotation by
+        ``cos_sin [max_pos, rotary_dim]`` (cos half, sin half; ``pairing`` "neox" turns dims ``(d, d + rotary_dim / 2)`` together, "interleaved" dims ``(2 j, 2 j + 1)``), and
         the write of k and v to ``cache [pages, 2, kv_heads, page_size, head_dim]`` at ``slots`` (the
         last two sizes are a page's geometry; the order of its elements is cache/layout.py's)."""
         tokens = qkv.shape[0]
