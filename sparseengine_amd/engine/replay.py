@@ -23,8 +23,6 @@ import json
 import os
 import sys
 
-import numpy as np
-
 from .runner import ModelRunner, StepEntry, kernels_for_program
 
 

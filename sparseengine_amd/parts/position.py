@@ -12,7 +12,7 @@ import weakref
 
 import torch
 
-from ..config.specs import NoPositionSpec, RotarySpec
+from ..config.specs import RotarySpec
 from .base import POSITIONS, FusedRotation, Part
 
 
